@@ -1,0 +1,99 @@
+"""ctypes binding of libhot_gfx950.so (declared in include/hot_gfx950.h).
+
+The library is the product: if it is missing this module raises, it never
+falls back to a CPU or eager-PyTorch implementation.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libhot_gfx950.so")
+
+HOT_MAX_HLA_N = 64
+
+# enums of include/hot_gfx950.h
+F32, BF16, F16 = 0, 1, 2
+ROUND_NEAREST, ROUND_STOCH = 0, 1
+SCALE_TENSOR, SCALE_ROW, SCALE_SAWB = 0, 1, 2
+STREAM_GX, STREAM_GW, STREAM_W, STREAM_ACT = 0, 1, 2, 3
+
+EXPORTS = (
+    "hot_last_error", "hot_abi_version", "hot_kpad", "hot_hq_rowwise", "hot_hla_tokenwise",
+    "hot_wq_colwise", "hot_colwise_workspace_bytes", "hot_gemm_i8", "hot_abc_workspace_bytes",
+    "hot_abc_forward", "hot_backward_workspace_bytes", "hot_linear_backward",
+)
+
+
+class HotConfig(C.Structure):
+    """struct hot_config."""
+    _fields_ = [
+        ("n_o", C.c_int32), ("hla_n", C.c_int32), ("hla_r", C.c_int32),
+        ("hla_rows", C.c_int32 * HOT_MAX_HLA_N),
+        ("gx_bits", C.c_int32), ("w_bits", C.c_int32), ("gw_bits", C.c_int32), ("act_bits", C.c_int32),
+        ("gx_round", C.c_int32), ("w_round", C.c_int32), ("gw_round", C.c_int32), ("act_round", C.c_int32),
+        ("gx_scale", C.c_int32), ("w_scale", C.c_int32), ("gw_scale", C.c_int32), ("act_scale", C.c_int32),
+        ("seed", C.c_uint64),
+    ]
+
+
+class HotError(RuntimeError):
+    pass
+
+
+_lib = None
+
+
+def _declare(lib):
+    vp, i32, i64, u32, u64, sz, fp = C.c_void_p, C.c_int, C.c_int64, C.c_uint32, C.c_uint64, C.c_size_t, C.c_float
+    cfgp = C.POINTER(HotConfig)
+    lib.hot_last_error.restype = C.c_char_p
+    lib.hot_last_error.argtypes = []
+    lib.hot_abi_version.restype = i32
+    lib.hot_abi_version.argtypes = []
+    lib.hot_kpad.restype = i64
+    lib.hot_kpad.argtypes = [i64]
+    lib.hot_hq_rowwise.restype = i32
+    lib.hot_hq_rowwise.argtypes = [vp, i32, i64, i64, i32, i32, i32, u64, u32, i32, vp, vp, vp, sz, vp]
+    lib.hot_hla_tokenwise.restype = i32
+    lib.hot_hla_tokenwise.argtypes = [vp, i32, i64, i64, i32, C.POINTER(C.c_int32), i32, i32, i32, u64, u32, i32,
+                                      vp, i64, vp, vp, sz, vp]
+    lib.hot_wq_colwise.restype = i32
+    lib.hot_wq_colwise.argtypes = [vp, i32, i64, i64, i32, i32, i32, u64, u32, i32, vp, i64, vp, vp, sz, vp]
+    lib.hot_colwise_workspace_bytes.restype = sz
+    lib.hot_colwise_workspace_bytes.argtypes = [i64]
+    lib.hot_gemm_i8.restype = i32
+    lib.hot_gemm_i8.argtypes = [vp, i64, vp, i64, i32, i64, i64, i64, vp, i32, vp, fp, vp, i32, i64, vp, vp]
+    lib.hot_abc_workspace_bytes.restype = sz
+    lib.hot_abc_workspace_bytes.argtypes = [i64, i64, cfgp]
+    lib.hot_abc_forward.restype = i32
+    lib.hot_abc_forward.argtypes = [vp, i32, i64, i64, cfgp, vp, vp, vp, sz, vp]
+    lib.hot_backward_workspace_bytes.restype = sz
+    lib.hot_backward_workspace_bytes.argtypes = [i64, i64, i64, cfgp]
+    lib.hot_linear_backward.restype = i32
+    lib.hot_linear_backward.argtypes = [vp, vp, i32, vp, vp, i64, i64, i64, cfgp, vp, vp, i32, vp, sz,
+                                        C.POINTER(C.c_float), vp]
+
+
+def lib():
+    """The loaded library; raises HotError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise HotError(
+                "libhot_gfx950.so is missing (%s). Build it with `python -m hot_amd.build`; "
+                "there is no fallback path." % LIB_PATH)
+        handle = C.CDLL(LIB_PATH)
+        for name in EXPORTS:
+            if not hasattr(handle, name):
+                raise HotError("libhot_gfx950.so does not export %s" % name)
+        _declare(handle)
+        _lib = handle
+    return _lib
+
+
+def check(rc: int) -> None:
+    if rc != 0:
+        msg = lib().hot_last_error()
+        raise HotError("libhot_gfx950 error %d: %s" % (rc, msg.decode("utf-8", "replace") if msg else "?"))

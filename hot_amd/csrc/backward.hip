@@ -1,0 +1,215 @@
+// C ABI of libhot_gfx950 and the fused HOT linear backward.
+//
+// hot_linear_backward sequences the kernels of the path on one HIP stream in
+// the stage order of the reference op backward_cuda
+// (cuda_measure/HLQ_backward_kernel.cu:457-737: transform -> quantise ->
+// low-rank -> GEMM x2 -> dequantise) with the numerics of FLinearQ.backward,
+// scheme gih_gwlr (utils/quant_matmul.py:215-348).  hot_abc_forward is the
+// forward-side activation buffer of FLinearQ.setup_context (:178-212).
+#include <string.h>
+
+#include "hot_device.h"
+#include "hot_host.h"
+
+namespace hot {
+
+static thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+int check_hip(hipError_t e, const char* what) {
+  if (e == hipSuccess) return HOT_OK;
+  return fail(HOT_ERR_HIP, "%s: %s", what, hipGetErrorString(e));
+}
+
+int check_launch(const char* what) { return check_hip(hipGetLastError(), what); }
+
+static int check_cfg(const hot_config* c, const char* who) {
+  if (!c) return fail(HOT_ERR_INVALID, "%s: null config", who);
+  if (c->n_o != 16 && c->n_o != 32 && c->n_o != 64) return fail(HOT_ERR_UNSUPPORTED, "%s: n_o=%d (16, 32 or 64)", who, c->n_o);
+  if (c->hla_n < 1 || c->hla_n > HOT_MAX_HLA_N || (c->hla_n & (c->hla_n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: hla_n=%d (power of two up to %d)", who, c->hla_n, HOT_MAX_HLA_N);
+  if (c->hla_r < 1 || c->hla_r > c->hla_n) return fail(HOT_ERR_INVALID, "%s: hla_r=%d outside [1, %d]", who, c->hla_r, c->hla_n);
+  const int bits[4] = {c->gx_bits, c->w_bits, c->gw_bits, c->act_bits};
+  for (int i = 0; i < 4; ++i)
+    if (bits[i] != 4 && bits[i] != 8) return fail(HOT_ERR_UNSUPPORTED, "%s: quantiser width %d (4 or 8)", who, bits[i]);
+  return HOT_OK;
+}
+
+struct BwdLayout {
+  int64_t ld_g, ld_w, ld_gp;                       // code pitches in bytes
+  size_t off_hq, off_colw, off_colg, off_sg, off_sw, off_sgp, off_qg, off_qw, off_qgp, total;
+};
+
+static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+static BwdLayout bwd_layout(int64_t L, int64_t O, int64_t I, const hot_config* c) {
+  BwdLayout b;
+  const int64_t lp = (L / c->hla_n) * c->hla_r;
+  b.ld_g = round_up(O, GEMM_KTILE) * c->gx_bits / 8;
+  b.ld_w = round_up(O, GEMM_KTILE) * c->w_bits / 8;
+  b.ld_gp = round_up(lp, GEMM_KTILE);
+  size_t o = 0;
+  b.off_hq = o;   o += 256;
+  b.off_colw = o; o += align256(colwise_workspace_bytes_impl(I));
+  b.off_colg = o; o += align256(colwise_workspace_bytes_impl(O));
+  b.off_sg = o;   o += align256((size_t)L * 4);
+  b.off_sw = o;   o += 256;
+  b.off_sgp = o;  o += align256((size_t)O * 4);
+  b.off_qg = o;   o += align256((size_t)L * b.ld_g);
+  b.off_qw = o;   o += align256((size_t)I * b.ld_w);
+  b.off_qgp = o;  o += align256((size_t)O * b.ld_gp);
+  b.total = o;
+  return b;
+}
+
+static const int32_t* identity_rows() {
+  static int32_t rows[HOT_MAX_HLA_N];
+  static bool init = false;
+  if (!init) { for (int i = 0; i < HOT_MAX_HLA_N; ++i) rows[i] = i; init = true; }
+  return rows;
+}
+
+}  // namespace hot
+
+using namespace hot;
+
+extern "C" {
+
+const char* hot_last_error(void) { return g_err; }
+int hot_abi_version(void) { return HOT_ABI_VERSION; }
+int64_t hot_kpad(int64_t k) { return round_up(k, GEMM_KTILE); }
+
+int hot_hq_rowwise(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, int rounding,
+                   uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, float* scales_out,
+                   void* workspace, size_t workspace_bytes, void* hip_stream) {
+  const int64_t ld = (bits == 4 || bits == 8) ? K * bits / 8 : 0;
+  return hq_rowwise_impl(in, dtype, M, K, n, bits, rounding, seed, rng_stream, scale_mode, codes_out, ld,
+                         scales_out, workspace, workspace_bytes, (hipStream_t)hip_stream);
+}
+
+size_t hot_colwise_workspace_bytes(int64_t C) { return colwise_workspace_bytes_impl(C > 0 ? C : 0); }
+
+int hot_hla_tokenwise(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r,
+                      int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
+                      void* codes_out, int64_t ld_out, float* scales_out, void* workspace,
+                      size_t workspace_bytes, void* hip_stream) {
+  return colwise_quant_impl(in, dtype, R, C, n, rows, r, bits, rounding, seed, rng_stream, scale_mode,
+                            codes_out, ld_out, /*store4=*/0, scales_out, workspace, workspace_bytes,
+                            (hipStream_t)hip_stream, "hot_hla_tokenwise");
+}
+
+int hot_wq_colwise(const void* in, int dtype, int64_t O, int64_t I, int n, int bits, int rounding,
+                   uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_out,
+                   float* scales_out, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  if (n != 16 && n != 32 && n != 64) return fail(HOT_ERR_UNSUPPORTED, "hot_wq_colwise: Hadamard block %d (16, 32 or 64)", n);
+  return colwise_quant_impl(in, dtype, O, I, n, identity_rows(), n, bits, rounding, seed, rng_stream, scale_mode,
+                            codes_out, ld_out, /*store4=*/bits == 4, scales_out, workspace, workspace_bytes,
+                            (hipStream_t)hip_stream, "hot_wq_colwise");
+}
+
+int hot_gemm_i8(const void* A, int64_t lda, const void* B, int64_t ldb, int bits, int64_t M, int64_t N,
+                int64_t K, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
+                void* out, int out_dtype, int64_t ldo, int32_t* acc_out, void* hip_stream) {
+  return gemm_i8_impl(A, lda, B, ldb, bits, M, N, K, scale_a, a_per_row, scale_b, post_scale, out, out_dtype,
+                      ldo, acc_out, (hipStream_t)hip_stream);
+}
+
+size_t hot_abc_workspace_bytes(int64_t L, int64_t I, const hot_config* cfg) {
+  (void)L; (void)cfg;
+  return colwise_workspace_bytes_impl(I > 0 ? I : 0);
+}
+
+int hot_abc_forward(const void* x, int dtype, int64_t L, int64_t I, const hot_config* cfg, void* xq_out,
+                    float* sx_out, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  if (int e = check_cfg(cfg, "hot_abc_forward")) return e;
+  if (L <= 0 || I <= 0 || L % cfg->hla_n) return fail(HOT_ERR_INVALID, "hot_abc_forward: L=%lld must be a positive multiple of hla_n=%d", (long long)L, cfg->hla_n);
+  if (cfg->act_scale == HOT_SCALE_ROW) return fail(HOT_ERR_UNSUPPORTED, "hot_abc_forward: the activation buffer uses one step per tensor");
+  const int64_t lp = (L / cfg->hla_n) * cfg->hla_r;
+  return colwise_quant_impl(x, dtype, L, I, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->act_bits, cfg->act_round,
+                            cfg->seed, HOT_STREAM_ACT, cfg->act_scale, xq_out, round_up(lp, GEMM_KTILE), 0,
+                            sx_out, workspace, workspace_bytes, (hipStream_t)hip_stream, "hot_abc_forward");
+}
+
+size_t hot_backward_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_config* cfg) {
+  if (check_cfg(cfg, "hot_backward_workspace_bytes") || L <= 0 || O <= 0 || I <= 0) return 0;
+  return bwd_layout(L, O, I, cfg).total;
+}
+
+int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,
+                        int64_t O, int64_t I, const hot_config* cfg, void* gx, void* gw, int out_dtype,
+                        void* workspace, size_t workspace_bytes, float* times4, void* hip_stream) {
+  const char* who = "hot_linear_backward";
+  if (int e = check_cfg(cfg, who)) return e;
+  if (!gy || !w || !xq || !sx || !gx || !gw) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
+  if (L <= 0 || O <= 0 || I <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape L=%lld O=%lld I=%lld", who, (long long)L, (long long)O, (long long)I);
+  if (O % cfg->n_o) return fail(HOT_ERR_INVALID, "%s: O=%lld is not a multiple of n_o=%d", who, (long long)O, cfg->n_o);
+  if (L % cfg->hla_n) return fail(HOT_ERR_INVALID, "%s: L=%lld is not a multiple of hla_n=%d", who, (long long)L, cfg->hla_n);
+  if (cfg->gx_bits != cfg->w_bits) return fail(HOT_ERR_UNSUPPORTED, "%s: gx_bits (%d) and w_bits (%d) must match", who, cfg->gx_bits, cfg->w_bits);
+  if (cfg->gx_scale == HOT_SCALE_SAWB) return fail(HOT_ERR_UNSUPPORTED, "%s: SAWB applies to W and x only", who);
+  if (cfg->w_scale == HOT_SCALE_ROW) return fail(HOT_ERR_UNSUPPORTED, "%s: W uses one step per tensor", who);
+  if (cfg->gw_scale == HOT_SCALE_SAWB) return fail(HOT_ERR_UNSUPPORTED, "%s: SAWB applies to W and x only", who);
+  const BwdLayout b = bwd_layout(L, O, I, cfg);
+  if (!workspace || workspace_bytes < b.total) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, b.total, workspace_bytes);
+  if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
+  hipStream_t st = (hipStream_t)hip_stream;
+  uint8_t* ws = (uint8_t*)workspace;
+  float* sg = (float*)(ws + b.off_sg);
+  float* sw = (float*)(ws + b.off_sw);
+  float* sgp = (float*)(ws + b.off_sgp);
+  const int64_t lp = (L / cfg->hla_n) * cfg->hla_r;
+
+  hipEvent_t ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
+  if (times4) {
+    for (int i = 0; i < 5; ++i)
+      if (int e = check_hip(hipEventCreate(&ev[i]), "hipEventCreate")) return e;
+    (void)hipEventRecord(ev[0], st);
+  }
+  int rc;
+  // g_y: Hadamard along O + quantise (g_x operand); HLA along tokens + quantise, transposed (g_W operand)
+  rc = hq_rowwise_impl(gy, dtype, L, O, cfg->n_o, cfg->gx_bits, cfg->gx_round, cfg->seed, HOT_STREAM_GX,
+                       cfg->gx_scale, ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, 256, st);
+  if (rc) goto done;
+  rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->gw_bits, cfg->gw_round,
+                          cfg->seed, HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp,
+                          ws + b.off_colg, colwise_workspace_bytes_impl(O), st, who);
+  if (rc) goto done;
+  if (times4) (void)hipEventRecord(ev[1], st);
+  // W: Hadamard along O + quantise, stored [I, O]
+  rc = colwise_quant_impl(w, dtype, O, I, cfg->n_o, identity_rows(), cfg->n_o, cfg->w_bits, cfg->w_round, cfg->seed,
+                          HOT_STREAM_W, cfg->w_scale, ws + b.off_qw, b.ld_w, cfg->w_bits == 4, sw,
+                          ws + b.off_colw, colwise_workspace_bytes_impl(I), st, who);
+  if (rc) goto done;
+  if (times4) (void)hipEventRecord(ev[2], st);
+  // g_x = (qG . qW^T) sG sW / n_o
+  rc = gemm_i8_impl(ws + b.off_qg, b.ld_g, ws + b.off_qw, b.ld_w, cfg->gx_bits, L, I, O, sg,
+                    cfg->gx_scale == HOT_SCALE_ROW, sw, 1.0f / (float)cfg->n_o, gx, out_dtype, I, nullptr, st);
+  if (rc) goto done;
+  if (times4) (void)hipEventRecord(ev[3], st);
+  // g_W = (qGp . xq^T) sGp sx / hla_n
+  rc = gemm_i8_impl(ws + b.off_qgp, b.ld_gp, xq, b.ld_gp, 8, O, I, lp, sgp, cfg->gw_scale == HOT_SCALE_ROW, sx,
+                    1.0f / (float)cfg->hla_n, gw, out_dtype, I, nullptr, st);
+  if (rc) goto done;
+  if (times4) {
+    (void)hipEventRecord(ev[4], st);
+    rc = check_hip(hipEventSynchronize(ev[4]), "hipEventSynchronize");
+    if (!rc) {
+      for (int i = 0; i < 4; ++i) {
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, ev[i], ev[i + 1]);
+        times4[i] = ms * 1e-3f;
+      }
+    }
+  }
+done:
+  for (int i = 0; i < 5; ++i)
+    if (ev[i]) (void)hipEventDestroy(ev[i]);
+  return rc;
+}
+
+}  // extern "C"

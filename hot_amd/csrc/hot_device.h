@@ -1,0 +1,168 @@
+// Device-side helpers shared by the gfx950 kernels: lane exchange, input
+// conversion, Philox-4x32-10, reductions.  wave64 only.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace hot {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+struct bf16_t { uint16_t v; };
+struct f16_t { _Float16 v; };
+
+template <typename T> struct dtype_of;
+template <> struct dtype_of<float> { static constexpr int value = 0; };
+template <> struct dtype_of<bf16_t> { static constexpr int value = 1; };
+template <> struct dtype_of<f16_t> { static constexpr int value = 2; };
+
+__device__ __forceinline__ float as_f(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+// Value held by lane (lane ^ MASK).  1 and 2 are DPP quad permutes (folded by
+// the compiler into the consuming VALU op), 4..16 go through the LDS crossbar
+// without touching memory, 32 uses the wave-wide permute.
+template <int MASK>
+__device__ __forceinline__ float lane_xor(float v) {
+  int i = __builtin_bit_cast(int, v);
+  if constexpr (MASK == 1) {
+    i = __builtin_amdgcn_update_dpp(0, i, 0xB1, 0xF, 0xF, true);  // quad_perm [1,0,3,2]
+  } else if constexpr (MASK == 2) {
+    i = __builtin_amdgcn_update_dpp(0, i, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
+  } else if constexpr (MASK == 3) {
+    i = __builtin_amdgcn_update_dpp(0, i, 0x1B, 0xF, 0xF, true);  // quad_perm [3,2,1,0]
+  } else if constexpr (MASK < 32) {
+    i = __builtin_amdgcn_ds_swizzle(i, (MASK << 10) | 0x1F);      // bitmask mode: xor MASK
+  } else {
+    i = __shfl_xor(i, MASK, 64);
+  }
+  return __builtin_bit_cast(float, i);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+  v = fmaxf(v, lane_xor<1>(v));
+  v = fmaxf(v, lane_xor<2>(v));
+  v = fmaxf(v, lane_xor<4>(v));
+  v = fmaxf(v, lane_xor<8>(v));
+  v = fmaxf(v, lane_xor<16>(v));
+  v = fmaxf(v, lane_xor<32>(v));
+  return v;
+}
+
+__device__ __forceinline__ double wave_sum(double v) {
+#pragma unroll
+  for (int m = 32; m >= 1; m >>= 1) v += __shfl_xor(v, m, 64);
+  return v;
+}
+
+// ---- 16-byte input vectors -> fp32 ---------------------------------------
+
+template <typename T> struct vec_traits;
+template <> struct vec_traits<float> { static constexpr int EPV = 4; };
+template <> struct vec_traits<bf16_t> { static constexpr int EPV = 8; };
+template <> struct vec_traits<f16_t> { static constexpr int EPV = 8; };
+
+template <typename T>
+__device__ __forceinline__ void unpack_vec(const uint4& raw, float* out);
+
+template <>
+__device__ __forceinline__ void unpack_vec<float>(const uint4& raw, float* out) {
+  out[0] = as_f(raw.x); out[1] = as_f(raw.y); out[2] = as_f(raw.z); out[3] = as_f(raw.w);
+}
+template <>
+__device__ __forceinline__ void unpack_vec<bf16_t>(const uint4& raw, float* out) {
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    out[2 * i] = as_f(w[i] << 16);
+    out[2 * i + 1] = as_f(w[i] & 0xFFFF0000u);
+  }
+}
+template <>
+__device__ __forceinline__ void unpack_vec<f16_t>(const uint4& raw, float* out) {
+  typedef _Float16 h2 __attribute__((ext_vector_type(2)));
+  const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    h2 p = __builtin_bit_cast(h2, w[i]);
+    out[2 * i] = (float)p.x;
+    out[2 * i + 1] = (float)p.y;
+  }
+}
+
+// Scalar element load -> fp32 (used by the column-wise kernels).
+template <typename T> __device__ __forceinline__ float load_scalar(const T* p);
+template <> __device__ __forceinline__ float load_scalar<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float load_scalar<bf16_t>(const bf16_t* p) { return as_f((uint32_t)p->v << 16); }
+template <> __device__ __forceinline__ float load_scalar<f16_t>(const f16_t* p) { return (float)p->v; }
+
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
+  uint32_t u = as_u(f);
+  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40);  // NaN
+  u += 0x7FFFu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <typename T> __device__ __forceinline__ void store_scalar(T* p, float v);
+template <> __device__ __forceinline__ void store_scalar<float>(float* p, float v) { *p = v; }
+template <> __device__ __forceinline__ void store_scalar<bf16_t>(bf16_t* p, float v) { p->v = f32_to_bf16_rne(v); }
+template <> __device__ __forceinline__ void store_scalar<f16_t>(f16_t* p, float v) { p->v = (_Float16)v; }
+
+// ---- Philox-4x32-10 -------------------------------------------------------
+
+struct philox4 { uint32_t w[4]; };
+
+__device__ __forceinline__ philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+                                                 uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
+    c0 = n0; c1 = lo1; c2 = n2; c3 = lo0;
+    k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
+  }
+  philox4 o; o.w[0] = c0; o.w[1] = c1; o.w[2] = c2; o.w[3] = c3;
+  return o;
+}
+
+// Uniforms for the four elements whose linear indices are 4*quad .. 4*quad+3.
+__device__ __forceinline__ void sr_uniform4(uint64_t quad, uint64_t seed, uint32_t stream, float* u) {
+  const philox4 p = philox4x32_10((uint32_t)quad, (uint32_t)(quad >> 32), stream, 0u,
+                                  (uint32_t)seed, (uint32_t)(seed >> 32));
+#pragma unroll
+  for (int i = 0; i < 4; ++i) u[i] = (float)(p.w[i] >> 8) * 5.9604644775390625e-08f;  // 2^-24
+}
+
+// Uniform of the single element with linear index e.
+__device__ __forceinline__ float sr_uniform1(uint64_t e, uint64_t seed, uint32_t stream) {
+  float u[4];
+  sr_uniform4(e >> 2, seed, stream, u);
+  const uint32_t l = (uint32_t)e & 3u;
+  return l == 0 ? u[0] : l == 1 ? u[1] : l == 2 ? u[2] : u[3];
+}
+
+// ---- quantisation of one value --------------------------------------------
+
+// y = x / d already divided.  Nearest: ties to even.
+__device__ __forceinline__ int q_nearest(float y) { return (int)rintf(y); }
+
+__device__ __forceinline__ int q_stoch(float y, float u) {
+  const float ay = fabsf(y);
+  const float fl = floorf(ay);
+  const float frac = ay - fl;
+  const int m = (int)fl + (u < frac ? 1 : 0);
+  return y < 0.f ? -m : m;
+}
+
+__device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
+
+// non-negative float max through an integer atomic (bit patterns of
+// non-negative floats are ordered like unsigned integers)
+__device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) {
+  atomicMax(reinterpret_cast<unsigned int*>(addr), as_u(v));
+}
+
+}  // namespace hot

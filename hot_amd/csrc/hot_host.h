@@ -1,0 +1,39 @@
+// Host-side plumbing shared by the translation units of libhot_gfx950:
+// error reporting and the internal (C++) entry points behind the C ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/hot_gfx950.h"
+
+namespace hot {
+
+// Records the message for hot_last_error() and returns `code`.
+int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+
+// hipGetLastError() after a launch -> HOT_OK or HOT_ERR_HIP.
+int check_launch(const char* what);
+int check_hip(hipError_t e, const char* what);
+
+inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
+
+constexpr int64_t GEMM_KTILE = 128;  // codes per K-tile of the int8 GEMM
+
+int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, int rounding,
+                    uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_codes,
+                    float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st);
+
+int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r,
+                       int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
+                       void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,
+                       size_t workspace_bytes, hipStream_t st, const char* who);
+size_t colwise_workspace_bytes_impl(int64_t C);
+
+int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bits, int64_t M, int64_t N,
+                 int64_t K, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
+                 void* out, int out_dtype, int64_t ldo, int32_t* acc_out, hipStream_t st);
+
+}  // namespace hot

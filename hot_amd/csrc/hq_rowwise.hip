@@ -1,0 +1,327 @@
+// hq_rowwise: block-Hadamard along the contiguous dimension fused with the
+// absmax step and INT4/INT8 quantisation.
+//
+// Replaces fwht_kernel / find_scale_kernel / quant_int4(_per_token)_kernel /
+// quant_int8_kernel of the reference CUDA op
+// (cuda_measure/HLQ_backward_kernel.cu:39-178,282-307) with the numerics of
+// lowering_matmul_front + int/stoch/norm_quantizer_BWD
+// (utils/hadamard_matmul.py:121-141, utils/quant_matmul.py:19-31,86-116).
+//
+// Data movement: every lane owns EPL = 8 consecutive elements (one 16-byte
+// load for 16-bit inputs, two for fp32), so a wave reads contiguous memory.
+// Butterfly stages h < 8 run in registers, stages h >= 8 exchange with lane
+// (lane ^ h/8) through DPP quad permutes or the LDS crossbar.  The stage order
+// h = 1, 2, 4, ... and the (x+y, x-y) convention are those of the reference
+// fwht_kernel (:63-78), which fixes the fp32 summation order.
+//
+// HBM traffic per element: sizeof(in) read once + bits/8 written; per-row
+// scales add 4 bytes per row.  Per-tensor scales need the global absmax first,
+// which costs a second read of the input.
+#include "hot_device.h"
+#include "hot_host.h"
+
+namespace hot {
+
+constexpr int EPL = 8;  // elements per lane-chunk
+
+template <typename T>
+__device__ __forceinline__ void load_chunk(const T* p, float* x) {
+  constexpr int EPV = vec_traits<T>::EPV;
+  const uint4* v = reinterpret_cast<const uint4*>(p);
+#pragma unroll
+  for (int i = 0; i < EPL / EPV; ++i) {
+    const uint4 raw = v[i];
+    unpack_vec<T>(raw, x + i * EPV);
+  }
+}
+
+// FWHT of the N-element blocks formed by N/EPL adjacent lanes.
+template <int N>
+__device__ __forceinline__ void fwht_lanes(float* x, int lane) {
+#pragma unroll
+  for (int h = 1; h < EPL; h <<= 1) {
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+      if ((j & h) == 0) {
+        const float a = x[j], b = x[j + h];
+        x[j] = a + b;
+        x[j + h] = a - b;
+      }
+    }
+  }
+  // lower lane: own + partner ; upper lane: partner - own  ==  partner + (-own)
+  if constexpr (N >= 16) {
+    const uint32_t sg = (lane & 1) ? 0x80000000u : 0u;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) x[j] = as_f(as_u(x[j]) ^ sg) + lane_xor<1>(x[j]);
+  }
+  if constexpr (N >= 32) {
+    const uint32_t sg = (lane & 2) ? 0x80000000u : 0u;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) x[j] = as_f(as_u(x[j]) ^ sg) + lane_xor<2>(x[j]);
+  }
+  if constexpr (N >= 64) {
+    const uint32_t sg = (lane & 4) ? 0x80000000u : 0u;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) x[j] = as_f(as_u(x[j]) ^ sg) + lane_xor<4>(x[j]);
+  }
+}
+
+template <int BITS, int ROUND>
+__device__ __forceinline__ void quant_store_chunk(const float* x, float d, uint64_t e0, uint64_t seed,
+                                                  uint32_t stream, int8_t* out_row_chunk) {
+  constexpr int QMAX = (1 << (BITS - 1)) - 1;
+  int q[EPL];
+  if constexpr (ROUND == 0) {
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) q[j] = clampi(q_nearest(x[j] / d), -QMAX, QMAX);
+  } else {
+    float u[EPL];
+    sr_uniform4(e0 >> 2, seed, stream, u);
+    sr_uniform4((e0 >> 2) + 1, seed, stream, u + 4);
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) q[j] = clampi(q_stoch(x[j] / d, u[j]), -QMAX, QMAX);
+  }
+  if constexpr (BITS == 4) {
+    uint32_t w = 0;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) w |= (uint32_t)(q[j] & 0xF) << (4 * j);
+    *reinterpret_cast<uint32_t*>(out_row_chunk) = w;
+  } else {
+    uint32_t w0 = 0, w1 = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      w0 |= (uint32_t)(q[j] & 0xFF) << (8 * j);
+      w1 |= (uint32_t)(q[j + 4] & 0xFF) << (8 * j);
+    }
+    *reinterpret_cast<uint2*>(out_row_chunk) = make_uint2(w0, w1);
+  }
+}
+
+// ---- per-row scales: one workgroup per row, row resident in registers ------
+
+template <typename T, int N, int BITS, int ROUND, int C>
+__global__ void hq_row_kernel(const T* __restrict__ in, int64_t K, int8_t* __restrict__ codes, int64_t ld,
+                              float* __restrict__ scales, uint64_t seed, uint32_t stream) {
+  __shared__ float s_red[16];
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int team = blockDim.x;
+  const int64_t row = blockIdx.x;
+  const int nch = (int)(K / EPL);
+  const T* rp = in + row * K;
+
+  float x[C][EPL];
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const int ch = tid + c * team;
+    if (ch < nch) {
+      load_chunk<T>(rp + (int64_t)ch * EPL, x[c]);
+    } else {
+#pragma unroll
+      for (int j = 0; j < EPL; ++j) x[c][j] = 0.f;
+    }
+  }
+  float mx = 0.f;
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    fwht_lanes<N>(x[c], lane);
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) mx = fmaxf(mx, fabsf(x[c][j]));
+  }
+  mx = wave_max(mx);
+  if (team > 64) {
+    if (lane == 0) s_red[tid >> 6] = mx;
+    __syncthreads();
+    const int nw = team >> 6;
+    float m = s_red[0];
+    for (int i = 1; i < nw; ++i) m = fmaxf(m, s_red[i]);
+    mx = m;
+  }
+  constexpr float QMAXF = (float)((1 << (BITS - 1)) - 1);
+  const float s = mx / QMAXF;
+  const float d = s + 1e-11f;
+  if (tid == 0) scales[row] = s;
+
+  int8_t* orow = codes + row * ld;
+#pragma unroll
+  for (int c = 0; c < C; ++c) {
+    const int ch = tid + c * team;
+    if (ch < nch) {
+      quant_store_chunk<BITS, ROUND>(x[c], d, (uint64_t)row * (uint64_t)K + (uint64_t)ch * EPL, seed,
+                                     stream, orow + (int64_t)ch * (EPL * BITS / 8));
+    }
+  }
+}
+
+// ---- per-tensor scale, pass 1: absmax of the transformed tensor -----------
+
+template <typename T, int N>
+__global__ void hq_absmax_kernel(const T* __restrict__ in, int64_t nchunks, float* __restrict__ absmax) {
+  __shared__ float s_red[16];
+  const int lane = threadIdx.x & 63;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  float mx = 0.f;
+  for (int64_t ch = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ch < nchunks; ch += stride) {
+    float x[EPL];
+    load_chunk<T>(in + ch * EPL, x);
+    fwht_lanes<N>(x, lane);
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) mx = fmaxf(mx, fabsf(x[j]));
+  }
+  mx = wave_max(mx);
+  if (lane == 0) s_red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float m = s_red[0];
+    for (int i = 1; i < (int)(blockDim.x >> 6); ++i) m = fmaxf(m, s_red[i]);
+    atomic_max_nonneg(absmax, m);
+  }
+}
+
+// ---- per-tensor scale, pass 2: transform again and quantise ----------------
+
+template <typename T, int N, int BITS, int ROUND>
+__global__ void hq_tensor_kernel(const T* __restrict__ in, int64_t nchunks, int64_t nch_row, int64_t ld,
+                                 const float* __restrict__ absmax, int8_t* __restrict__ codes,
+                                 float* __restrict__ scale_out, uint64_t seed, uint32_t stream) {
+  const int lane = threadIdx.x & 63;
+  constexpr float QMAXF = (float)((1 << (BITS - 1)) - 1);
+  const float s = *absmax / QMAXF;
+  const float d = s + 1e-11f;
+  if (blockIdx.x == 0 && threadIdx.x == 0) *scale_out = s;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t ch = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ch < nchunks; ch += stride) {
+    float x[EPL];
+    load_chunk<T>(in + ch * EPL, x);
+    fwht_lanes<N>(x, lane);
+    int64_t off = ch * (EPL * BITS / 8);
+    if (ld != nch_row * (EPL * BITS / 8)) {  // padded rows
+      const int64_t row = ch / nch_row;
+      off = row * ld + (ch - row * nch_row) * (EPL * BITS / 8);
+    }
+    quant_store_chunk<BITS, ROUND>(x, d, (uint64_t)ch * EPL, seed, stream, codes + off);
+  }
+}
+
+// zero the bytes [row_bytes, ld) of every row (K padding for the GEMM)
+__global__ void zero_pad_kernel(int8_t* codes, int64_t M, int64_t row_bytes, int64_t ld) {
+  const int64_t padw = (ld - row_bytes) / 4;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= M * padw) return;
+  const int64_t row = i / padw, j = i - row * padw;
+  *reinterpret_cast<uint32_t*>(codes + row * ld + row_bytes + j * 4) = 0u;
+}
+
+__global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
+}
+
+// ---- host dispatch -----------------------------------------------------------
+
+template <typename T, int N, int BITS, int ROUND>
+static int launch_row(const void* in, int64_t M, int64_t K, void* codes, int64_t ld, float* scales, uint64_t seed,
+                      uint32_t stream_id, hipStream_t st) {
+  const int64_t nch = K / EPL;
+  int team = 64;
+  while (team < 1024 && nch > 4 * (int64_t)team) team <<= 1;
+  const int64_t c = (nch + team - 1) / team;
+  if (c > 8) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: K=%lld too large for per-row scales (max 65536)", (long long)K);
+  const dim3 grid((unsigned)M), block(team);
+#define HOT_ROW_CASE(CC)                                                                              \
+  hipLaunchKernelGGL((hq_row_kernel<T, N, BITS, ROUND, CC>), grid, block, 0, st, (const T*)in, K, \
+                     (int8_t*)codes, ld, scales, seed, stream_id)
+  switch (c) {
+    case 1: HOT_ROW_CASE(1); break;
+    case 2: HOT_ROW_CASE(2); break;
+    case 3: HOT_ROW_CASE(3); break;
+    case 4: HOT_ROW_CASE(4); break;
+    case 5: case 6: HOT_ROW_CASE(6); break;
+    default: HOT_ROW_CASE(8); break;
+  }
+#undef HOT_ROW_CASE
+  return check_launch("hq_row_kernel");
+}
+
+template <typename T, int N, int BITS, int ROUND>
+static int launch_tensor(const void* in, int64_t M, int64_t K, void* codes, int64_t ld, float* scales, float* absmax,
+                         uint64_t seed, uint32_t stream_id, hipStream_t st) {
+  const int64_t nch = M * K / EPL;
+  const int block = 256;
+  int64_t blocks = (nch + block - 1) / block;
+  const int64_t cap = 256 * 16;  // 16 workgroups per CU, grid-stride beyond
+  if (blocks > cap) blocks = cap;
+  if (blocks < 1) blocks = 1;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, (uint32_t*)absmax, 0u, 1);
+  hipLaunchKernelGGL((hq_absmax_kernel<T, N>), dim3((unsigned)blocks), dim3(block), 0, st, (const T*)in, nch, absmax);
+  hipLaunchKernelGGL((hq_tensor_kernel<T, N, BITS, ROUND>), dim3((unsigned)blocks), dim3(block), 0, st,
+                     (const T*)in, nch, K / EPL, ld, absmax, (int8_t*)codes, scales, seed, stream_id);
+  return check_launch("hq_tensor_kernel");
+}
+
+template <typename T, int N, int BITS, int ROUND>
+static int dispatch_mode(int scale_mode, const void* in, int64_t M, int64_t K, void* codes, int64_t ld, float* scales,
+                         float* absmax, uint64_t seed, uint32_t stream_id, hipStream_t st) {
+  const int64_t row_bytes = K * BITS / 8;
+  if (ld > row_bytes) {
+    const int64_t n = M * ((ld - row_bytes) / 4);
+    hipLaunchKernelGGL(zero_pad_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (int8_t*)codes, M, row_bytes, ld);
+  }
+  if (scale_mode == HOT_SCALE_ROW) return launch_row<T, N, BITS, ROUND>(in, M, K, codes, ld, scales, seed, stream_id, st);
+  return launch_tensor<T, N, BITS, ROUND>(in, M, K, codes, ld, scales, absmax, seed, stream_id, st);
+}
+
+template <typename T, int N>
+static int dispatch_bits(int bits, int rounding, int scale_mode, const void* in, int64_t M, int64_t K,
+                         void* codes, int64_t ld, float* scales, float* absmax, uint64_t seed, uint32_t stream_id,
+                         hipStream_t st) {
+  if (bits == 4) {
+    return rounding == HOT_ROUND_NEAREST
+               ? dispatch_mode<T, N, 4, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st)
+               : dispatch_mode<T, N, 4, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st);
+  }
+  return rounding == HOT_ROUND_NEAREST
+             ? dispatch_mode<T, N, 8, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st)
+             : dispatch_mode<T, N, 8, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st);
+}
+
+template <typename T>
+static int dispatch_n(int n, int bits, int rounding, int scale_mode, const void* in, int64_t M, int64_t K,
+                      void* codes, int64_t ld, float* scales, float* absmax, uint64_t seed, uint32_t stream_id,
+                      hipStream_t st) {
+  switch (n) {
+    case 16: return dispatch_bits<T, 16>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st);
+    case 32: return dispatch_bits<T, 32>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st);
+    default: return dispatch_bits<T, 64>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st);
+  }
+}
+
+int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, int rounding,
+                    uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_codes,
+                    float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st) {
+  if (M != 0 && (!in || !codes_out || !scales_out)) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: null pointer");
+  if (M < 0 || K <= 0) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: bad shape M=%lld K=%lld", (long long)M, (long long)K);
+  if (n != 16 && n != 32 && n != 64) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: Hadamard block %d (16, 32 or 64)", n);
+  if (K % n) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: K=%lld is not a multiple of the block %d", (long long)K, n);
+  if (bits != 4 && bits != 8) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: bits=%d (4 or 8)", bits);
+  if (rounding != HOT_ROUND_NEAREST && rounding != HOT_ROUND_STOCH) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: bad rounding %d", rounding);
+  if (scale_mode != HOT_SCALE_TENSOR && scale_mode != HOT_SCALE_ROW) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: scale mode %d (tensor or row)", scale_mode);
+  if (((uintptr_t)in & 15) || ((uintptr_t)codes_out & 7)) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: input must be 16-byte and output 8-byte aligned");
+  if (M >= (1ll << 31)) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: M too large");
+  if (ld_codes < K * bits / 8 || (ld_codes & 7)) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: code pitch %lld must be a multiple of 8 and >= %lld", (long long)ld_codes, (long long)(K * bits / 8));
+  float* absmax = nullptr;
+  if (scale_mode == HOT_SCALE_TENSOR) {
+    if (!workspace || workspace_bytes < 256) return fail(HOT_ERR_WORKSPACE, "hot_hq_rowwise: per-tensor scale needs a 256-byte workspace");
+    absmax = (float*)workspace;
+  }
+  if (M == 0) return HOT_OK;
+  switch (dtype) {
+    case HOT_F32: return dispatch_n<float>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st);
+    case HOT_BF16: return dispatch_n<bf16_t>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st);
+    case HOT_F16: return dispatch_n<f16_t>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st);
+    default: return fail(HOT_ERR_INVALID, "hot_hq_rowwise: bad dtype %d", dtype);
+  }
+}
+
+}  // namespace hot

@@ -1,0 +1,213 @@
+"""Torch-facing wrappers of the C ABI: tensors in, tensors out.
+
+PyTorch is used for device memory (its caching allocator provides outputs and
+workspaces, so nothing is hipMalloc'ed per call) and for the current stream;
+all arithmetic happens in libhot_gfx950.so.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass, field
+from typing import Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import (BF16, F16, F32, ROUND_NEAREST, ROUND_STOCH, SCALE_ROW, SCALE_SAWB, SCALE_TENSOR,
+                   STREAM_ACT, STREAM_GW, STREAM_GX, STREAM_W, HotError)
+
+_DTYPES = {torch.float32: F32, torch.bfloat16: BF16, torch.float16: F16}
+_ROUND = {"nearest": ROUND_NEAREST, "int": ROUND_NEAREST, "stoch": ROUND_STOCH, "stochastic": ROUND_STOCH,
+          ROUND_NEAREST: ROUND_NEAREST, ROUND_STOCH: ROUND_STOCH}
+_SCALE = {"tensor": SCALE_TENSOR, "row": SCALE_ROW, "token": SCALE_ROW, "sawb": SCALE_SAWB,
+          SCALE_TENSOR: SCALE_TENSOR, SCALE_ROW: SCALE_ROW, SCALE_SAWB: SCALE_SAWB}
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DTYPES[t.dtype]
+    except KeyError:
+        raise RuntimeError("unsupported dtype %s (float32, bfloat16 or float16)" % t.dtype)
+
+
+def _need_gpu_2d(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError("%s must be a CUDA tensor!" % name)
+    if not t.is_contiguous():
+        raise RuntimeError("%s must be contiguous!" % name)
+    if t.dim() != 2:
+        raise RuntimeError("%s must be 2D!" % name)
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ws(nbytes: int, device) -> torch.Tensor:
+    # torch allocations are at least 512-byte aligned
+    return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+
+
+def kpad(k: int) -> int:
+    return int(_lib.lib().hot_kpad(int(k)))
+
+
+@dataclass
+class HotOptions:
+    """Options of the fused path (struct hot_config); the fields FLinearQ reads
+    from the reference's module-global ``args`` for scheme gih_gwlr."""
+    n_o: int = 16
+    hla_n: int = 1
+    hla_rows: Sequence[int] = (0,)
+    gx_bits: int = 4
+    w_bits: int = 4
+    gw_bits: int = 8
+    act_bits: int = 8
+    gx_round: int = ROUND_NEAREST
+    w_round: int = ROUND_NEAREST
+    gw_round: int = ROUND_NEAREST
+    act_round: int = ROUND_NEAREST
+    gx_scale: int = SCALE_TENSOR
+    w_scale: int = SCALE_TENSOR
+    gw_scale: int = SCALE_TENSOR
+    act_scale: int = SCALE_TENSOR
+    seed: int = 0
+
+    @property
+    def hla_r(self) -> int:
+        return len(self.hla_rows)
+
+    def lprime(self, L: int) -> int:
+        return (L // self.hla_n) * self.hla_r
+
+    def to_c(self) -> _lib.HotConfig:
+        if self.hla_n > _lib.HOT_MAX_HLA_N:
+            raise HotError("HLA block %d exceeds the native maximum %d" % (self.hla_n, _lib.HOT_MAX_HLA_N))
+        c = _lib.HotConfig()
+        c.n_o, c.hla_n, c.hla_r = self.n_o, self.hla_n, self.hla_r
+        for i, v in enumerate(self.hla_rows):
+            c.hla_rows[i] = int(v)
+        c.gx_bits, c.w_bits, c.gw_bits, c.act_bits = self.gx_bits, self.w_bits, self.gw_bits, self.act_bits
+        c.gx_round, c.w_round, c.gw_round, c.act_round = (_ROUND[self.gx_round], _ROUND[self.w_round],
+                                                          _ROUND[self.gw_round], _ROUND[self.act_round])
+        c.gx_scale, c.w_scale, c.gw_scale, c.act_scale = (_SCALE[self.gx_scale], _SCALE[self.w_scale],
+                                                          _SCALE[self.gw_scale], _SCALE[self.act_scale])
+        c.seed = int(self.seed) & 0xFFFFFFFFFFFFFFFF
+        return c
+
+
+def hq_rowwise(x: torch.Tensor, n: int = 16, bits: int = 4, rounding="nearest", scale="tensor",
+               seed: int = 0, rng_stream: int = STREAM_GX) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Block-Hadamard along the last dim + absmax step + quantise.
+    Returns (codes int8 [M, K*bits/8], steps fp32 [1] or [M])."""
+    _need_gpu_2d(x, "input")
+    M, K = x.shape
+    mode = _SCALE[scale]
+    codes = torch.empty((M, K * bits // 8), dtype=torch.int8, device=x.device)
+    scales = torch.empty((M if mode == SCALE_ROW else 1,), dtype=torch.float32, device=x.device)
+    ws = _ws(256, x.device)
+    _lib.check(_lib.lib().hot_hq_rowwise(x.data_ptr(), _dt(x), M, K, n, bits, _ROUND[rounding], seed, rng_stream,
+                                         mode, codes.data_ptr(), scales.data_ptr(), ws.data_ptr(), ws.numel(),
+                                         _stream()))
+    return codes, scales
+
+
+def hla_tokenwise(x: torch.Tensor, n: int, rows: Sequence[int], bits: int = 8, rounding="nearest",
+                  scale="tensor", seed: int = 0, rng_stream: int = STREAM_GW):
+    """HLA along dim 0 + quantise, stored transposed.
+    Returns (codes int8 [C, kpad(L')], steps fp32 [1] or [C], L')."""
+    _need_gpu_2d(x, "input")
+    R, Cc = x.shape
+    r = len(rows)
+    kout = (R // max(n, 1)) * r
+    ld = kpad(kout)
+    mode = _SCALE[scale]
+    codes = torch.empty((Cc, ld), dtype=torch.int8, device=x.device)
+    scales = torch.empty((Cc if mode == SCALE_ROW else 1,), dtype=torch.float32, device=x.device)
+    ws = _ws(_lib.lib().hot_colwise_workspace_bytes(Cc), x.device)
+    rows_c = (C.c_int32 * r)(*[int(v) for v in rows])
+    _lib.check(_lib.lib().hot_hla_tokenwise(x.data_ptr(), _dt(x), R, Cc, n, rows_c, r, bits, _ROUND[rounding], seed,
+                                            rng_stream, mode, codes.data_ptr(), ld, scales.data_ptr(),
+                                            ws.data_ptr(), ws.numel(), _stream()))
+    return codes, scales, kout
+
+
+def wq_colwise(w: torch.Tensor, n: int = 16, bits: int = 4, rounding="nearest", scale="tensor",
+               seed: int = 0, rng_stream: int = STREAM_W):
+    """Block-Hadamard of W [O, I] along O + quantise, stored as [I, kpad(O)*bits/8]."""
+    _need_gpu_2d(w, "W")
+    O, I = w.shape
+    ld = kpad(O) * bits // 8
+    codes = torch.empty((I, ld), dtype=torch.int8, device=w.device)
+    scales = torch.empty((1,), dtype=torch.float32, device=w.device)
+    ws = _ws(_lib.lib().hot_colwise_workspace_bytes(I), w.device)
+    _lib.check(_lib.lib().hot_wq_colwise(w.data_ptr(), _dt(w), O, I, n, bits, _ROUND[rounding], seed, rng_stream,
+                                         _SCALE[scale], codes.data_ptr(), ld, scales.data_ptr(), ws.data_ptr(),
+                                         ws.numel(), _stream()))
+    return codes, scales
+
+
+def gemm_i8(a: torch.Tensor, b: torch.Tensor, k: int, bits: int, scale_a: torch.Tensor, scale_b: torch.Tensor,
+            post_scale: float = 1.0, out_dtype=torch.float32, return_acc: bool = False):
+    """out[M,N] = ((A . B^T) * scale_a) * scale_b * post_scale on K-major codes.
+    a [M, lda bytes], b [N, ldb bytes] int8 tensors whose rows hold k codes of
+    `bits` bits, zero-padded to kpad(k)."""
+    _need_gpu_2d(a, "A")
+    _need_gpu_2d(b, "B")
+    M, N = a.shape[0], b.shape[0]
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    acc = torch.empty((M, N), dtype=torch.int32, device=a.device) if return_acc else None
+    per_row = 1 if scale_a.numel() > 1 else 0
+    if per_row and scale_a.numel() != M:
+        raise RuntimeError("scale_a must have 1 or M entries")
+    _lib.check(_lib.lib().hot_gemm_i8(a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), bits, M, N, k,
+                                      scale_a.data_ptr(), per_row, scale_b.data_ptr(), float(post_scale),
+                                      out.data_ptr(), _DTYPES[out_dtype], N,
+                                      acc.data_ptr() if acc is not None else None, _stream()))
+    return (out, acc) if return_acc else out
+
+
+def abc_forward(x: torch.Tensor, opt: HotOptions):
+    """INT8 Hadamard-compressed activation buffer: (xq int8 [I, kpad(L')], sx fp32 [1])."""
+    _need_gpu_2d(x, "X")
+    L, I = x.shape
+    cfg = opt.to_c()
+    xq = torch.empty((I, kpad(opt.lprime(L))), dtype=torch.int8, device=x.device)
+    sx = torch.empty((1,), dtype=torch.float32, device=x.device)
+    ws = _ws(_lib.lib().hot_abc_workspace_bytes(L, I, C.byref(cfg)), x.device)
+    _lib.check(_lib.lib().hot_abc_forward(x.data_ptr(), _dt(x), L, I, C.byref(cfg), xq.data_ptr(), sx.data_ptr(),
+                                          ws.data_ptr(), ws.numel(), _stream()))
+    return xq, sx
+
+
+def linear_backward(gy: torch.Tensor, w: torch.Tensor, xq: torch.Tensor, sx: torch.Tensor, opt: HotOptions,
+                    out_dtype=None, timing: bool = False, workspace: Optional[torch.Tensor] = None):
+    """g_x [L, I], g_W [O, I] (and the four stage times in seconds when timing)."""
+    _need_gpu_2d(gy, "Go")
+    _need_gpu_2d(w, "Wt")
+    L, O = gy.shape
+    if w.shape[0] != O:
+        raise RuntimeError("W must be [O, I] with O = Go.shape[1]")
+    if w.dtype != gy.dtype:
+        raise RuntimeError("Go and W must have the same dtype")
+    I = w.shape[1]
+    out_dtype = out_dtype or gy.dtype
+    cfg = opt.to_c()
+    lp = opt.lprime(L)
+    if tuple(xq.shape) != (I, kpad(lp)) or xq.dtype != torch.int8:
+        raise RuntimeError("xq must be the int8 [I, kpad(L')] buffer written by abc_forward")
+    need = _lib.lib().hot_backward_workspace_bytes(L, O, I, C.byref(cfg))
+    if need == 0:
+        raise HotError("bad configuration: %s" % _lib.lib().hot_last_error().decode())
+    if workspace is None or workspace.numel() < need:
+        workspace = _ws(need, gy.device)
+    gx = torch.empty((L, I), dtype=out_dtype, device=gy.device)
+    gw = torch.empty((O, I), dtype=out_dtype, device=gy.device)
+    times = (C.c_float * 4)() if timing else None
+    _lib.check(_lib.lib().hot_linear_backward(gy.data_ptr(), w.data_ptr(), _dt(gy), xq.data_ptr(), sx.data_ptr(),
+                                              L, O, I, C.byref(cfg), gx.data_ptr(), gw.data_ptr(),
+                                              _DTYPES[out_dtype], workspace.data_ptr(), workspace.numel(), times,
+                                              _stream()))
+    if timing:
+        return gx, gw, [float(t) for t in times]
+    return gx, gw

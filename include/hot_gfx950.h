@@ -1,0 +1,167 @@
+/*
+ * libhot_gfx950 -- C ABI of the MI355X-native HOT linear-layer backward path.
+ *
+ * Plain pointers and sizes only; every pointer named "device" must point to
+ * memory of the current HIP device.  Every function returns 0 on success or a
+ * negative hot_status; hot_last_error() gives the message of the last failure
+ * on the calling thread.  No function allocates or frees device memory and
+ * none synchronises the stream, except hot_linear_backward() when it is asked
+ * for stage timings.
+ *
+ * What each entry point replaces in the reference (sungonuni/HOT):
+ *   hot_hq_rowwise       fwht_kernel + find_scale_kernel + quant_int4_kernel /
+ *                        quant_int4_per_token_kernel / quant_int8_kernel
+ *                        (cuda_measure/HLQ_backward_kernel.cu:39-178,282-307);
+ *                        numerics of lowering_matmul_front + *_quantizer_BWD
+ *                        (utils/hadamard_matmul.py:121-141,
+ *                         utils/quant_matmul.py:19-31,86-116)
+ *   hot_hla_tokenwise    lowering_matmul_back(P, .) + quantiser + the
+ *                        transposes feeding the int8 GEMM
+ *                        (utils/hadamard_matmul.py:143-161,209-226;
+ *                         utils/quant_matmul.py:190,197-198,301,307-320;
+ *                         HLQ_backward_kernel.cu:539-543,593-596,607-611)
+ *   hot_wq_colwise       lowering_matmul_back(H_n, W) + quantiser + W^T pack
+ *                        (utils/quant_matmul.py:270,276-285;
+ *                         HLQ_backward_kernel.cu:533-537,561,587-591)
+ *   hot_gemm_i8          CutlassSgemmNN_int4 / CutlassSgemmNN_int8 +
+ *                        dequantize_cuda(_per_token)_kernel
+ *                        (HLQ_backward_kernel.cu:181-280,309-384,386-450)
+ *   hot_abc_forward      FLinearQ.setup_context (utils/quant_matmul.py:178-212)
+ *   hot_linear_backward  backward_cuda (HLQ_backward_kernel.cu:457-737) with
+ *                        the numerics of FLinearQ.backward, scheme gih_gwlr
+ *                        (utils/quant_matmul.py:215-348)
+ */
+#ifndef HOT_GFX950_H
+#define HOT_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HOT_ABI_VERSION 1
+#define HOT_API __attribute__((visibility("default")))
+
+enum hot_status {
+  HOT_OK = 0,
+  HOT_ERR_INVALID = -1,     /* bad argument (null pointer, bad enum, bad size) */
+  HOT_ERR_UNSUPPORTED = -2, /* shape or option outside what the kernels cover */
+  HOT_ERR_WORKSPACE = -3,   /* workspace too small */
+  HOT_ERR_HIP = -4          /* a HIP runtime call failed */
+};
+
+enum hot_dtype { HOT_F32 = 0, HOT_BF16 = 1, HOT_F16 = 2 };
+enum hot_rounding { HOT_ROUND_NEAREST = 0, HOT_ROUND_STOCH = 1 };
+enum hot_scale_mode {
+  HOT_SCALE_TENSOR = 0, /* one absmax step for the whole tensor */
+  HOT_SCALE_ROW = 1,    /* one absmax step per row of the quantised matrix */
+  HOT_SCALE_SAWB = 2    /* one step from clip = 12.1 rms - 12.2 mean|.| */
+};
+
+/* Counter-based RNG stream identifiers (Philox counter word 2). */
+enum hot_rng_stream { HOT_STREAM_GX = 0, HOT_STREAM_GW = 1, HOT_STREAM_W = 2, HOT_STREAM_ACT = 3 };
+
+#define HOT_MAX_HLA_N 64
+
+/* Options of the fused path; mirrors the fields FLinearQ reads from the
+ * reference's module-global `args` (args.py:29-49), scheme gih_gwlr. */
+typedef struct hot_config {
+  int32_t n_o;      /* Hadamard block along O: 16, 32 or 64                       */
+  int32_t hla_n;    /* HLA block along tokens: 1, 2, 4, ..., HOT_MAX_HLA_N        */
+  int32_t hla_r;    /* kept coefficients per block, 1..hla_n                      */
+  int32_t hla_rows[HOT_MAX_HLA_N]; /* natural-order row of output coefficient k  */
+  int32_t gx_bits, w_bits, gw_bits, act_bits;         /* 4 or 8                   */
+  int32_t gx_round, w_round, gw_round, act_round;     /* hot_rounding             */
+  int32_t gx_scale, w_scale, gw_scale, act_scale;     /* hot_scale_mode           */
+  uint64_t seed;    /* stochastic-rounding key                                    */
+} hot_config;
+
+HOT_API const char* hot_last_error(void);
+HOT_API int hot_abi_version(void);
+
+/* Bytes of the leading dimension (row pitch) the library uses for a K-major
+ * int8 code matrix with `k` codes per row: k rounded up to the GEMM K-tile. */
+HOT_API int64_t hot_kpad(int64_t k);
+
+/*
+ * Block-Hadamard along the contiguous dimension + absmax step + quantise.
+ *   in          device, [M, K] row-major, dtype
+ *   n           Hadamard block, 16 | 32 | 64; K % n == 0
+ *   bits        4: codes_out is [M, K/2] bytes, element 2j in bits 3:0 of byte j
+ *               8: codes_out is [M, K] int8
+ *   scale_mode  HOT_SCALE_TENSOR -> scales_out[1]; HOT_SCALE_ROW -> scales_out[M]
+ *   workspace   device, >= 256 bytes, 256-byte aligned (TENSOR mode only)
+ */
+HOT_API int hot_hq_rowwise(const void* in, int dtype, int64_t M, int64_t K, int n, int bits,
+                   int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
+                   void* codes_out, float* scales_out, void* workspace,
+                   size_t workspace_bytes, void* hip_stream);
+
+/*
+ * Hadamard low-rank projection along the row (token) dimension, quantise, and
+ * store TRANSPOSED (K-major) for the int8 GEMM.
+ *   in          device, [R, C] row-major, dtype; R % n == 0
+ *   rows        host, r natural-order row indices in [0, n)
+ *   codes_out   device, logical [C, (R/n)*r] codes; row pitch ld_out bytes;
+ *               bytes beyond the logical row up to ld_out are written as zero
+ *   scales_out  [1] (TENSOR, SAWB) or [C] (ROW)
+ *   workspace   device, >= hot_colwise_workspace_bytes(C)
+ * The stochastic-rounding element index of coefficient (c, k) is c*Kout + k.
+ */
+HOT_API int hot_hla_tokenwise(const void* in, int dtype, int64_t R, int64_t C, int n,
+                      const int32_t* rows, int r, int bits, int rounding, uint64_t seed,
+                      uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_out,
+                      float* scales_out, void* workspace, size_t workspace_bytes,
+                      void* hip_stream);
+
+/* Full block-Hadamard (all n rows kept) along the row dimension of W [O, I],
+ * quantise, store as [I, O] codes (K-major).  Same conventions as above. */
+HOT_API int hot_wq_colwise(const void* in, int dtype, int64_t O, int64_t I, int n, int bits,
+                   int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
+                   void* codes_out, int64_t ld_out, float* scales_out, void* workspace,
+                   size_t workspace_bytes, void* hip_stream);
+
+HOT_API size_t hot_colwise_workspace_bytes(int64_t C);
+
+/*
+ * out[M, N] = ((acc * scale_a[row or 0]) * scale_b[0]) * post_scale,
+ * acc[M, N] (int32) = A[M, K] . B[N, K]^T on integer codes (MFMA int8).
+ *   A, B        device, K-major codes, both `bits` wide (4: packed nibbles,
+ *               8: int8); row pitches lda, ldb in BYTES, each >= the bytes of
+ *               hot_kpad(K) codes, and the codes in [K, hot_kpad(K)) must be 0
+ *   scale_a     device; [M] when a_per_row != 0, else [1]
+ *   out         device, [M, N] row-major of out_dtype, pitch ldo ELEMENTS
+ *   acc_out     device int32 [M, N] (pitch N) or NULL
+ */
+HOT_API int hot_gemm_i8(const void* A, int64_t lda, const void* B, int64_t ldb, int bits,
+                int64_t M, int64_t N, int64_t K, const float* scale_a, int a_per_row,
+                const float* scale_b, float post_scale, void* out, int out_dtype,
+                int64_t ldo, int32_t* acc_out, void* hip_stream);
+
+/* Forward-side activation buffer: xq[I, hot_kpad(L')] = quant8(P x)^T, sx[1]. */
+HOT_API size_t hot_abc_workspace_bytes(int64_t L, int64_t I, const hot_config* cfg);
+HOT_API int hot_abc_forward(const void* x, int dtype, int64_t L, int64_t I, const hot_config* cfg,
+                    void* xq_out, float* sx_out, void* workspace, size_t workspace_bytes,
+                    void* hip_stream);
+
+/*
+ * The fused backward: g_x[L, I] and g_W[O, I] (both of out_dtype, dense).
+ *   gy [L, O], w [O, I] of dtype; xq / sx as written by hot_abc_forward
+ *   times4      host, NULL or 4 floats receiving the seconds spent in
+ *               {transform+quantise of g_y (both operands), transform+quantise
+ *               of W, g_x GEMM+dequant, g_W GEMM+dequant}; non-NULL makes the
+ *               call synchronise the stream
+ */
+HOT_API size_t hot_backward_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_config* cfg);
+HOT_API int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq,
+                        const float* sx, int64_t L, int64_t O, int64_t I,
+                        const hot_config* cfg, void* gx, void* gw, int out_dtype,
+                        void* workspace, size_t workspace_bytes, float* times4,
+                        void* hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HOT_GFX950_H */

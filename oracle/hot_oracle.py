@@ -1,0 +1,455 @@
+"""Canonical CPU oracle (NumPy, fp32) for the HOT linear backward path.
+
+TEST INFRASTRUCTURE ONLY -- never imported by the shipped package.
+
+Every function restates one piece of the reference's fake-quant path
+(/root/reference/utils/quant_matmul.py, utils/hadamard_matmul.py) or of the
+wire format of its CUDA op (cuda_measure/HLQ_backward_kernel.cu); the cited
+file:line is given per function.  Two deliberate, documented differences:
+
+* Transforms are evaluated as fp32 butterflies in ONE fixed order
+  (h = 1, 2, 4, ...; (x+y, x-y)), the order of the reference CUDA kernel
+  ``fwht_kernel`` (HLQ_backward_kernel.cu:63-78), instead of the BLAS matmul
+  ``reshape(-1, n) @ H`` of hadamard_matmul.py:121-161 whose last-ulp
+  summation order depends on the BLAS build.  Mathematically identical.
+* Stochastic rounding draws its uniforms from Philox-4x32-10 keyed by
+  (seed, element index) instead of the global torch generator
+  (quant_matmul.py:96), so that CPU and GPU agree bit for bit.
+
+How each function is pinned (tests/test_oracle_*.py):
+  pow2_factor / pow2_factor_max16   closed form n & -n; hand-derived table
+  hadamard                          scipy.linalg.hadamard; H H^T = n I
+  sequency_of_natural / wht_rows    brute-force sign-change count + stable sort
+  kept_sequencies                   hand-derived sets for n = 1, 2, 4, 16, 64
+  fwht_blocks_last / _first         explicit block-diagonal matmul on small
+                                    integer inputs (exact in fp32)
+  quant_rne / quant_sr / quant_sawb textbook absmax quantiser; ties-to-even
+                                    table; all-zero input; max -> +-qmax;
+                                    SR mean/variance; Philox known answers
+  pack_int4 / unpack_int4           all 225 code pairs round trip; byte value
+                                    formula of HLQ_backward_kernel.cu:140
+  int_gemm_nt                       numpy int64 matmul
+  linear_backward / abc_forward     composition; with quantisation off and
+                                    r = n they equal g_y W and g_y^T x
+No function here is "parity unpinned" except the last-ulp BLAS summation order
+of the reference's transform matmuls, which is intentionally not matched.
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass, field
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+
+F32 = np.float32
+EPS = 1e-11  # args.py:34
+
+# --------------------------------------------------------------------------
+# sizes and matrices
+# --------------------------------------------------------------------------
+
+
+def pow2_factor(size: int) -> int:
+    """Largest power-of-two divisor of ``size`` (hadamard_matmul.py:9-15)."""
+    if size < 1:
+        raise ValueError("size must be >= 1")
+    return size & -size
+
+
+def pow2_factor_max16(size: int) -> int:
+    """hadamard_matmul.py:17-27: as pow2_factor but 16 when the factor exceeds
+    16 (and size > 16)."""
+    p = pow2_factor(size)
+    return 16 if (p > 16 and size > 16) else p
+
+
+def hadamard(n: int) -> np.ndarray:
+    """Sylvester Hadamard matrix, natural order, entries +-1
+    (hadamard_matmul.py:32-51).  H[i, j] = (-1)^popcount(i & j)."""
+    if n < 1 or (n & (n - 1)):
+        raise ValueError("n must be int and power of 2.")
+    i = np.arange(n, dtype=np.int64)
+    a = i[:, None] & i[None, :]
+    pc = np.zeros_like(a)
+    while a.any():
+        pc += a & 1
+        a >>= 1
+    return (1 - 2 * (pc & 1)).astype(np.int64)
+
+
+def make_hadamard(size: int) -> np.ndarray:
+    """hadamard_matmul.py:57-59."""
+    return hadamard(pow2_factor_max16(size))
+
+
+def sequency_of_natural(n: int) -> np.ndarray:
+    """seq[i] = number of sign changes along row i of the Sylvester matrix
+    = gray_decode(bit_reverse(i)).  (Replaces the row sort by counted sign
+    changes of hadamard_matmul.py:210-213.)"""
+    bits = n.bit_length() - 1
+    out = np.zeros(n, dtype=np.int64)
+    for i in range(n):
+        r = 0
+        for b in range(bits):
+            if i >> b & 1:
+                r |= 1 << (bits - 1 - b)
+        g = r
+        s = r >> 1
+        while s:
+            g ^= s
+            s >>= 1
+        out[i] = g
+    return out
+
+
+def natural_of_sequency(n: int) -> np.ndarray:
+    """Inverse permutation of sequency_of_natural."""
+    seq = sequency_of_natural(n)
+    inv = np.empty(n, dtype=np.int64)
+    inv[seq] = np.arange(n)
+    return inv
+
+
+def kept_sequencies(n: int, percentile: float = 50) -> np.ndarray:
+    """Sequency indices kept by the low-rank selection of make_WHT
+    (hadamard_matmul.py:215-225), increasing order."""
+    # biggest_sqrt_factor (hadamard_matmul.py:172-178): largest power of 4 <= n
+    p4 = 1
+    while p4 * 4 <= n:
+        p4 *= 4
+    s = int(math.isqrt(p4))
+    sf = int(0.1 * (-np.sqrt(2 * s ** 2 * percentile + 25) + 10 * s + 5))
+    idx = np.arange(n)
+    parts = []
+    for i in range(s):
+        if i % 2 == 0:
+            parts.append(idx[s * i: s * (i + 1) - (i + sf)])
+        else:
+            parts.append(idx[s * i + (i + sf): s * (i + 1)])
+    return np.concatenate(parts).astype(np.int64)
+
+
+def hla_rows(size: int, percentile: float = 50) -> Tuple[int, np.ndarray]:
+    """(n, natural-order row index of each kept coefficient, in output order)
+    for a token count ``size``: the python rule of make_WHT
+    (hadamard_matmul.py:209-226; n = make_non_block_hadamard :167-170)."""
+    n = 1 if size == 1 else pow2_factor(size)
+    keep = kept_sequencies(n, percentile)
+    return n, natural_of_sequency(n)[keep]
+
+
+def make_WHT(size: int, percentile: float = 50) -> np.ndarray:
+    """The r x n matrix P of hadamard_matmul.py:209-226."""
+    n, rows = hla_rows(size, percentile)
+    return hadamard(n)[rows]
+
+
+def paper_rows(n: int = 16, r: int = 8) -> Tuple[int, np.ndarray]:
+    """Cost-model setting (analysis_calculator.py:174-175): the r lowest
+    sequencies of an n-block."""
+    return n, natural_of_sequency(n)[np.arange(r)]
+
+
+# --------------------------------------------------------------------------
+# transforms, canonical butterfly order (HLQ_backward_kernel.cu:63-78)
+# --------------------------------------------------------------------------
+
+
+def _fwht_axis(v: np.ndarray, axis: int) -> np.ndarray:
+    """Unnormalised FWHT of length v.shape[axis] (a power of two) along
+    ``axis``: stages h = 1, 2, 4, ...; pair (j, j+h) with (j // h) even becomes
+    (v[j] + v[j+h], v[j] - v[j+h]).  fp32 throughout."""
+    v = np.ascontiguousarray(np.moveaxis(v, axis, -1), dtype=F32).copy()
+    n = v.shape[-1]
+    h = 1
+    while h < n:
+        w = v.reshape(v.shape[:-1] + (n // (2 * h), 2, h))
+        a = w[..., 0, :].copy()
+        b = w[..., 1, :].copy()
+        w[..., 0, :] = a + b
+        w[..., 1, :] = a - b
+        h *= 2
+    return np.moveaxis(v, -1, axis)
+
+
+def fwht_blocks_last(a: np.ndarray, n: int) -> np.ndarray:
+    """A [.., K] -> each contiguous n-chunk of the last dim times H_n:
+    lowering_matmul_front(A, H_n) (hadamard_matmul.py:121-141)."""
+    a = np.asarray(a, dtype=F32)
+    k = a.shape[-1]
+    if k % n:
+        raise ValueError("last dim must be a multiple of n")
+    return _fwht_axis(a.reshape(a.shape[:-1] + (k // n, n)), -1).reshape(a.shape)
+
+
+def fwht_blocks_first(a: np.ndarray, n: int, rows: Optional[np.ndarray] = None) -> np.ndarray:
+    """A [R, C] -> H_n applied to every block of n consecutive rows; when
+    ``rows`` (natural-order indices) is given only those coefficients of each
+    block are kept, in that order: out[b*r + k, :] = T_b[rows[k], :].
+    = lowering_matmul_back(H_n or P, A) (hadamard_matmul.py:143-161)."""
+    a = np.asarray(a, dtype=F32)
+    R, C = a.shape
+    if R % n:
+        raise ValueError("row count must be a multiple of n")
+    t = _fwht_axis(a.reshape(R // n, n, C), 1)
+    if rows is not None:
+        t = t[:, np.asarray(rows), :]
+    return np.ascontiguousarray(t.reshape(-1, C))
+
+
+# --------------------------------------------------------------------------
+# Philox-4x32-10 (Salmon et al., SC'11) -- counter-based uniforms for SR
+# --------------------------------------------------------------------------
+
+_PH_M0 = np.uint64(0xD2511F53)
+_PH_M1 = np.uint64(0xCD9E8D57)
+_PH_W0 = 0x9E3779B9
+_PH_W1 = 0xBB67AE85
+_MASK = np.uint64(0xFFFFFFFF)
+
+
+def philox4x32(c0, c1, c2, c3, k0: int, k1: int, rounds: int = 10):
+    """Vectorised Philox-4x32; counters are uint32 arrays, key two ints."""
+    c0 = np.asarray(c0, dtype=np.uint64)
+    c1 = np.asarray(c1, dtype=np.uint64)
+    c2 = np.asarray(c2, dtype=np.uint64)
+    c3 = np.asarray(c3, dtype=np.uint64)
+    k0 &= 0xFFFFFFFF
+    k1 &= 0xFFFFFFFF
+    for _ in range(rounds):
+        p0 = _PH_M0 * c0
+        p1 = _PH_M1 * c2
+        hi0, lo0 = p0 >> np.uint64(32), p0 & _MASK
+        hi1, lo1 = p1 >> np.uint64(32), p1 & _MASK
+        c0, c1, c2, c3 = (hi1 ^ c1 ^ np.uint64(k0)), lo1, (hi0 ^ c3 ^ np.uint64(k1)), lo0
+        k0 = (k0 + _PH_W0) & 0xFFFFFFFF
+        k1 = (k1 + _PH_W1) & 0xFFFFFFFF
+    return (c0.astype(np.uint32), c1.astype(np.uint32), c2.astype(np.uint32), c3.astype(np.uint32))
+
+
+def sr_uniform(index: np.ndarray, seed: int, stream: int) -> np.ndarray:
+    """u in [0, 1) on a 2^-24 grid for the element with linear index ``index``
+    (int64 array): counter = (index>>2 lo, index>>2 hi, stream, 0),
+    key = (seed lo, seed hi), word = index & 3, u = (word >> 8) * 2^-24."""
+    index = np.asarray(index, dtype=np.uint64)
+    q = index >> np.uint64(2)
+    w = philox4x32(q & _MASK, q >> np.uint64(32), np.full(q.shape, stream, np.uint64),
+                   np.zeros(q.shape, np.uint64), seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF)
+    lane = (index & np.uint64(3)).astype(np.int64)
+    word = np.choose(lane, w)
+    return ((word >> np.uint32(8)).astype(F32) * F32(2.0 ** -24)).astype(F32)
+
+
+# --------------------------------------------------------------------------
+# quantisers
+# --------------------------------------------------------------------------
+
+ROUND_NEAREST = 0
+ROUND_STOCH = 1
+SCALE_TENSOR = 0
+SCALE_ROW = 1
+SCALE_SAWB = 2
+
+STREAM_GX = 0   # g_y H  quantiser
+STREAM_GW = 1   # (P g_y)^T quantiser
+STREAM_W = 2    # H W quantiser
+STREAM_ACT = 3  # P x quantiser
+
+
+def _qmax(bits: int) -> int:
+    return 2 ** (bits - 1) - 1
+
+
+def quant_scale(t: np.ndarray, bits: int, mode: int) -> np.ndarray:
+    """Step size s (WITHOUT eps) and clip: int_quantizer_BWD
+    (quant_matmul.py:112-113), norm_quantizer_BWD (:20-21),
+    sawb_quantizer_BWD (:41-44).  Returns (s, clip) broadcastable to t."""
+    t = np.asarray(t, dtype=F32)
+    q = F32(_qmax(bits))
+    if mode == SCALE_TENSOR:
+        mx = np.max(np.abs(t)).astype(F32) if t.size else F32(0)
+        return (mx / q).astype(F32), mx
+    if mode == SCALE_ROW:
+        mx = np.max(np.abs(t), axis=1, keepdims=True).astype(F32)
+        return (mx / q).astype(F32), mx
+    if mode == SCALE_SAWB:
+        # sums in float64, result rounded to fp32 once
+        t64 = t.astype(np.float64)
+        clip = F32(12.1 * np.sqrt(np.mean(t64 * t64)) - 12.2 * np.mean(np.abs(t64)))
+        return (clip / q).astype(F32), clip
+    raise ValueError("bad scale mode")
+
+
+def quant(t: np.ndarray, bits: int, mode: int = SCALE_TENSOR, rounding: int = ROUND_NEAREST,
+          seed: int = 0, stream: int = 0, index: Optional[np.ndarray] = None):
+    """Codes (int8) and step size s (fp32, without eps).
+
+    y = clamp(t, -clip, clip) / fl32(s + 1e-11)           (IEEE fp32 division)
+    nearest:     q = rint(y), ties to even   (int_quantizer_BWD  :112-116,
+                                              sawb_quantizer_BWD :40-49)
+    stochastic:  q = sign(y) (floor|y| + (u < |y| - floor|y|))
+                                             (stoch_quantizer_BWD :86-100,
+                                              norm_quantizer_BWD  :19-31)
+    ``index`` gives the RNG element index of every entry (default: row-major
+    position in t)."""
+    t = np.asarray(t, dtype=F32)
+    s, clip = quant_scale(t, bits, mode)
+    d = (s + F32(EPS)).astype(F32)
+    y = (np.clip(t, -clip, clip).astype(F32) / d).astype(F32)
+    if rounding == ROUND_NEAREST:
+        q = np.rint(y)
+    else:
+        if index is None:
+            index = np.arange(t.size, dtype=np.int64).reshape(t.shape)
+        u = sr_uniform(index, seed, stream)
+        ay = np.abs(y)
+        fl = np.floor(ay)
+        frac = (ay - fl).astype(F32)
+        q = np.sign(y) * (fl + (u < frac))
+    qm = _qmax(bits)
+    q = np.clip(q, -qm, qm)  # never active for absmax scales; guards sawb/eps
+    s_out = s.reshape(-1) if mode == SCALE_ROW else np.asarray(s, dtype=F32).reshape(1)
+    return q.astype(np.int8), s_out.astype(F32)
+
+
+# --------------------------------------------------------------------------
+# INT4 wire format (HLQ_backward_kernel.cu:135-140; = cutlass::int4b_t order)
+# --------------------------------------------------------------------------
+
+
+def pack_int4(q: np.ndarray) -> np.ndarray:
+    """[.., K] int8 codes in [-8, 7] -> [.., K/2] bytes; byte j holds element
+    2j in bits 3:0 and element 2j+1 in bits 7:4 (two's complement nibbles)."""
+    q = np.asarray(q, dtype=np.int8)
+    if q.shape[-1] % 2:
+        raise ValueError("K must be even")
+    u = q.view(np.uint8)
+    return ((u[..., 1::2] << 4) | (u[..., 0::2] & 0x0F)).astype(np.uint8).view(np.int8)
+
+
+def unpack_int4(p: np.ndarray) -> np.ndarray:
+    p = np.asarray(p).view(np.uint8)
+    lo = (p & 0x0F).astype(np.int16)
+    hi = (p >> 4).astype(np.int16)
+    lo = np.where(lo > 7, lo - 16, lo)
+    hi = np.where(hi > 7, hi - 16, hi)
+    out = np.empty(p.shape[:-1] + (p.shape[-1] * 2,), dtype=np.int8)
+    out[..., 0::2] = lo
+    out[..., 1::2] = hi
+    return out
+
+
+# --------------------------------------------------------------------------
+# integer GEMM contract (HLQ_backward_kernel.cu:181-280, 309-384)
+# --------------------------------------------------------------------------
+
+
+def int_gemm_nt(a: np.ndarray, b: np.ndarray) -> np.ndarray:
+    """C[M, N] (int32) = A[M, K] . B[N, K]^T on integer codes.  Evaluated in
+    float64 BLAS, exact because |acc| <= 127^2 K << 2^53."""
+    c = np.asarray(a, dtype=np.float64) @ np.asarray(b, dtype=np.float64).T
+    return np.rint(c).astype(np.int64).astype(np.int32)
+
+
+# --------------------------------------------------------------------------
+# the path: forward activation buffer (ABC) and backward
+# --------------------------------------------------------------------------
+
+
+@dataclass
+class HotConfig:
+    """The knobs FLinearQ reads from the module ``args`` (args.py:29-49),
+    restricted to scheme ``gih_gwlr``."""
+    n_o: int = 16                      # Hadamard block along O (make_hadamard)
+    hla_n: int = 1                     # HLA block along tokens
+    hla_rows: Sequence[int] = (0,)     # kept natural-order rows, output order
+    gx_bits: int = 4                   # GogiQuantBit
+    w_bits: int = 4                    # weightQuantBit
+    gw_bits: int = 8                   # GogwQuantBit
+    act_bits: int = 8                  # actQuantBit
+    gx_round: int = ROUND_NEAREST      # quantBWDGogi: int | stoch | nq
+    gx_scale: int = SCALE_TENSOR       #   nq = stochastic + SCALE_ROW
+    w_round: int = ROUND_NEAREST       # quantBWDWgt: int | stoch | sawb
+    w_scale: int = SCALE_TENSOR
+    gw_round: int = ROUND_NEAREST      # quantBWDGogw
+    gw_scale: int = SCALE_TENSOR
+    act_round: int = ROUND_NEAREST     # quantBWDAct
+    act_scale: int = SCALE_TENSOR
+    seed: int = 0
+
+    @staticmethod
+    def python_rule(L: int, **kw) -> "HotConfig":
+        n, rows = hla_rows(L)
+        return HotConfig(hla_n=n, hla_rows=tuple(int(v) for v in rows), **kw)
+
+    @staticmethod
+    def paper(n: int = 16, r: int = 8, **kw) -> "HotConfig":
+        n, rows = paper_rows(n, r)
+        return HotConfig(hla_n=n, hla_rows=tuple(int(v) for v in rows), **kw)
+
+
+def abc_forward(x: np.ndarray, cfg: HotConfig):
+    """FLinearQ.setup_context (quant_matmul.py:178-212), scheme gih_gwlr:
+    x <- P x (HLA along tokens) then quantise to INT8.
+    Returns (xq int8 [L', I], sx fp32 [1])."""
+    xp = fwht_blocks_first(np.asarray(x, dtype=F32), cfg.hla_n, np.asarray(cfg.hla_rows))
+    return quant(xp, cfg.act_bits, cfg.act_scale, cfg.act_round, cfg.seed, STREAM_ACT)
+
+
+@dataclass
+class BackwardTrace:
+    qG: np.ndarray = None
+    sG: np.ndarray = None
+    qW: np.ndarray = None
+    sW: np.ndarray = None
+    acc_x: np.ndarray = None
+    qGp: np.ndarray = None
+    sGp: np.ndarray = None
+    acc_w: np.ndarray = None
+    g_x: np.ndarray = None
+    g_w: np.ndarray = None
+
+
+def linear_backward(g_y: np.ndarray, w: np.ndarray, xq: np.ndarray, sx: np.ndarray,
+                    cfg: HotConfig) -> BackwardTrace:
+    """FLinearQ.backward (quant_matmul.py:215-348), scheme gih_gwlr, 2-D inputs.
+
+    g_y [L, O], w [O, I], xq int8 [L', I] with step sx (from abc_forward)."""
+    g_y = np.asarray(g_y, dtype=F32)
+    w = np.asarray(w, dtype=F32)
+    L, O = g_y.shape
+    tr = BackwardTrace()
+    # :238  g_y blkdiag(H)  ; :244-257 quantise
+    G = fwht_blocks_last(g_y, cfg.n_o)
+    tr.qG, tr.sG = quant(G, cfg.gx_bits, cfg.gx_scale, cfg.gx_round, cfg.seed, STREAM_GX)
+    # :270  blkdiag(H) W ; :276-285 quantise
+    Wh = fwht_blocks_first(w, cfg.n_o)
+    tr.qW, tr.sW = quant(Wh, cfg.w_bits, cfg.w_scale, cfg.w_round, cfg.seed, STREAM_W)
+    # :288-290, :343
+    tr.acc_x = int_gemm_nt(tr.qG, tr.qW.T)
+    sg = tr.sG.reshape(-1, 1) if cfg.gx_scale == SCALE_ROW else tr.sG.reshape(1, 1)
+    tr.g_x = (((tr.acc_x.astype(F32) * sg).astype(F32) * tr.sW[0]).astype(F32) / F32(cfg.n_o)).astype(F32)
+    # :301 (P g_y)^T ; :307-320 quantise
+    GpT = np.ascontiguousarray(fwht_blocks_first(g_y, cfg.hla_n, np.asarray(cfg.hla_rows)).T)
+    tr.qGp, tr.sGp = quant(GpT, cfg.gw_bits, cfg.gw_scale, cfg.gw_round, cfg.seed, STREAM_GW)
+    # :322-324, :344
+    tr.acc_w = int_gemm_nt(tr.qGp, np.asarray(xq).T)
+    sgw = tr.sGp.reshape(-1, 1) if cfg.gw_scale == SCALE_ROW else tr.sGp.reshape(1, 1)
+    tr.g_w = (((tr.acc_w.astype(F32) * sgw).astype(F32) * F32(np.asarray(sx).reshape(-1)[0])).astype(F32)
+              / F32(cfg.hla_n)).astype(F32)
+    return tr
+
+
+def stoch_round_mantissa(x: np.ndarray) -> np.ndarray:
+    """The reference CUDA op's pseudo-stochastic rounding
+    (HLQ_backward_kernel.cu:19-36), kept only to characterise its bias; the
+    build does not use it."""
+    x = np.asarray(x, dtype=F32)
+    bits = x.view(np.uint32)
+    mant = bits & np.uint32(0x007FFFFF)
+    prob = mant >> np.uint32(11)
+    rnd = mant & np.uint32(0x7FF)
+    flip = (prob <= rnd).astype(np.int64)
+    sign = np.where(x < 0, -1, 1)
+    return sign * (np.floor(np.abs(x)).astype(np.int64) + flip)

@@ -1,0 +1,276 @@
+"""Parity of every HIP kernel (through the C ABI) with the CPU oracle.
+
+Integer stages (codes, int32 accumulators) must be bit-exact; step sizes are
+fp32 values computed by the same IEEE operations and must be equal too.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import hot_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+TDT = {"f32": torch.float32, "bf16": torch.bfloat16, "f16": torch.float16}
+
+
+def make_input(M, K, dtype, seed, outliers=True):
+    """g_y-like data: N(0, 1e-3) with 1 % of entries x50, rounded to dtype."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(M, K, generator=g) * 1e-3
+    if outliers:
+        mask = torch.rand(M, K, generator=g) < 0.01
+        x = torch.where(mask, x * 50, x)
+    x = x.to(TDT[dtype])
+    return x, x.float().numpy()
+
+
+def np_codes(codes, bits, K):
+    c = codes.cpu().numpy()
+    return orc.unpack_int4(c)[:, :K] if bits == 4 else c[:, :K]
+
+
+# ---------------------------------------------------------------- hq_rowwise
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16", "f16"])
+@pytest.mark.parametrize("n", [16, 32, 64])
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("scale", ["tensor", "row"])
+def test_hq_rowwise_nearest(gpu, dtype, n, bits, scale):
+    from hot_amd import ops
+    M, K = 300, 768
+    x, xn = make_input(M, K, dtype, seed=n + bits)
+    codes, s = ops.hq_rowwise(x.to(gpu), n=n, bits=bits, rounding="nearest", scale=scale)
+    mode = orc.SCALE_ROW if scale == "row" else orc.SCALE_TENSOR
+    q_ref, s_ref = orc.quant(orc.fwht_blocks_last(xn, n), bits, mode)
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    assert np.array_equal(np_codes(codes, bits, K), q_ref)
+
+
+@pytest.mark.parametrize("K", [16, 64, 1024, 3072, 4096, 11008, 20480])
+@pytest.mark.parametrize("scale", ["tensor", "row"])
+def test_hq_rowwise_widths(gpu, K, scale):
+    """Every per-row chunk count the dispatcher can pick, and ragged last sweeps."""
+    from hot_amd import ops
+    M = 37
+    x, xn = make_input(M, K, "bf16", seed=K)
+    codes, s = ops.hq_rowwise(x.to(gpu), n=16, bits=4, scale=scale)
+    mode = orc.SCALE_ROW if scale == "row" else orc.SCALE_TENSOR
+    q_ref, s_ref = orc.quant(orc.fwht_blocks_last(xn, 16), 4, mode)
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    assert np.array_equal(np_codes(codes, 4, K), q_ref)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("scale", ["tensor", "row"])
+def test_hq_rowwise_stochastic_matches_oracle(gpu, dtype, bits, scale):
+    """Same counter-based RNG on both sides: identical codes for a given seed."""
+    from hot_amd import ops
+    M, K = 200, 1536
+    x, xn = make_input(M, K, dtype, seed=5)
+    seed = 0x1234_5678_9ABC_DEF0
+    codes, s = ops.hq_rowwise(x.to(gpu), n=16, bits=bits, rounding="stoch", scale=scale, seed=seed)
+    mode = orc.SCALE_ROW if scale == "row" else orc.SCALE_TENSOR
+    q_ref, s_ref = orc.quant(orc.fwht_blocks_last(xn, 16), bits, mode, orc.ROUND_STOCH, seed, orc.STREAM_GX)
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    assert np.array_equal(np_codes(codes, bits, K), q_ref)
+
+
+def test_hq_rowwise_stochastic_unbiased(gpu):
+    """E[q] = y over seeds: the mean code of many seeds approaches y = t/d and
+    every code is floor(y) or ceil(y)."""
+    from hot_amd import ops
+    M, K = 64, 256
+    x, xn = make_input(M, K, "f32", seed=11, outliers=False)
+    t = orc.fwht_blocks_last(xn, 16)
+    s, _ = orc.quant_scale(t, 4, orc.SCALE_TENSOR)
+    y = t / (s + np.float32(orc.EPS))
+    xd = x.to(gpu)
+    nseed = 400
+    acc = np.zeros_like(y, dtype=np.float64)
+    for seed in range(nseed):
+        codes, _ = ops.hq_rowwise(xd, n=16, bits=4, rounding="stoch", scale="tensor", seed=seed)
+        q = np_codes(codes, 4, K).astype(np.float64)
+        assert np.all((q == np.floor(y)) | (q == np.ceil(y)))
+        acc += q
+    err = acc / nseed - y
+    # per-element std of the mean <= 0.5/sqrt(nseed) = 0.025; allow 5 sigma per element and a tight global mean
+    assert np.max(np.abs(err)) < 0.13
+    assert abs(err.mean()) < 5 * 0.5 / np.sqrt(nseed * y.size)
+
+
+def test_hq_rowwise_zero_and_empty(gpu):
+    from hot_amd import ops
+    z = torch.zeros(8, 64, device=gpu)
+    for scale in ("tensor", "row"):
+        codes, s = ops.hq_rowwise(z, n=16, bits=4, scale=scale)
+        assert torch.all(codes == 0) and torch.all(s == 0)
+    e = torch.zeros(0, 64, device=gpu)
+    codes, s = ops.hq_rowwise(e, n=16, bits=8, scale="row")
+    assert codes.shape == (0, 64)
+
+
+def test_hq_rowwise_errors(gpu):
+    from hot_amd import ops
+    from hot_amd._lib import HotError
+    with pytest.raises(HotError):
+        ops.hq_rowwise(torch.zeros(4, 40, device=gpu), n=16)        # K % n
+    with pytest.raises(HotError):
+        ops.hq_rowwise(torch.zeros(4, 64, device=gpu), n=8)         # block size
+    with pytest.raises(HotError):
+        ops.hq_rowwise(torch.zeros(4, 64, device=gpu), bits=5)
+    with pytest.raises(RuntimeError):
+        ops.hq_rowwise(torch.zeros(4, 64), n=16)                    # not on the GPU
+    with pytest.raises(RuntimeError):
+        ops.hq_rowwise(torch.zeros(4, 64, 2, device=gpu), n=16)     # not 2-D
+
+
+# ------------------------------------------------------------------- colwise
+
+def hla_case(L, C, dtype, seed):
+    return make_input(L, C, dtype, seed)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("n,rule", [(64, "python"), (16, "paper"), (32, "python"), (1, "python"), (4, "python"), (16, "python")])
+@pytest.mark.parametrize("scale", ["tensor", "row"])
+def test_hla_tokenwise_nearest(gpu, dtype, n, rule, scale):
+    from hot_amd import ops
+    L, C = n * 23 if n > 1 else 49, 200
+    if rule == "paper":
+        _, rows = orc.paper_rows(n, n // 2)
+    else:
+        nn, rows = orc.hla_rows(n) if n > 1 else (1, np.array([0]))
+        assert nn == n
+    x, xn = hla_case(L, C, dtype, seed=n)
+    codes, s, kout = ops.hla_tokenwise(x.to(gpu), n, list(rows), bits=8, scale=scale)
+    t = np.ascontiguousarray(orc.fwht_blocks_first(xn, n, rows).T)  # [C, L']
+    assert kout == t.shape[1]
+    mode = orc.SCALE_ROW if scale == "row" else orc.SCALE_TENSOR
+    q_ref, s_ref = orc.quant(t, 8, mode)
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    got = codes.cpu().numpy()
+    assert np.array_equal(got[:, :kout], q_ref)
+    assert not got[:, kout:].any(), "K padding must be zero"
+
+
+def test_hla_tokenwise_vit_shape_slice(gpu):
+    """n = 64, r = 36 on 12608 tokens (the ViT-B token count), bf16."""
+    from hot_amd import ops
+    L, C = 12608, 256
+    n, rows = orc.hla_rows(L)
+    assert (n, len(rows)) == (64, 36)
+    x, xn = hla_case(L, C, "bf16", seed=3)
+    codes, s, kout = ops.hla_tokenwise(x.to(gpu), n, list(rows), bits=8, scale="tensor")
+    assert kout == 7092
+    t = np.ascontiguousarray(orc.fwht_blocks_first(xn, n, rows).T)
+    q_ref, s_ref = orc.quant(t, 8, orc.SCALE_TENSOR)
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    got = codes.cpu().numpy()
+    assert np.array_equal(got[:, :kout], q_ref) and not got[:, kout:].any()
+
+
+@pytest.mark.parametrize("scale", ["tensor", "row"])
+def test_hla_tokenwise_stochastic_matches_oracle(gpu, scale):
+    from hot_amd import ops
+    L, C, n = 64 * 5, 72, 64
+    _, rows = orc.hla_rows(64)
+    x, xn = hla_case(L, C, "f32", seed=8)
+    codes, s, kout = ops.hla_tokenwise(x.to(gpu), n, list(rows), bits=8, rounding="stoch", scale=scale, seed=77)
+    t = np.ascontiguousarray(orc.fwht_blocks_first(xn, n, rows).T)
+    mode = orc.SCALE_ROW if scale == "row" else orc.SCALE_TENSOR
+    q_ref, s_ref = orc.quant(t, 8, mode, orc.ROUND_STOCH, 77, orc.STREAM_GW)
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    assert np.array_equal(codes.cpu().numpy()[:, :kout], q_ref)
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("n", [16, 32, 64])
+def test_wq_colwise_nearest(gpu, dtype, bits, n):
+    from hot_amd import ops
+    O, I = 64 * 7, 136
+    g = torch.Generator().manual_seed(n)
+    w = ((torch.rand(O, I, generator=g) * 2 - 1) / np.sqrt(I)).to(TDT[dtype])
+    codes, s = ops.wq_colwise(w.to(gpu), n=n, bits=bits)
+    t = np.ascontiguousarray(orc.fwht_blocks_first(w.float().numpy(), n).T)  # [I, O]
+    q_ref, s_ref = orc.quant(t, bits, orc.SCALE_TENSOR)
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    got = codes.cpu().numpy()
+    full = orc.unpack_int4(got) if bits == 4 else got
+    assert np.array_equal(full[:, :O], q_ref)
+    assert not full[:, O:].any()
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_wq_colwise_sawb(gpu, bits):
+    from hot_amd import ops
+    O, I = 256, 200
+    g = torch.Generator().manual_seed(1)
+    w = torch.randn(O, I, generator=g) * 0.05
+    codes, s = ops.wq_colwise(w.to(gpu), n=16, bits=bits, scale="sawb")
+    t = np.ascontiguousarray(orc.fwht_blocks_first(w.numpy(), 16).T)
+    q_ref, s_ref = orc.quant(t, bits, orc.SCALE_SAWB)
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    got = codes.cpu().numpy()
+    full = orc.unpack_int4(got) if bits == 4 else got
+    assert np.array_equal(full[:, :O], q_ref)
+
+
+# ---------------------------------------------------------------------- gemm
+
+def rand_codes(M, K, bits, seed):
+    rng = np.random.default_rng(seed)
+    qm = 2 ** (bits - 1) - 1
+    return rng.integers(-qm, qm + 1, size=(M, K), dtype=np.int8)
+
+
+def to_operand(q, bits, kp):
+    M, K = q.shape
+    full = np.zeros((M, kp), dtype=np.int8)
+    full[:, :K] = q
+    return torch.from_numpy(orc.pack_int4(full) if bits == 4 else full)
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+@pytest.mark.parametrize("M,N,K", [(128, 128, 128), (200, 72, 300), (1, 1, 16), (515, 260, 1000), (130, 768, 7092)])
+@pytest.mark.parametrize("per_row", [False, True])
+def test_gemm_i8_exact(gpu, bits, M, N, K, per_row):
+    from hot_amd import ops
+    a, b = rand_codes(M, K, bits, 1), rand_codes(N, K, bits, 2)
+    kp = ops.kpad(K)
+    rng = np.random.default_rng(3)
+    sa = rng.uniform(1e-4, 2e-4, size=(M if per_row else 1)).astype(np.float32)
+    sb = rng.uniform(1e-3, 2e-3, size=1).astype(np.float32)
+    out, acc = ops.gemm_i8(to_operand(a, bits, kp).to(gpu), to_operand(b, bits, kp).to(gpu), K, bits,
+                           torch.from_numpy(sa).to(gpu), torch.from_numpy(sb).to(gpu), post_scale=1 / 16,
+                           return_acc=True)
+    acc_ref = orc.int_gemm_nt(a, b)
+    assert np.array_equal(acc.cpu().numpy(), acc_ref)
+    ref = ((acc_ref.astype(np.float32) * sa.reshape(-1, 1)).astype(np.float32) * sb[0]).astype(np.float32) / np.float32(16)
+    assert np.array_equal(out.cpu().numpy(), ref.astype(np.float32))
+
+
+def test_gemm_i8_extreme_codes(gpu):
+    """All operands at +-qmax: the largest accumulators the path can produce."""
+    from hot_amd import ops
+    for bits, K in ((4, 11008), (8, 7092)):
+        qm = 2 ** (bits - 1) - 1
+        a = np.full((64, K), qm, dtype=np.int8)
+        b = np.full((96, K), -qm, dtype=np.int8)
+        kp = ops.kpad(K)
+        one = torch.ones(1, device=gpu)
+        _, acc = ops.gemm_i8(to_operand(a, bits, kp).to(gpu), to_operand(b, bits, kp).to(gpu), K, bits, one, one,
+                             return_acc=True)
+        assert torch.all(acc == -qm * qm * K)
+
+
+def test_gemm_i8_bf16_out(gpu):
+    from hot_amd import ops
+    a, b = rand_codes(100, 256, 8, 5), rand_codes(60, 256, 8, 6)
+    one = torch.ones(1, device=gpu)
+    out = ops.gemm_i8(torch.from_numpy(a).to(gpu), torch.from_numpy(b).to(gpu), 256, 8, one, one,
+                      out_dtype=torch.bfloat16)
+    ref = torch.from_numpy(orc.int_gemm_nt(a, b).astype(np.float32)).to(torch.bfloat16)
+    assert torch.equal(out.cpu(), ref)
