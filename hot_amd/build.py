@@ -21,6 +21,8 @@ FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # the column-wise kernels hold a whole token block in registers: their loops must unroll fully
+    "-mllvm", "-pragma-unroll-threshold=1000000",
 ]
 
 

@@ -202,7 +202,7 @@ __global__ void __launch_bounds__(256) colwise_finalize_kernel(const ColArgs a, 
 
 // ---- pass 2: transform again, quantise, transpose through LDS, store --------
 
-template <typename T, int N>
+template <typename T, int N, int ROUND, bool SAWB>
 __global__ void __launch_bounds__(COL_THREADS) colwise_quant_kernel(const ColArgs a) {
   constexpr int CPL = cpl_of<N>::value;
   constexpr int CG = 64 * CPL;  // channels per workgroup
@@ -246,17 +246,23 @@ __global__ void __launch_bounds__(COL_THREADS) colwise_quant_kernel(const ColArg
     for (int i = 0; i < N; ++i) {
       const int sl = a.slot[i];
       if (sl >= 0) {
+        float u[4];
+        if constexpr (ROUND == HOT_ROUND_STOCH) {
+          // element index of coefficient (k, c) is k * C + c; c0 is a multiple of CPL, so the
+          // lane's channels share one (CPL = 4) or half of one (CPL = 2) counter value
+          const uint64_t e = (uint64_t)(blk * a.r + sl) * (uint64_t)a.C + (uint64_t)c0;
+          sr_uniform4(e >> 2, a.seed, a.stream, u);
+        }
 #pragma unroll
         for (int c = 0; c < CPL; ++c) {
           float v = x[i][c];
-          if (a.mode == HOT_SCALE_SAWB) v = fminf(fmaxf(v, -clip), clip);
+          if constexpr (SAWB) v = fminf(fmaxf(v, -clip), clip);
           const float y = v / d[c];
           int q;
-          if (a.rounding == HOT_ROUND_NEAREST) {
+          if constexpr (ROUND == HOT_ROUND_NEAREST) {
             q = q_nearest(y);
           } else {
-            const uint64_t e = (uint64_t)(c0 + c) * (uint64_t)a.Kout + (uint64_t)(blk * a.r + sl);
-            q = q_stoch(y, sr_uniform1(e, a.seed, a.stream));
+            q = q_stoch(y, CPL == 4 ? u[c] : ((c0 & 2) ? u[2 + c] : u[c]));
           }
           q = clampi(q, -qmax, qmax);
           lds[(lane * CPL + c) * pitch + kl0 + sl] = (uint8_t)(q & 0xFF);
@@ -326,7 +332,13 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
                      a.mode == HOT_SCALE_ROW ? a.colmax : (float*)nullptr, a.C);
   hipLaunchKernelGGL((colwise_stats_kernel<T, N>), grid, block, 0, st, a);
   hipLaunchKernelGGL(colwise_finalize_kernel, dim3(1), dim3(256), 0, st, a, gx * gy);
-  hipLaunchKernelGGL((colwise_quant_kernel<T, N>), grid, block, lds, st, a);
+  if (a.rounding == HOT_ROUND_STOCH) {
+    if (a.mode == HOT_SCALE_SAWB) hipLaunchKernelGGL((colwise_quant_kernel<T, N, 1, true>), grid, block, lds, st, a);
+    else hipLaunchKernelGGL((colwise_quant_kernel<T, N, 1, false>), grid, block, lds, st, a);
+  } else {
+    if (a.mode == HOT_SCALE_SAWB) hipLaunchKernelGGL((colwise_quant_kernel<T, N, 0, true>), grid, block, lds, st, a);
+    else hipLaunchKernelGGL((colwise_quant_kernel<T, N, 0, false>), grid, block, lds, st, a);
+  }
   return check_launch("colwise_quant_kernel");
 }
 

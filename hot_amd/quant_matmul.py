@@ -1,0 +1,173 @@
+"""FLinearQ / HQ_Linear on the native gfx950 path.
+
+Same class names, argument order and attributes as the reference's
+utils/quant_matmul.py:169-422, so that
+``replace_layers(model, nn.Linear, HQ_Linear)`` (utils/utils.py:53-74) works
+unchanged.  Forward stays full precision (:173-175); ``setup_context`` writes
+the INT8 Hadamard-compressed activation buffer (:178-212) with the native
+kernel and ``backward`` (:215-348, scheme gih_gwlr) calls the fused native op.
+There is no eager fallback: on a CPU tensor the native path raises.
+"""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import numpy as np
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+from torch import Tensor
+from torch.autograd.function import Function
+
+from . import args
+from . import ops
+from .hadamard_matmul import (Transform_Dict, biggest_power2_factor, hla_rows, paper_rows)
+
+TD = Transform_Dict()
+
+_QUANT_SCHEMES = {
+    # name in args.layer_quant_dict -> (rounding, scale mode)
+    "int_quantizer": (ops.ROUND_NEAREST, ops.SCALE_TENSOR),
+    "stoch_quantizer": (ops.ROUND_STOCH, ops.SCALE_TENSOR),
+    "norm_quantizer": (ops.ROUND_STOCH, ops.SCALE_ROW),
+    "sawb_quantizer": (ops.ROUND_NEAREST, ops.SCALE_SAWB),
+}
+_FLAG_SCHEMES = {"int": "int_quantizer", "stoch": "stoch_quantizer", "nq": "norm_quantizer",
+                 "sawb": "sawb_quantizer"}
+
+
+def _scheme(flag: str, what: str, allowed) -> Tuple[int, int]:
+    if flag not in allowed:
+        raise NotImplementedError("%s rounding scheme %r is not implemented on the native path (use one of %s)"
+                                  % (what, flag, sorted(allowed)))
+    return _QUANT_SCHEMES[_FLAG_SCHEMES[flag]]
+
+
+def token_rule(tokens: int):
+    """(n, rows) of the low-rank projection for a token count under args.hla_rule."""
+    if args.hla_rule == "paper":
+        if tokens % 16:
+            return 1, np.array([0])
+        return paper_rows(16, 8)
+    n, rows = hla_rows(tokens, args.vectorPercentile)
+    if n > args.hla_max_block:
+        n, rows = hla_rows(args.hla_max_block, args.vectorPercentile)
+    return n, rows
+
+
+def options_for(tokens: int, layer_name: str = " ") -> ops.HotOptions:
+    """args.* -> HotOptions, following the branch structure of FLinearQ."""
+    if args.transform_scheme != "gih_gwlr":
+        raise NotImplementedError("transform scheme %r: only gih_gwlr runs natively" % args.transform_scheme)
+    if not (args.TransformGogi and args.TransformWgt and args.TransformGogw and args.TransformInput):
+        raise NotImplementedError("the native path needs all four Transform* flags on")
+    n, rows = token_rule(tokens)
+    gx_bits, gw_bits = args.GogiQuantBit, args.GogwQuantBit
+    if args.quantAuto and len(args.layer_quant_dict) > 0:
+        # utils/quant_matmul.py:244-245 and :307-308 (the g_W branch reads GogiQuantBit there)
+        gx_round, gx_scale = _QUANT_SCHEMES[args.layer_quant_dict[layer_name + "_gx"]]
+        gw_round, gw_scale = _QUANT_SCHEMES[args.layer_quant_dict[layer_name + "_gw"]]
+        gw_bits = args.GogiQuantBit
+    else:
+        gx_round, gx_scale = _scheme(args.quantBWDGogi, "GradHo", ("int", "stoch", "nq"))
+        gw_round, gw_scale = _scheme(args.quantBWDGogw, "GradHb", ("int", "stoch", "nq"))
+    w_round, w_scale = _scheme(args.quantBWDWgt, "Weight", ("int", "stoch", "sawb"))
+    act_round, act_scale = _scheme(args.quantBWDAct, "Activation", ("int", "stoch", "sawb"))
+    return ops.HotOptions(
+        n_o=16, hla_n=int(n), hla_rows=tuple(int(v) for v in rows),
+        gx_bits=gx_bits, w_bits=args.weightQuantBit, gw_bits=gw_bits, act_bits=args.actQuantBit,
+        gx_round=gx_round, w_round=w_round, gw_round=gw_round, act_round=act_round,
+        gx_scale=gx_scale, w_scale=w_scale, gw_scale=gw_scale, act_scale=act_scale,
+        seed=(int(args.sr_seed) << 20) + int(args.sr_step))
+
+
+class FLinearQ(Function):
+    """torch.autograd.Function with the reference's forward / setup_context /
+    backward triple (utils/quant_matmul.py:169-348)."""
+
+    @staticmethod
+    def forward(x, w, h_out, h_bs, name):
+        return F.linear(x, w)
+
+    @staticmethod
+    def setup_context(ctx, inputs, output):
+        x, w, _h_out, _h_bs, name = inputs
+        ctx.name = name
+        ctx.x_shape = tuple(x.shape)
+        if x.dim() == 3 and args.batched_mode == "per_sample":
+            tokens = x.shape[1]
+            opt = options_for(tokens, name)
+            bufs = [ops.abc_forward(x[b].contiguous(), opt) for b in range(x.shape[0])]
+            xq = torch.stack([b[0] for b in bufs])
+            sx = torch.cat([b[1] for b in bufs])
+        else:
+            x2 = x.reshape(-1, x.shape[-1]).contiguous()
+            opt = options_for(x2.shape[0], name)
+            xq, sx = ops.abc_forward(x2, opt)
+        ctx.opt = opt
+        args.sr_step += 1
+        ctx.save_for_backward(xq, w, sx)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        xq, w, sx = ctx.saved_tensors
+        opt = ctx.opt
+        go = grad_output
+        wc = w.contiguous()
+        if go.dtype != wc.dtype:
+            go = go.to(wc.dtype)
+        if go.dim() == 3 and args.batched_mode == "per_sample":
+            gxs, gw = [], None
+            for b in range(go.shape[0]):
+                gx_b, gw_b = ops.linear_backward(go[b].contiguous(), wc, xq[b], sx[b:b + 1], opt)
+                gxs.append(gx_b)
+                gw = gw_b.float() if gw is None else gw + gw_b.float()
+            grad_input = torch.stack(gxs)
+            grad_w = gw.to(wc.dtype)
+        else:
+            go2 = go.reshape(-1, go.shape[-1]).contiguous()
+            gx, grad_w = ops.linear_backward(go2, wc, xq, sx, opt)
+            grad_input = gx.reshape(ctx.x_shape)
+        return grad_input, grad_w, None, None, None
+
+
+class HQ_Linear(nn.Linear):
+    """nn.Linear whose backward runs the HOT path (utils/quant_matmul.py:350-422).
+
+    ``hadamard_out`` (H_16 for the out-features) and ``hadamard_bs`` (the
+    low-rank rows P for the token count) are kept as attributes for
+    compatibility; they are non-persistent buffers because P depends on the
+    token count of the batch at hand (the reference deletes them from
+    checkpoints for that reason, ViT_main.py:302-304)."""
+
+    def __init__(self, in_features, out_features, bias=True) -> None:
+        super().__init__(in_features, out_features, bias)
+        self.register_buffer("hadamard_out", torch.tensor(TD.get_or_register("hadamard", self.out_features),
+                                                          dtype=self.weight.dtype), persistent=False)
+        self.register_buffer("hadamard_bs", torch.ones((1, 1), dtype=self.weight.dtype), persistent=False)
+        self._bs_tokens = None
+        self.layer_name = " "
+
+    def _refresh_bs(self, tokens: int) -> None:
+        if self._bs_tokens == tokens:
+            return
+        n, rows = token_rule(tokens)
+        # P = rows of H_n; small (at most 64 x 64) because of args.hla_max_block
+        idx = torch.as_tensor(np.asarray(rows), dtype=torch.long)
+        i = idx[:, None] & torch.arange(n)[None, :]
+        par = torch.zeros_like(i)
+        while bool(i.any()):
+            par ^= i & 1
+            i >>= 1
+        self.hadamard_bs = (1 - 2 * par).to(self.weight.dtype).to(self.weight.device)
+        self._bs_tokens = tokens
+
+    def forward(self, input: Tensor) -> Tensor:
+        if input.dim() == 3 and args.batched_mode == "per_sample":
+            self._refresh_bs(input.shape[1])
+        else:
+            self._refresh_bs(input.numel() // input.shape[-1])
+        output = FLinearQ.apply(input, self.weight, self.hadamard_out, self.hadamard_bs, self.layer_name)
+        if self.bias is not None:
+            output = output + self.bias.to(output.device)
+        return output

@@ -108,7 +108,8 @@ HOT_API int hot_hq_rowwise(const void* in, int dtype, int64_t M, int64_t K, int 
  *               bytes beyond the logical row up to ld_out are written as zero
  *   scales_out  [1] (TENSOR, SAWB) or [C] (ROW)
  *   workspace   device, >= hot_colwise_workspace_bytes(C)
- * The stochastic-rounding element index of coefficient (c, k) is c*Kout + k.
+ * The stochastic-rounding element index of coefficient k of channel c is
+ * k*C + c (row-major position in the untransposed [Kout, C] matrix).
  */
 HOT_API int hot_hla_tokenwise(const void* in, int dtype, int64_t R, int64_t C, int n,
                       const int32_t* rows, int r, int bits, int rounding, uint64_t seed,

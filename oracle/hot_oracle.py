@@ -397,6 +397,14 @@ def abc_forward(x: np.ndarray, cfg: HotConfig):
     return quant(xp, cfg.act_bits, cfg.act_scale, cfg.act_round, cfg.seed, STREAM_ACT)
 
 
+def _untransposed_index(shape) -> np.ndarray:
+    """RNG element index of entry (c, k) of a [C, K] matrix that is the
+    transpose of a row-major [K, C] one: the kernels number the coefficients of
+    the column-wise transforms by their position k * C + c before the transpose."""
+    C, K = shape
+    return (np.arange(K, dtype=np.int64)[None, :] * C + np.arange(C, dtype=np.int64)[:, None])
+
+
 @dataclass
 class BackwardTrace:
     qG: np.ndarray = None
@@ -432,7 +440,8 @@ def linear_backward(g_y: np.ndarray, w: np.ndarray, xq: np.ndarray, sx: np.ndarr
     tr.g_x = (((tr.acc_x.astype(F32) * sg).astype(F32) * tr.sW[0]).astype(F32) / F32(cfg.n_o)).astype(F32)
     # :301 (P g_y)^T ; :307-320 quantise
     GpT = np.ascontiguousarray(fwht_blocks_first(g_y, cfg.hla_n, np.asarray(cfg.hla_rows)).T)
-    tr.qGp, tr.sGp = quant(GpT, cfg.gw_bits, cfg.gw_scale, cfg.gw_round, cfg.seed, STREAM_GW)
+    tr.qGp, tr.sGp = quant(GpT, cfg.gw_bits, cfg.gw_scale, cfg.gw_round, cfg.seed, STREAM_GW,
+                           index=_untransposed_index(GpT.shape))
     # :322-324, :344
     tr.acc_w = int_gemm_nt(tr.qGp, np.asarray(xq).T)
     sgw = tr.sGp.reshape(-1, 1) if cfg.gw_scale == SCALE_ROW else tr.sGp.reshape(1, 1)

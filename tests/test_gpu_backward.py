@@ -1,0 +1,266 @@
+"""Parity of the fused path (hot_abc_forward + hot_linear_backward through the
+C ABI, and the Python drop-in surface above it) with the CPU oracle and with
+the op-for-op port of the reference's fake-quant path.
+
+Bars: integer stages bit-exact under round-to-nearest (and, because both sides
+share the counter-based generator, under stochastic rounding too); fp32 g_x /
+g_W equal to the canonical oracle and within 1e-3 relative Frobenius error of
+the fake-quant port."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import fakequant_port as fq
+from oracle import hot_oracle as orc
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-3   # north-star tolerance on final fp32 g_x / g_W
+
+
+def rel(a, b):
+    a = np.asarray(a, dtype=np.float64)
+    b = np.asarray(b, dtype=np.float64)
+    return np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-300)
+
+
+def make_case(L, O, I, seed=0, dtype=torch.float32, outliers=True):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(L, I, generator=g)
+    w = (torch.rand(O, I, generator=g) * 2 - 1) / I ** 0.5
+    gy = torch.randn(L, O, generator=g) * 1e-3
+    if outliers:
+        gy = torch.where(torch.rand(L, O, generator=g) < 0.01, gy * 50, gy)
+    return x.to(dtype), w.to(dtype), gy.to(dtype)
+
+
+def both_configs(L, rule="python", **kw):
+    from hot_amd import ops
+    ocfg = orc.HotConfig.python_rule(L, **kw) if rule == "python" else orc.HotConfig.paper(16, 8, **kw)
+    if ocfg.hla_n > 64:
+        n, rows = orc.hla_rows(64)
+        ocfg.hla_n, ocfg.hla_rows = n, tuple(int(v) for v in rows)
+    opt = ops.HotOptions(n_o=ocfg.n_o, hla_n=ocfg.hla_n, hla_rows=ocfg.hla_rows, gx_bits=ocfg.gx_bits,
+                         w_bits=ocfg.w_bits, gw_bits=ocfg.gw_bits, act_bits=ocfg.act_bits,
+                         gx_round=ocfg.gx_round, w_round=ocfg.w_round, gw_round=ocfg.gw_round,
+                         act_round=ocfg.act_round, gx_scale=ocfg.gx_scale, w_scale=ocfg.w_scale,
+                         gw_scale=ocfg.gw_scale, act_scale=ocfg.act_scale, seed=ocfg.seed)
+    return ocfg, opt
+
+
+def run_both(x, w, gy, ocfg, opt, gpu):
+    from hot_amd import ops
+    xq, sx = ops.abc_forward(x.to(gpu), opt)
+    gx, gw = ops.linear_backward(gy.to(gpu), w.to(gpu), xq, sx, opt)
+    xq_ref, sx_ref = orc.abc_forward(x.float().numpy(), ocfg)
+    tr = orc.linear_backward(gy.float().numpy(), w.float().numpy(), xq_ref, sx_ref, ocfg)
+    lp = xq_ref.shape[0]
+    got_xq = xq.cpu().numpy()
+    assert np.array_equal(got_xq[:, :lp], xq_ref.T) and not got_xq[:, lp:].any()
+    assert np.array_equal(sx.cpu().numpy(), sx_ref)
+    return gx, gw, tr
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(448, 192, 160), (64 * 5, 208, 72), (128, 2304, 768)])
+@pytest.mark.parametrize("variant", [
+    dict(),                                                                       # INT4 / INT8, nearest, per tensor
+    dict(gx_bits=8, w_bits=8),
+    dict(gx_scale=orc.SCALE_ROW, gw_scale=orc.SCALE_ROW),                         # per token / per channel
+    dict(gx_round=orc.ROUND_STOCH, gw_round=orc.ROUND_STOCH, seed=99),            # stoch_quantizer
+    dict(gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW, gw_round=orc.ROUND_STOCH,
+         gw_scale=orc.SCALE_ROW, seed=7),                                         # norm_quantizer
+    dict(w_scale=orc.SCALE_SAWB, act_scale=orc.SCALE_SAWB),                       # canonical W / x recipe
+    dict(gw_bits=4, act_bits=4),
+])
+def test_backward_matches_oracle(gpu, dtype, shape, variant):
+    L, O, I = shape
+    x, w, gy = make_case(L, O, I, seed=L + O, dtype=dtype)
+    ocfg, opt = both_configs(L, **variant)
+    gx, gw, tr = run_both(x, w, gy, ocfg, opt, gpu)
+    if dtype == torch.float32:
+        # same IEEE operations in the same order on both sides
+        assert np.array_equal(gx.cpu().numpy(), tr.g_x)
+        assert np.array_equal(gw.cpu().numpy(), tr.g_w)
+    else:
+        assert torch.equal(gx.cpu(), torch.from_numpy(tr.g_x).to(dtype))
+        assert torch.equal(gw.cpu(), torch.from_numpy(tr.g_w).to(dtype))
+
+
+def test_backward_paper_rule(gpu):
+    L, O, I = 512, 256, 128
+    x, w, gy = make_case(L, O, I, seed=1)
+    ocfg, opt = both_configs(L, rule="paper")
+    assert (opt.hla_n, opt.hla_r) == (16, 8)
+    gx, gw, tr = run_both(x, w, gy, ocfg, opt, gpu)
+    assert np.array_equal(gx.cpu().numpy(), tr.g_x) and np.array_equal(gw.cpu().numpy(), tr.g_w)
+
+
+def test_backward_no_hla_for_odd_token_counts(gpu):
+    """L = 49 (the reference harness' token count) and L = 197: n = 1, r = 1."""
+    for L in (49, 197):
+        x, w, gy = make_case(L, 128, 64, seed=L)
+        ocfg, opt = both_configs(L)
+        assert opt.hla_n == 1
+        gx, gw, tr = run_both(x, w, gy, ocfg, opt, gpu)
+        assert np.array_equal(gx.cpu().numpy(), tr.g_x) and np.array_equal(gw.cpu().numpy(), tr.g_w)
+
+
+def test_backward_against_fakequant_port(gpu):
+    """The reference's own evaluation order (dense matmul transforms): final
+    fp32 gradients within 1e-3 relative Frobenius error."""
+    L, O, I = 1344, 768, 384          # 1344 = 64 * 21: the python rule gives n = 64, r = 36
+    x, w, gy = fq.config1_inputs(L, O, I, seed=0)
+    ocfg, opt = both_configs(L)
+    gx, gw, _ = run_both(x, w, gy, ocfg, opt, gpu)
+    h_out, h_bs = fq.matrices(L, O)
+    assert h_bs.shape == (len(ocfg.hla_rows), ocfg.hla_n) == (36, 64)
+    xq, sx = fq.setup_context(x, h_bs, fq.PortConfig())
+    gi_ref, gw_ref = fq.backward(gy, w, xq, sx, h_out, h_bs, fq.PortConfig())
+    assert rel(gx.cpu().numpy(), gi_ref.numpy()) < REL_TOL
+    assert rel(gw.cpu().numpy(), gw_ref.numpy()) < REL_TOL
+
+
+def test_vit_fc1_full_size(gpu):
+    """BASELINE configuration 1 at full size (L = 12608, O = 3072, I = 768):
+    bit-exact against the canonical oracle, 1e-3 against the fake-quant port."""
+    L, O, I = 12608, 3072, 768
+    x, w, gy = fq.config1_inputs(L, O, I, seed=0)
+    ocfg, opt = both_configs(L)
+    assert (opt.hla_n, opt.hla_r) == (64, 36)
+    gx, gw, tr = run_both(x, w, gy, ocfg, opt, gpu)
+    assert np.array_equal(gx.cpu().numpy(), tr.g_x)
+    assert np.array_equal(gw.cpu().numpy(), tr.g_w)
+    h_out, h_bs = fq.matrices(L, O)
+    xq, sx = fq.setup_context(x, h_bs, fq.PortConfig())
+    gi_ref, gw_ref = fq.backward(gy, w, xq, sx, h_out, h_bs, fq.PortConfig())
+    assert rel(gx.cpu().numpy(), gi_ref.numpy()) < REL_TOL
+    assert rel(gw.cpu().numpy(), gw_ref.numpy()) < REL_TOL
+
+
+@pytest.mark.parametrize("shape", [(8192, 11008, 4096), (8192, 4096, 11008)])
+def test_llama_shapes_properties(gpu, shape):
+    """Llama-7B MLP shapes, bf16, too large for the CPU oracle: checked through
+    size-independent properties.
+      * scaling g_y by a power of two scales both gradients by exactly that
+        factor (absmax quantisation commutes with it);
+      * INT8 everywhere with all coefficients kept approximates the bf16 matmul."""
+    from hot_amd import ops
+    L, O, I = shape
+    g = torch.Generator(device="cpu").manual_seed(1)
+    # unit-variance g_y keeps every step size far above the 1e-11 guard added to it,
+    # which is the only term that does not scale
+    gy = torch.randn(L, O, generator=g).to(torch.bfloat16).to(gpu)
+    w = ((torch.rand(O, I, generator=g) * 2 - 1) / I ** 0.5).to(torch.bfloat16).to(gpu)
+    x = torch.randn(L, I, generator=g).to(torch.bfloat16).to(gpu)
+    _, opt = both_configs(L, rule="paper")
+    xq, sx = ops.abc_forward(x, opt)
+    gx, gw = ops.linear_backward(gy, w, xq, sx, opt, out_dtype=torch.float32)
+    gx4, gw4 = ops.linear_backward(gy * 4, w, xq, sx, opt, out_dtype=torch.float32)
+    assert torch.equal(gx4, gx * 4) and torch.equal(gw4, gw * 4)
+    full = ops.HotOptions(hla_n=16, hla_rows=tuple(range(16)), gx_bits=8, w_bits=8, gw_bits=8, act_bits=8)
+    xq8, sx8 = ops.abc_forward(x, full)
+    gx8, gw8 = ops.linear_backward(gy, w, xq8, sx8, full, out_dtype=torch.float32)
+    ref_gx = gy.float() @ w.float()
+    ref_gw = gy.float().T @ x.float()
+    assert float((gx8 - ref_gx).norm() / ref_gx.norm()) < 0.03
+    assert float((gw8 - ref_gw).norm() / ref_gw.norm()) < 0.03
+
+
+def test_hlq_backward_op_surface(gpu):
+    """HLQ_backward.backward(Go, W, X, 0, 0, 16, per_token) -> (gx, gw, 4 floats)."""
+    from hot_amd import HLQ_backward
+    L, O, I = 192, 3072, 768
+    rng = np.random.default_rng(2023)
+    X = torch.tensor(rng.lognormal(1.0, 0.1, (L, I)), dtype=torch.float32)
+    Go = torch.tensor(rng.lognormal(1.0, 0.1, (L, O)), dtype=torch.float32)
+    W = torch.tensor(rng.lognormal(1.0, 0.1, (O, I)), dtype=torch.float32)
+    for per_token in (True, False):
+        gx, gw, times = HLQ_backward.backward(Go.to(gpu), W.to(gpu), X.to(gpu), 0, 0, 16, per_token)
+        assert gx.shape == (L, I) and gw.shape == (O, I) and gx.dtype == Go.dtype
+        assert isinstance(times, list) and len(times) == 4 and all(isinstance(t, float) and t > 0 for t in times)
+        opt = HLQ_backward.options(L, 16, per_token)
+        ocfg = orc.HotConfig(n_o=16, hla_n=opt.hla_n, hla_rows=opt.hla_rows, gx_round=orc.ROUND_STOCH,
+                             gx_scale=orc.SCALE_ROW if per_token else orc.SCALE_TENSOR, seed=HLQ_backward.seed)
+        xq_ref, sx_ref = orc.abc_forward(X.numpy(), ocfg)
+        tr = orc.linear_backward(Go.numpy(), W.numpy(), xq_ref, sx_ref, ocfg)
+        assert np.array_equal(gx.cpu().numpy(), tr.g_x) and np.array_equal(gw.cpu().numpy(), tr.g_w)
+    with pytest.raises(RuntimeError, match="Go must be contiguous!"):
+        HLQ_backward.backward(Go.to(gpu).t().contiguous().t(), W.to(gpu), X.to(gpu), 0, 0, 16, True)
+    with pytest.raises(RuntimeError, match="X must be 2D!"):
+        HLQ_backward.backward(Go.to(gpu), W.to(gpu), X.to(gpu)[None], 0, 0, 16, True)
+
+
+@pytest.fixture
+def fresh_args():
+    from hot_amd import args
+    saved = {k: getattr(args, k) for k in dir(args) if not k.startswith("_")}
+    yield args
+    for k, v in saved.items():
+        setattr(args, k, v)
+
+
+def test_hq_linear_training_step(gpu, fresh_args):
+    """HQ_Linear forward (full precision) + backward (HOT) through autograd."""
+    from hot_amd.quant_matmul import HQ_Linear
+    L, I, O = 256, 96, 128
+    torch.manual_seed(0)
+    lin = HQ_Linear(I, O).to(gpu)
+    x = torch.randn(L, I, device=gpu, requires_grad=True)
+    y = lin(x)
+    assert torch.allclose(y, torch.nn.functional.linear(x, lin.weight, lin.bias))
+    gy = torch.randn(L, O, device=gpu) * 1e-3
+    y.backward(gy)
+    ocfg, _ = both_configs(L)
+    xq_ref, sx_ref = orc.abc_forward(x.detach().cpu().numpy(), ocfg)
+    tr = orc.linear_backward(gy.cpu().numpy(), lin.weight.detach().cpu().numpy(), xq_ref, sx_ref, ocfg)
+    assert np.array_equal(x.grad.cpu().numpy(), tr.g_x)
+    assert np.array_equal(lin.weight.grad.cpu().numpy(), tr.g_w)
+    assert torch.allclose(lin.bias.grad, gy.sum(0), rtol=1e-5, atol=1e-8)
+    assert lin.hadamard_bs.shape == (36, 128 if L % 128 == 0 and fresh_args.hla_max_block >= 128 else 64)
+
+
+@pytest.mark.parametrize("mode", ["per_sample", "flatten"])
+def test_hq_linear_3d_input(gpu, fresh_args, mode):
+    """[B, L, C] activations: per-sample steps as in the reference (vmap over
+    the batch, utils/quant_matmul.py:118-122) or flattened tokens."""
+    from hot_amd.quant_matmul import HQ_Linear
+    fresh_args.batched_mode = mode
+    B, L, I, O = 3, 64, 48, 80
+    torch.manual_seed(1)
+    lin = HQ_Linear(I, O, bias=False).to(gpu)
+    x = torch.randn(B, L, I, device=gpu, requires_grad=True)
+    gy = torch.randn(B, L, O, device=gpu) * 1e-3
+    lin(x).backward(gy)
+    wn = lin.weight.detach().cpu().numpy()
+    if mode == "per_sample":
+        ocfg, _ = both_configs(L)
+        gxs, gw = [], 0
+        for b in range(B):
+            xq_ref, sx_ref = orc.abc_forward(x[b].detach().cpu().numpy(), ocfg)
+            tr = orc.linear_backward(gy[b].cpu().numpy(), wn, xq_ref, sx_ref, ocfg)
+            gxs.append(tr.g_x)
+            gw = gw + tr.g_w
+        assert np.array_equal(x.grad.cpu().numpy(), np.stack(gxs))
+        assert rel(lin.weight.grad.cpu().numpy(), gw) < 1e-6
+    else:
+        ocfg, _ = both_configs(B * L)
+        xq_ref, sx_ref = orc.abc_forward(x.detach().reshape(B * L, I).cpu().numpy(), ocfg)
+        tr = orc.linear_backward(gy.reshape(B * L, O).cpu().numpy(), wn, xq_ref, sx_ref, ocfg)
+        assert np.array_equal(x.grad.cpu().numpy().reshape(B * L, I), tr.g_x)
+        assert np.array_equal(lin.weight.grad.cpu().numpy(), tr.g_w)
+
+
+def test_backward_errors(gpu):
+    from hot_amd import ops
+    from hot_amd._lib import HotError
+    x, w, gy = make_case(128, 64, 32)
+    _, opt = both_configs(128)
+    xq, sx = ops.abc_forward(x.to(gpu), opt)
+    with pytest.raises(RuntimeError):
+        ops.linear_backward(gy.to(gpu), w.to(gpu)[:32].contiguous(), xq, sx, opt)        # O mismatch
+    bad = ops.HotOptions(hla_n=opt.hla_n, hla_rows=opt.hla_rows, gx_bits=4, w_bits=8)
+    with pytest.raises(HotError, match="must match"):
+        ops.linear_backward(gy.to(gpu), w.to(gpu), xq, sx, bad)
+    with pytest.raises(HotError):
+        ops.abc_forward(x.to(gpu)[:100].contiguous(), opt)                               # L % n

@@ -1,0 +1,343 @@
+"""Pins the CPU oracle.  The reference ships no tests, golden vectors or
+fixtures for this path, so every function is checked against what the
+mathematics fixes: closed forms, library routines (scipy.linalg.hadamard /
+block_diag), brute force on small sizes, hand-derived tables, published
+known-answer vectors (Philox, Random123) and statistical properties.  None of
+the checks re-types the oracle's own formula."""
+import itertools
+
+import numpy as np
+import pytest
+import scipy.linalg
+
+from oracle import hot_oracle as orc
+
+F32 = np.float32
+
+
+# ------------------------------------------------------------------ sizes
+
+def test_pow2_factor_bruteforce():
+    for size in range(1, 400):
+        best = max(d for d in range(1, size + 1) if size % d == 0 and (d & (d - 1)) == 0)
+        assert orc.pow2_factor(size) == best
+        assert orc.pow2_factor_max16(size) == (16 if best > 16 and size > 16 else best)
+
+
+def test_pow2_factor_table():
+    # sizes of the graded configurations
+    assert [orc.pow2_factor_max16(v) for v in (768, 2304, 3072, 4096, 11008)] == [16] * 5
+    assert orc.pow2_factor(12608) == 64 and orc.pow2_factor(8192) == 8192
+    assert orc.pow2_factor(197) == 1 and orc.pow2_factor(49) == 1 and orc.pow2_factor(25216) == 128
+    assert orc.pow2_factor_max16(16) == 16 and orc.pow2_factor_max16(8) == 8 and orc.pow2_factor_max16(12) == 4
+
+
+# --------------------------------------------------------------- matrices
+
+@pytest.mark.parametrize("n", [1, 2, 4, 8, 16, 32, 64, 128])
+def test_hadamard_is_sylvester(n):
+    H = orc.hadamard(n)
+    if n > 1:
+        assert np.array_equal(H, scipy.linalg.hadamard(n))
+    assert np.array_equal(H, H.T)
+    assert np.array_equal(H @ H.T, n * np.eye(n, dtype=np.int64))
+
+
+def test_hadamard_rejects_non_power_of_two():
+    for bad in (0, 3, 12, -4):
+        with pytest.raises(ValueError):
+            orc.hadamard(bad)
+
+
+@pytest.mark.parametrize("n", [1, 2, 4, 8, 16, 32, 64, 128, 256])
+def test_sequency_bruteforce(n):
+    H = scipy.linalg.hadamard(n) if n > 1 else np.array([[1]])
+    changes = np.array([(H[i, :-1] != H[i, 1:]).sum() for i in range(n)])
+    assert np.array_equal(orc.sequency_of_natural(n), changes)
+    assert sorted(changes) == list(range(n))          # unique: the sort is unambiguous
+    assert np.array_equal(orc.sequency_of_natural(n)[orc.natural_of_sequency(n)], np.arange(n))
+
+
+def test_kept_sequencies_hand_derived():
+    # derived by hand from the band rule: band i of width s keeps its first s-i
+    # entries when i is even and its last s-i entries when i is odd
+    assert list(orc.kept_sequencies(1)) == [0]
+    assert list(orc.kept_sequencies(2)) == [0]
+    assert list(orc.kept_sequencies(4)) == [0, 1, 3]
+    assert list(orc.kept_sequencies(8)) == [0, 1, 3]
+    assert list(orc.kept_sequencies(16)) == [0, 1, 2, 3, 5, 6, 7, 8, 9, 15]
+    k64 = list(orc.kept_sequencies(64))
+    assert k64 == (list(range(0, 8)) + list(range(9, 16)) + list(range(16, 22)) + list(range(27, 32))
+                   + list(range(32, 36)) + list(range(45, 48)) + list(range(48, 50)) + [63])
+    for n, r in ((32, 10), (64, 36), (128, 36), (256, 136), (2048, 528), (4096, 2080), (8192, 2080)):
+        assert len(orc.kept_sequencies(n)) == r
+
+
+@pytest.mark.parametrize("size", [16, 48, 64, 192, 12608 // 197 * 3])
+def test_make_wht_bruteforce(size):
+    """P = rows of the Sylvester matrix sorted by counted sign changes, then the
+    hand-derived index set."""
+    n = orc.pow2_factor(size)
+    H = scipy.linalg.hadamard(n) if n > 1 else np.array([[1]])
+    order = sorted(range(n), key=lambda i: int((H[i, :-1] != H[i, 1:]).sum()))
+    want = H[order][orc.kept_sequencies(n)]
+    P = orc.make_WHT(size)
+    assert np.array_equal(P, want)
+    r = P.shape[0]
+    assert np.array_equal(P @ P.T, n * np.eye(r, dtype=np.int64))
+
+
+def test_vit_and_llama_token_rules():
+    n, rows = orc.hla_rows(12608)
+    assert (n, len(rows)) == (64, 36)
+    n, rows = orc.hla_rows(8192)
+    assert (n, len(rows)) == (8192, 2080)
+    n, rows = orc.hla_rows(197)
+    assert (n, list(rows)) == (1, [0])
+    n, rows = orc.paper_rows(16, 8)
+    H = scipy.linalg.hadamard(16)
+    assert sorted(int((H[i, :-1] != H[i, 1:]).sum()) for i in rows) == list(range(8))
+
+
+# -------------------------------------------------------------- transforms
+
+@pytest.mark.parametrize("n", [2, 16, 32, 64])
+def test_fwht_blocks_last_vs_blockdiag(n):
+    rng = np.random.default_rng(n)
+    a = rng.integers(-100, 100, size=(7, 3 * n)).astype(F32)      # exact in fp32
+    bd = scipy.linalg.block_diag(*[orc.hadamard(n)] * 3).astype(F32)
+    assert np.array_equal(orc.fwht_blocks_last(a, n), a @ bd)
+
+
+@pytest.mark.parametrize("n", [1, 4, 16, 64])
+def test_fwht_blocks_first_vs_blockdiag(n):
+    rng = np.random.default_rng(n)
+    a = rng.integers(-100, 100, size=(3 * n, 5)).astype(F32)
+    bd = scipy.linalg.block_diag(*[orc.hadamard(n)] * 3).astype(F32)
+    assert np.array_equal(orc.fwht_blocks_first(a, n), bd @ a)
+    _, rows = orc.hla_rows(n) if n > 1 else (1, np.array([0]))
+    P = orc.hadamard(n)[rows].astype(F32)
+    bdp = scipy.linalg.block_diag(*[P] * 3)
+    assert np.array_equal(orc.fwht_blocks_first(a, n, rows), bdp @ a)
+
+
+def test_fwht_is_the_canonical_butterfly():
+    """Stage order h = 1, 2, 4, 8 with (x+y, x-y), evaluated by a scalar loop."""
+    rng = np.random.default_rng(0)
+    v = rng.standard_normal(16).astype(F32)
+    w = v.copy()
+    h = 1
+    while h < 16:
+        for j in range(16):
+            if (j // h) % 2 == 0:
+                x, y = w[j], w[j + h]
+                w[j], w[j + h] = F32(x + y), F32(x - y)
+        h *= 2
+    assert np.array_equal(orc.fwht_blocks_last(v[None, :], 16)[0], w)
+
+
+def test_transform_rejects_ragged():
+    with pytest.raises(ValueError):
+        orc.fwht_blocks_last(np.zeros((2, 40), F32), 16)
+    with pytest.raises(ValueError):
+        orc.fwht_blocks_first(np.zeros((40, 2), F32), 16)
+
+
+# ------------------------------------------------------------------ Philox
+
+def test_philox_known_answers():
+    """Random123 kat_vectors, philox4x32-10."""
+    kat = [
+        ((0, 0, 0, 0), (0, 0), (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
+        ((0xffffffff,) * 4, (0xffffffff, 0xffffffff), (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
+        ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
+         (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1)),
+    ]
+    for ctr, key, want in kat:
+        got = orc.philox4x32(*[[c] for c in ctr], key[0], key[1])
+        assert tuple(int(g[0]) for g in got) == want
+
+
+def test_sr_uniform_range_and_moments():
+    u = orc.sr_uniform(np.arange(1 << 16), seed=12345, stream=1)
+    assert u.dtype == F32 and u.min() >= 0.0 and u.max() < 1.0
+    assert abs(u.mean() - 0.5) < 0.005 and abs(u.var() - 1 / 12) < 0.003
+    hist = np.histogram(u, bins=16, range=(0, 1))[0]
+    assert np.all(np.abs(hist - 4096) < 5 * 64)
+    # different seeds / streams / indices give different draws
+    assert not np.array_equal(u, orc.sr_uniform(np.arange(1 << 16), seed=12346, stream=1))
+    assert not np.array_equal(u, orc.sr_uniform(np.arange(1 << 16), seed=12345, stream=2))
+    assert np.array_equal(u[4:8], orc.sr_uniform(np.arange(4, 8), seed=12345, stream=1))
+
+
+# --------------------------------------------------------------- quantisers
+
+def test_quant_nearest_ties_to_even():
+    # mx = 7, bits = 4 -> s = 1, fl32(1 + 1e-11) = 1 -> y = t exactly
+    t = np.array([[0.5, 1.5, 2.5, 3.5, -0.5, -1.5, -2.5, 6.5, 7.0, 0.49999997, 0.50000006]], F32)
+    q, s = orc.quant(t, 4, orc.SCALE_TENSOR)
+    assert s[0] == 1.0
+    assert q.tolist() == [[0, 2, 2, 4, 0, -2, -2, 6, 7, 0, 1]]
+    t8 = np.array([[127.0, 0.5, 1.5, -126.5, 63.5]], F32)
+    q, s = orc.quant(t8, 8, orc.SCALE_TENSOR)
+    assert s[0] == 1.0 and q.tolist() == [[127, 0, 2, -126, 64]]
+
+
+def test_quant_zero_tensor_and_max():
+    q, s = orc.quant(np.zeros((3, 8), F32), 4, orc.SCALE_TENSOR)
+    assert not q.any() and s[0] == 0
+    q, s = orc.quant(np.zeros((3, 8), F32), 8, orc.SCALE_ROW)
+    assert not q.any() and not s.any() and s.shape == (3,)
+    rng = np.random.default_rng(1)
+    for bits in (4, 8):
+        qm = 2 ** (bits - 1) - 1
+        t = rng.standard_normal((40, 64)).astype(F32) * F32(1e-3)
+        q, s = orc.quant(t, bits, orc.SCALE_TENSOR)
+        i = np.unravel_index(np.argmax(np.abs(t)), t.shape)
+        assert abs(int(q[i])) == qm and np.abs(q).max() == qm
+        assert s[0] == F32(np.abs(t).max()) / F32(qm)
+        # textbook absmax quantiser: reconstruction within half a step
+        assert np.all(np.abs(q.astype(np.float64) * float(s[0]) - t) <= 0.5 * float(s[0]) * (1 + 1e-5))
+        qr, sr = orc.quant(t, bits, orc.SCALE_ROW)
+        assert np.all(np.abs(qr).max(axis=1) == qm)
+        for r in (0, 17, 39):                      # rows are independent
+            q1, s1 = orc.quant(t[r:r + 1], bits, orc.SCALE_TENSOR)
+            assert np.array_equal(q1[0], qr[r]) and s1[0] == sr[r]
+
+
+def test_quant_stochastic_statistics():
+    rng = np.random.default_rng(2)
+    t = rng.standard_normal((16, 64)).astype(F32)
+    s, _ = orc.quant_scale(t, 4, orc.SCALE_TENSOR)
+    y = (t / (s + F32(1e-11))).astype(np.float64)
+    nseed = 600
+    acc = np.zeros_like(y)
+    acc2 = np.zeros_like(y)
+    for seed in range(nseed):
+        q, s2 = orc.quant(t, 4, orc.SCALE_TENSOR, orc.ROUND_STOCH, seed=seed, stream=0)
+        q = q.astype(np.float64)
+        assert np.all((q == np.floor(y)) | (q == np.ceil(y)))
+        assert np.abs(q).max() <= 7 and s2[0] == s
+        acc += q
+        acc2 += q * q
+    mean = acc / nseed
+    assert np.max(np.abs(mean - y)) < 0.11                       # 5 sigma of 0.5 / sqrt(600)
+    assert abs((mean - y).mean()) < 5 * 0.5 / np.sqrt(nseed * y.size)
+    p = y - np.floor(y)
+    var = acc2 / nseed - mean ** 2
+    assert abs(var.mean() - (p * (1 - p)).mean()) < 0.01          # Bernoulli variance
+
+
+def test_quant_sawb_closed_form():
+    rng = np.random.default_rng(3)
+    t = rng.standard_normal((64, 64)).astype(F32) * F32(0.02)
+    q, s = orc.quant(t, 4, orc.SCALE_SAWB)
+    clip = 12.1 * np.sqrt((t.astype(np.float64) ** 2).mean()) - 12.2 * np.abs(t.astype(np.float64)).mean()
+    assert abs(float(s[0]) - clip / 7) < 1e-7 * clip
+    # Gaussian data: clip = (12.1 - 12.2 sqrt(2/pi)) sigma ~ 2.37 sigma
+    assert 2.2 * 0.02 < clip < 2.55 * 0.02
+    assert np.abs(q).max() == 7
+    inside = np.abs(t) < clip * 0.99
+    assert np.all(np.abs(q[inside] * float(s[0]) - t[inside]) <= 0.5 * float(s[0]) * (1 + 1e-4))
+
+
+# ------------------------------------------------------------- wire format
+
+def test_int4_pack_all_pairs():
+    pairs = np.array(list(itertools.product(range(-7, 8), repeat=2)), dtype=np.int8)   # 225 pairs
+    assert pairs.shape == (225, 2)
+    packed = orc.pack_int4(pairs)
+    assert packed.shape == (225, 1)
+    for (lo, hi), byte in zip(pairs.tolist(), packed.view(np.uint8)[:, 0].tolist()):
+        assert byte == (((hi & 0xF) << 4) | (lo & 0xF))
+    assert np.array_equal(orc.unpack_int4(packed), pairs)
+    assert orc.pack_int4(np.array([[-1, 3]], np.int8)).view(np.uint8)[0, 0] == 0x3F
+    assert orc.pack_int4(np.array([[7, -7]], np.int8)).view(np.uint8)[0, 0] == 0x97
+    with pytest.raises(ValueError):
+        orc.pack_int4(np.zeros((1, 3), np.int8))
+
+
+def test_int_gemm_exact():
+    rng = np.random.default_rng(4)
+    a = rng.integers(-127, 128, size=(33, 700), dtype=np.int8)
+    b = rng.integers(-127, 128, size=(21, 700), dtype=np.int8)
+    assert np.array_equal(orc.int_gemm_nt(a, b), a.astype(np.int64) @ b.astype(np.int64).T)
+    full = np.full((4, 11008), 127, np.int8)
+    assert np.all(orc.int_gemm_nt(full, -full) == -127 * 127 * 11008)
+
+
+# ------------------------------------------------------- the composed path
+
+def _case(L=128, O=64, I=48, seed=0, outliers=False):
+    rng = np.random.default_rng(seed)
+    x = rng.standard_normal((L, I)).astype(F32)
+    w = (rng.uniform(-1, 1, (O, I)) / np.sqrt(I)).astype(F32)
+    gy = (rng.standard_normal((L, O)) * 1e-3).astype(F32)
+    if outliers:
+        gy = np.where(rng.uniform(size=gy.shape) < 0.01, gy * 50, gy).astype(F32)
+    return x, w, gy
+
+
+def _rel(a, b):
+    return np.linalg.norm(a.astype(np.float64) - b) / np.linalg.norm(b)
+
+
+def test_transforms_alone_are_exact():
+    """H_n H_n^T = n I: without quantisation the path reproduces g_y W and, with
+    all rows kept, g_y^T x (integer-valued inputs make fp32 exact)."""
+    rng = np.random.default_rng(5)
+    gy = rng.integers(-8, 8, (64, 32)).astype(F32)
+    w = rng.integers(-8, 8, (32, 24)).astype(F32)
+    x = rng.integers(-8, 8, (64, 24)).astype(F32)
+    G, Wh = orc.fwht_blocks_last(gy, 16), orc.fwht_blocks_first(w, 16)
+    assert np.array_equal(G @ Wh / 16, gy @ w)
+    Gp = orc.fwht_blocks_first(gy, 16, np.arange(16))
+    Xp = orc.fwht_blocks_first(x, 16, np.arange(16))
+    assert np.array_equal(Gp.T @ Xp / 16, gy.T @ x)
+
+
+def test_backward_int8_full_rank_is_close_to_fp():
+    x, w, gy = _case()
+    cfg = orc.HotConfig(hla_n=16, hla_rows=tuple(range(16)), gx_bits=8, w_bits=8, gw_bits=8, act_bits=8)
+    xq, sx = orc.abc_forward(x, cfg)
+    tr = orc.linear_backward(gy, w, xq, sx, cfg)
+    assert _rel(tr.g_x, gy.astype(np.float64) @ w) < 0.02
+    assert _rel(tr.g_w, gy.astype(np.float64).T @ x) < 0.02
+    assert np.array_equal(tr.acc_x, tr.qG.astype(np.int64) @ tr.qW.astype(np.int64))
+    assert np.array_equal(tr.acc_w, tr.qGp.astype(np.int64) @ xq.astype(np.int64))
+    assert tr.g_x.shape == (128, 48) and tr.g_w.shape == (64, 48)
+
+
+def test_hadamard_spreads_outliers():
+    """INT8 g_x error with 1 % x50 outliers is lower (here about 3x) with the
+    Hadamard transform than when quantising g_y and W directly."""
+    x, w, gy = _case(L=256, O=128, I=64, seed=7, outliers=True)
+    cfg = orc.HotConfig.python_rule(256, gx_bits=8, w_bits=8)
+    xq, sx = orc.abc_forward(x, cfg)
+    tr = orc.linear_backward(gy, w, xq, sx, cfg)
+    exact = gy.astype(np.float64) @ w
+    qg, sg = orc.quant(gy, 8, orc.SCALE_TENSOR)
+    qw, sw = orc.quant(w.T.copy(), 8, orc.SCALE_TENSOR)
+    plain = orc.int_gemm_nt(qg, qw).astype(np.float64) * float(sg[0]) * float(sw[0])
+    assert _rel(tr.g_x, exact) < 0.6 * _rel(plain, exact)
+
+
+def test_backward_low_rank_is_a_projection():
+    """g_W of the low-rank path equals (P g_y)^T (P x) / n up to quantisation."""
+    x, w, gy = _case(L=128, seed=9)
+    cfg = orc.HotConfig.python_rule(128)
+    n, rows = orc.hla_rows(128)
+    assert cfg.hla_n == n == 128 and len(rows) == 36
+    cfg8 = orc.HotConfig(hla_n=n, hla_rows=tuple(rows), gw_bits=8, act_bits=8)
+    xq, sx = orc.abc_forward(x, cfg8)
+    tr = orc.linear_backward(gy, w, xq, sx, cfg8)
+    P = orc.make_WHT(128).astype(np.float64)
+    want = (P @ gy).T @ (P @ x) / n
+    assert _rel(tr.g_w, want) < 0.02
+
+
+def test_reference_cuda_rounding_is_biased():
+    """The reference op's mantissa-driven rounding (kept for characterisation
+    only): values with an all-zero mantissa (0 and the powers of two) are
+    rounded UP, so it cannot be unbiased."""
+    assert orc.stoch_round_mantissa(np.array([2.0, -3.0, 0.0, 4.0], F32)).tolist() == [3, -3, 1, 5]
