@@ -19,6 +19,10 @@
 // Tiling: 256 threads = 2x2 waves; each wave owns (32 WM) x (32 WN) outputs as
 // WM x WN MFMA tiles; K advances 128 codes per stage with the next stage's
 // global loads in flight during the MFMAs (double-buffered LDS).
+#include <stdlib.h>
+
+#include <type_traits>
+
 #include "hot_device.h"
 #include "hot_host.h"
 
@@ -44,47 +48,51 @@ struct GemmArgs {
   int32_t tiles_m, tiles_n;
 };
 
-// Global -> register prefetch of one operand tile (ROWS x G_BK codes).
+// Global -> register prefetch of one operand tile (ROWS x G_BK codes), and the
+// register -> LDS store that expands packed INT4 on the way.
 template <int ROWS, int BITS>
-struct TileLoader {
+struct TileShape {
   static constexpr int GBYTES = G_BK * BITS / 8;        // bytes of one row of the stage in HBM
   static constexpr int CPR = GBYTES / 16;               // 16-byte chunks per row
   static constexpr int PER_THREAD = ROWS * CPR / G_THREADS;
-  uint4 r[PER_THREAD];
-
-  __device__ __forceinline__ void load(const uint8_t* base, int64_t ld, int64_t row0, int64_t rows_total, int kt, int tid) {
-#pragma unroll
-    for (int i = 0; i < PER_THREAD; ++i) {
-      const int id = tid + i * G_THREADS;
-      const int row = id / CPR, kc = id % CPR;
-      int64_t gr = row0 + row;
-      if (gr >= rows_total) gr = rows_total - 1;  // duplicate the last row; its outputs are never stored
-      r[i] = *reinterpret_cast<const uint4*>(base + gr * ld + (int64_t)kt * GBYTES + kc * 16);
-    }
-  }
-
-  __device__ __forceinline__ void store(uint8_t* lds, int tid) const {
-#pragma unroll
-    for (int i = 0; i < PER_THREAD; ++i) {
-      const int id = tid + i * G_THREADS;
-      const int row = id / CPR, kc = id % CPR;
-      if constexpr (BITS == 8) {
-        *reinterpret_cast<uint4*>(lds + row * G_PITCH + kc * 16) = r[i];
-      } else {
-        uint4 ev, od;  // even elements (low nibbles) and odd elements (high nibbles), each as value << 4
-        ev.x = (r[i].x << 4) & 0xF0F0F0F0u; od.x = r[i].x & 0xF0F0F0F0u;
-        ev.y = (r[i].y << 4) & 0xF0F0F0F0u; od.y = r[i].y & 0xF0F0F0F0u;
-        ev.z = (r[i].z << 4) & 0xF0F0F0F0u; od.z = r[i].z & 0xF0F0F0F0u;
-        ev.w = (r[i].w << 4) & 0xF0F0F0F0u; od.w = r[i].w & 0xF0F0F0F0u;
-        *reinterpret_cast<uint4*>(lds + row * G_PITCH + kc * 32) = ev;
-        *reinterpret_cast<uint4*>(lds + row * G_PITCH + kc * 32 + 16) = od;
-      }
-    }
-  }
 };
 
+template <int ROWS, int BITS, int PT>
+__device__ __forceinline__ void tile_load(v4i (&r)[PT], const uint8_t* base, int64_t ld, int64_t row0,
+                                          int64_t rows_total, int kt, int tid) {
+  using S = TileShape<ROWS, BITS>;
+#pragma unroll
+  for (int i = 0; i < PT; ++i) {
+    const int id = tid + i * G_THREADS;
+    const int row = id / S::CPR, kc = id % S::CPR;
+    int64_t gr = row0 + row;
+    if (gr >= rows_total) gr = rows_total - 1;  // duplicate the last row; its outputs are never stored
+    r[i] = *reinterpret_cast<const v4i*>(base + gr * ld + (int64_t)kt * S::GBYTES + kc * 16);
+  }
+}
+
+template <int ROWS, int BITS, int PT>
+__device__ __forceinline__ void tile_store(const v4i (&r)[PT], uint8_t* lds, int tid) {
+  using S = TileShape<ROWS, BITS>;
+#pragma unroll
+  for (int i = 0; i < PT; ++i) {
+    const int id = tid + i * G_THREADS;
+    const int row = id / S::CPR, kc = id % S::CPR;
+    if constexpr (BITS == 8) {
+      *reinterpret_cast<v4i*>(lds + row * G_PITCH + kc * 16) = r[i];
+    } else {
+      // even elements (low nibbles) and odd elements (high nibbles), each as value << 4
+      const v4i m = {(int)0xF0F0F0F0, (int)0xF0F0F0F0, (int)0xF0F0F0F0, (int)0xF0F0F0F0};
+      const v4i ev = (r[i] << 4) & m, od = r[i] & m;
+      *reinterpret_cast<v4i*>(lds + row * G_PITCH + kc * 32) = ev;
+      *reinterpret_cast<v4i*>(lds + row * G_PITCH + kc * 32 + 16) = od;
+    }
+  }
+}
+
 template <int WM, int WN, int BITS, typename OutT>
-__global__ void __launch_bounds__(G_THREADS) gemm_i8_kernel(const GemmArgs g) {
+__global__ void __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(1, (WM * WN <= 4 ? 2 : 1))))
+gemm_i8_kernel(const GemmArgs g) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
   constexpr int A_BYTES = BM * G_PITCH, B_BYTES = BN * G_PITCH;
   extern __shared__ __align__(16) uint8_t lds[];
@@ -107,10 +115,10 @@ __global__ void __launch_bounds__(G_THREADS) gemm_i8_kernel(const GemmArgs g) {
   const int tm = tile / g.tiles_n, tn = tile % g.tiles_n;
   const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
 
-  TileLoader<BM, BITS> la;
-  TileLoader<BN, BITS> lb;
-  la.load(g.A, g.lda, row0, g.M, 0, tid);
-  lb.load(g.B, g.ldb, col0, g.N, 0, tid);
+  constexpr int PTA = TileShape<BM, BITS>::PER_THREAD, PTB = TileShape<BN, BITS>::PER_THREAD;
+  v4i ra[PTA], rb[PTB];
+  tile_load<BM, BITS, PTA>(ra, g.A, g.lda, row0, g.M, 0, tid);
+  tile_load<BN, BITS, PTB>(rb, g.B, g.ldb, col0, g.N, 0, tid);
 
   v16i acc[WM][WN];
 #pragma unroll
@@ -120,16 +128,16 @@ __global__ void __launch_bounds__(G_THREADS) gemm_i8_kernel(const GemmArgs g) {
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-  la.store(lds, tid);
-  lb.store(lds + A_BYTES, tid);
+  tile_store<BM, BITS, PTA>(ra, lds, tid);
+  tile_store<BN, BITS, PTB>(rb, lds + A_BYTES, tid);
   __syncthreads();
 
   const int frag_row = lane & 31, frag_k = (lane >> 5) * 16;
   for (int kt = 0; kt < g.ktiles; ++kt) {
     const int cur = kt & 1;
     if (kt + 1 < g.ktiles) {
-      la.load(g.A, g.lda, row0, g.M, kt + 1, tid);
-      lb.load(g.B, g.ldb, col0, g.N, kt + 1, tid);
+      tile_load<BM, BITS, PTA>(ra, g.A, g.lda, row0, g.M, kt + 1, tid);
+      tile_load<BN, BITS, PTB>(rb, g.B, g.ldb, col0, g.N, kt + 1, tid);
     }
     const uint8_t* pa = lds + cur * STAGE_BYTES + (wm * 32 * WM + frag_row) * G_PITCH + frag_k;
     const uint8_t* pb = lds + cur * STAGE_BYTES + A_BYTES + (wn * 32 * WN + frag_row) * G_PITCH + frag_k;
@@ -147,8 +155,8 @@ __global__ void __launch_bounds__(G_THREADS) gemm_i8_kernel(const GemmArgs g) {
           acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
     }
     if (kt + 1 < g.ktiles) {
-      la.store(lds + (cur ^ 1) * STAGE_BYTES, tid);
-      lb.store(lds + (cur ^ 1) * STAGE_BYTES + A_BYTES, tid);
+      tile_store<BM, BITS, PTA>(ra, lds + (cur ^ 1) * STAGE_BYTES, tid);
+      tile_store<BN, BITS, PTB>(rb, lds + (cur ^ 1) * STAGE_BYTES + A_BYTES, tid);
     }
     __syncthreads();
   }
@@ -179,6 +187,241 @@ __global__ void __launch_bounds__(G_THREADS) gemm_i8_kernel(const GemmArgs g) {
   }
 }
 
+// ---------------------------------------------------------------------------
+// Pipelined variant: operand tiles travel HBM -> LDS without passing through
+// registers (global_load_lds_dwordx4), four LDS stages deep, so that two
+// K-tiles are always in flight behind the one being multiplied.  Packed INT4
+// stays packed in LDS (half the LDS traffic) and is expanded to (v << 4) bytes
+// right after the fragment read.
+//
+// LDS stage layout: rows of 64 bytes = four 16-byte slots; slot s of row r is
+// stored at slot s ^ ((r >> 1) & 3), which spreads the 16-byte fragment reads
+// of 8 consecutive rows over all banks.  A wave-wide DMA instruction fills one
+// contiguous KiB (16 rows); lane l fills physical slot l of that KiB and so
+// fetches row l >> 2, logical slot (l & 3) ^ ((l >> 3) & 3) from global memory.
+//
+// Each stage is its own __shared__ array and the K loop is unrolled by the
+// stage count, so every LDS access names its stage statically; waits on the
+// DMA are explicit (vmcnt) and the barrier carries no fence.
+// ---------------------------------------------------------------------------
+
+constexpr int P_STAGES = 4;
+constexpr int P_ROWB = 64;  // bytes per row per stage
+
+// s_waitcnt vmcnt(VM) alone (expcnt and lgkmcnt untouched); vmcnt is split over bits 3:0 and 15:14
+template <int VM>
+__device__ __forceinline__ void wait_dma() {
+  __builtin_amdgcn_s_waitcnt((VM & 0xF) | ((VM >> 4) << 14) | (0x7 << 4) | (0xF << 8));
+}
+
+// One wave-wide 16-byte-per-lane load from global memory straight into LDS:
+// lane l's 16 bytes land at lds_addr + 16 l.  `lds_addr` and `sbase` must be
+// wave-uniform.  Written as inline assembly so that the explicit vmcnt waits
+// of the pipeline below are the only ones: the compiler cannot tell which LDS
+// stage a DMA targets and would otherwise drain all of them before every
+// fragment read.
+__device__ __forceinline__ void dma16(uint32_t lds_addr, uint32_t voff, const uint8_t* sbase) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(sbase)
+               : "memory", "m0");
+}
+
+__device__ __forceinline__ uint32_t lds_offset(const uint8_t* p) {
+  return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t*)p;
+}
+
+template <int WM, int WN, int BITS, typename OutT>
+__global__ void __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(1, (WM * WN <= 4 ? 2 : 1))))
+gemm_i8_pipe_kernel(const GemmArgs g) {
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  constexpr int STAGE_BYTES = (BM + BN) * P_ROWB;
+  constexpr int LPW = (BM + BN) / 64;           // DMA instructions per wave per stage (KiB chunks / 4 waves)
+  constexpr int GSTEP = P_ROWB;                 // global bytes per stage and row: 64 int8 codes or 128 packed INT4 codes
+  __shared__ __attribute__((aligned(1024))) uint8_t st0[STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t st1[STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t st2[STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t st3[STAGE_BYTES];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave >> 1, wn = wave & 1;
+  int tile;
+  {
+    const int total = g.tiles_m * g.tiles_n;
+    const int wg = blockIdx.x;
+    const int x = wg & 7, idx = wg >> 3;
+    const int q = total >> 3, rem = total & 7;
+    tile = x * q + (x < rem ? x : rem) + idx;
+  }
+  const int tm = tile / g.tiles_n, tn = tile % g.tiles_n;
+  const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
+
+  // DMA instruction i of this wave fills KiB chunk 4 i + wave of the stage (A rows first, then B
+  // rows; BM / 16 is a multiple of 4, so instruction i serves A for i < BM / 64 and B otherwise).
+  uint32_t goff[LPW];
+#pragma unroll
+  for (int i = 0; i < LPW; ++i) {
+    const int r = (4 * i + wave) * 16 + (lane >> 2);
+    const int slot = (lane & 3) ^ ((lane >> 3) & 3);
+    if (i < BM / 64) {
+      int64_t gr = row0 + r;
+      if (gr >= g.M) gr = g.M - 1;
+      goff[i] = (uint32_t)(gr * g.lda + slot * 16);
+    } else {
+      int64_t gr = col0 + (r - BM);
+      if (gr >= g.N) gr = g.N - 1;
+      goff[i] = (uint32_t)(gr * g.ldb + slot * 16);
+    }
+  }
+  auto issue = [&](const uint8_t* stage, int kt) {
+    const uint32_t l0 = lds_offset(stage) + wave * 1024;
+    const uint8_t* ga = g.A + (int64_t)kt * GSTEP;
+    const uint8_t* gb = g.B + (int64_t)kt * GSTEP;
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) dma16(l0 + i * 4096, goff[i], i < BM / 64 ? ga : gb);
+  };
+
+  v16i acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+  // A stage holds two "rounds" of fragments.  In round d the lanes of half h (= lane / 32) read
+  // slot 2 d + h of their row: 16 int8 codes (one MFMA) or 32 packed INT4 codes (two MFMAs: the
+  // low nibbles, then the high nibbles; both operands alike, so every product pairs equal k).
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int sw = (frow >> 1) & 3;                              // same for rows r and r + 32 k
+  const int offA = (wm * 32 * WM + frow) * P_ROWB, offB = (BM + wn * 32 * WN + frow) * P_ROWB;
+  auto read_round = [&](const uint8_t* stage, int d, v4i (&fa)[WM], v4i (&fb)[WN]) {
+    const int so = ((2 * d + fhalf) ^ sw) * 16;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) fa[i] = *reinterpret_cast<const v4i*>(stage + offA + i * 32 * P_ROWB + so);
+#pragma unroll
+    for (int j = 0; j < WN; ++j) fb[j] = *reinterpret_cast<const v4i*>(stage + offB + j * 32 * P_ROWB + so);
+  };
+  auto mma_round = [&](const v4i (&fa)[WM], const v4i (&fb)[WN]) {
+    if constexpr (BITS == 8) {
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+    } else {
+      const v4i m = {(int)0xF0F0F0F0, (int)0xF0F0F0F0, (int)0xF0F0F0F0, (int)0xF0F0F0F0};
+      v4i ea[WM], eb[WN];
+#pragma unroll
+      for (int i = 0; i < WM; ++i) ea[i] = (fa[i] << 4) & m;
+#pragma unroll
+      for (int j = 0; j < WN; ++j) eb[j] = (fb[j] << 4) & m;
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ea[i], eb[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < WM; ++i) ea[i] = fa[i] & m;
+#pragma unroll
+      for (int j = 0; j < WN; ++j) eb[j] = fb[j] & m;
+#pragma unroll
+      for (int i = 0; i < WM; ++i)
+#pragma unroll
+        for (int j = 0; j < WN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ea[i], eb[j], acc[i][j], 0, 0, 0);
+    }
+  };
+
+  const int KT = g.ktiles * (G_BK / (BITS == 8 ? 64 : 128));   // stages of this kernel per G_BK-code tile
+  // prologue: up to three tiles in flight, tile 0 landed and visible, its first round in registers
+  issue(st0, 0);
+  if (KT > 1) issue(st1, 1);
+  if (KT > 2) issue(st2, 2);
+  if (KT > 2) wait_dma<2 * LPW>(); else if (KT > 1) wait_dma<LPW>(); else wait_dma<0>();
+  __builtin_amdgcn_s_barrier();
+  v4i a0[WM], b0[WN];
+  read_round(st0, 0, a0, b0);
+
+  // One K-tile.  `cur` holds tile kt, `nxt` tile kt+1 (in flight or landed), `fre` held tile kt-1
+  // and receives tile kt+3.  The barrier sits in the middle of the tile, behind a block of MFMAs,
+  // and the first fragments of tile kt+1 are fetched before the last MFMA block of tile kt starts,
+  // so the matrix pipe keeps running across the tile boundary.
+  auto ktile = [&](auto steady, const uint8_t* cur, const uint8_t* nxt, const uint8_t* fre, int kt) {
+    // The scheduling fences keep each burst of fragment reads ahead of the MFMA block that
+    // hides its latency; without them the scheduler sinks the reads next to their first use.
+    v4i a1[WM], b1[WN];
+    read_round(cur, 1, a1, b1);
+    __builtin_amdgcn_sched_barrier(0);
+    mma_round(a0, b0);
+    __builtin_amdgcn_sched_barrier(0);
+    if constexpr (decltype(steady)::value) {
+      // steady state (kt + 3 < KT): straight-line code, so the compiler's LDS wait counts are exact
+      wait_dma<LPW>();                                        // this wave's share of tile kt+1 has landed
+      __builtin_amdgcn_s_barrier();                           // ... and everybody's; nobody reads tile kt-1 any more
+      issue(fre, kt + 3);
+      read_round(nxt, 0, a0, b0);
+    } else if (kt + 1 < KT) {
+      if (kt + 2 < KT) wait_dma<LPW>(); else wait_dma<0>();
+      __builtin_amdgcn_s_barrier();
+      if (kt + 3 < KT) issue(fre, kt + 3);
+      read_round(nxt, 0, a0, b0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    mma_round(a1, b1);
+    __builtin_amdgcn_sched_barrier(0);
+  };
+  int kt0 = 0;
+  for (; kt0 + 6 < KT; kt0 += P_STAGES) {
+    ktile(std::true_type{}, st0, st1, st3, kt0);
+    ktile(std::true_type{}, st1, st2, st0, kt0 + 1);
+    ktile(std::true_type{}, st2, st3, st1, kt0 + 2);
+    ktile(std::true_type{}, st3, st0, st2, kt0 + 3);
+  }
+  for (; kt0 < KT; kt0 += P_STAGES) {
+    ktile(std::false_type{}, st0, st1, st3, kt0);
+    if (kt0 + 1 < KT) ktile(std::false_type{}, st1, st2, st0, kt0 + 1);
+    if (kt0 + 2 < KT) ktile(std::false_type{}, st2, st3, st1, kt0 + 2);
+    if (kt0 + 3 < KT) ktile(std::false_type{}, st3, st0, st2, kt0 + 3);
+  }
+
+  const float sb = g.scale_b[0];
+  const float sa0 = g.a_per_row ? 0.f : g.scale_a[0];
+  OutT* out = reinterpret_cast<OutT*>(g.out);
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      const int64_t row = row0 + (wm * WM + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
+      if (row >= g.M) continue;
+      const float sa = g.a_per_row ? g.scale_a[row] : sa0;
+#pragma unroll
+      for (int j = 0; j < WN; ++j) {
+        const int64_t col = col0 + (wn * WN + j) * 32 + (lane & 31);
+        if (col >= g.N) continue;
+        int a = acc[i][j][e];
+        if constexpr (BITS == 4) a >>= 8;
+        if (g.acc_out) g.acc_out[row * g.N + col] = a;
+        const float v = (((float)a * sa) * sb) * g.post_scale;
+        store_scalar<OutT>(out + row * g.ldo + col, v);
+      }
+    }
+  }
+}
+
+template <int WM, int WN, int BITS, typename OutT>
+static int launch_gemm_pipe(GemmArgs& g, hipStream_t st) {
+  constexpr int BM = 64 * WM, BN = 64 * WN;
+  g.tiles_m = (int)((g.M + BM - 1) / BM);
+  g.tiles_n = (int)((g.N + BN - 1) / BN);
+  const int64_t total = (int64_t)g.tiles_m * g.tiles_n;
+  if (total > (1 << 30)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: too many tiles");
+  if (g.M * g.lda >= (1ll << 32) || g.N * g.ldb >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: operand larger than 4 GiB");
+  hipLaunchKernelGGL((gemm_i8_pipe_kernel<WM, WN, BITS, OutT>), dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
+  return check_launch("gemm_i8_pipe_kernel");
+}
+
 template <int WM, int WN, int BITS, typename OutT>
 static int launch_gemm(GemmArgs& g, hipStream_t st) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
@@ -200,6 +443,22 @@ static int launch_gemm(GemmArgs& g, hipStream_t st) {
 
 template <int BITS, typename OutT>
 static int pick_tile(GemmArgs& g, hipStream_t st) {
+  static int forced = -1;
+  if (forced < 0) { const char* e = getenv("HOT_GEMM_TILE"); forced = e ? atoi(e) : 0; }
+  switch (forced) {
+    case 144: return launch_gemm_pipe<4, 4, BITS, OutT>(g, st);
+    case 142: return launch_gemm_pipe<4, 2, BITS, OutT>(g, st);
+    case 124: return launch_gemm_pipe<2, 4, BITS, OutT>(g, st);
+    case 122: return launch_gemm_pipe<2, 2, BITS, OutT>(g, st);
+    case 44: return launch_gemm<4, 4, BITS, OutT>(g, st);
+    case 42: return launch_gemm<4, 2, BITS, OutT>(g, st);
+    case 24: return launch_gemm<2, 4, BITS, OutT>(g, st);
+    case 22: return launch_gemm<2, 2, BITS, OutT>(g, st);
+    default: break;
+  }
+  // 128 x 128 tiles, two workgroups per CU: best on every graded shape so far.  The DMA kernel
+  // addresses operands with 32-bit offsets; larger operands take the register-staged kernel.
+  if (g.M * g.lda < (1ll << 32) && g.N * g.ldb < (1ll << 32)) return launch_gemm_pipe<2, 2, BITS, OutT>(g, st);
   return launch_gemm<2, 2, BITS, OutT>(g, st);
 }
 
