@@ -12,13 +12,15 @@
 // 86-122) and by the transposes the reference op feeds its GEMMs with
 // (cuda_measure/HLQ_backward_kernel.cu:561,610-611).
 //
-// Mapping: a lane owns CPL adjacent channels (columns) and all n rows of one
-// token block, so the butterflies need no cross-lane traffic and every load is
-// contiguous across the wave.  The four waves of a workgroup share a channel
-// group and take different token blocks; codes are staged in LDS as
-// [channel][k] so that each channel's K-run leaves the CU as one contiguous
-// segment.  Two passes over the input (statistics, then quantise): the scale
-// of a tensor depends on all of it.
+// Data movement.  A workgroup owns 256 adjacent channels (columns) and a run
+// of token blocks.  Rows arrive 16 at a time through coalesced 16-byte loads
+// (each row of the tile is one contiguous segment of HBM), are parked in a
+// double-buffered LDS tile, and every thread then pulls ITS channel's 16
+// values out of LDS: from there on a thread holds whole columns, so the
+// butterflies (stage order h = 1, 2, 4, ..., the canonical fp32 order) need
+// no cross-lane traffic.  Quantised codes are staged in LDS as [channel][k]
+// and leave the CU as one contiguous K-run per channel.  Two passes over the
+// input (statistics, then quantise): the step of a tensor depends on all of it.
 //
 // HBM traffic per input element: 2 * sizeof(in) read + (r/n) * bits/8 written.
 #include "hot_device.h"
@@ -26,8 +28,8 @@
 
 namespace hot {
 
-constexpr int COL_THREADS = 256;
-constexpr int COL_WAVES = COL_THREADS / 64;
+constexpr int CW = 256;        // threads per workgroup = channels per workgroup
+constexpr int CW_ROWS = 16;    // rows staged per step
 
 struct ColArgs {
   const void* in;
@@ -42,123 +44,282 @@ struct ColArgs {
   float* scales_out;
   uint64_t seed;
   uint32_t stream;
-  int32_t r, bits, store4, rounding, mode, bpw;
+  int32_t r, rpad, bits, store4, rounding, mode, tb;
   int8_t slot[HOT_MAX_HLA_N];  // output position of natural row i, -1 = dropped
 };
 
-template <int N> struct cpl_of { static constexpr int value = N >= 64 ? 2 : 4; };
+template <typename T> struct raw_of { typedef uint16_t type; };
+template <> struct raw_of<float> { typedef uint32_t type; };
 
-template <typename T, int CPL>
-__device__ __forceinline__ void load_cpl(const T* p, float* o) {
-  constexpr int BYTES = CPL * (int)sizeof(T);
-  if constexpr (BYTES == 4) {
-    const uint32_t w = *reinterpret_cast<const uint32_t*>(p);
-    if constexpr (sizeof(T) == 4) { o[0] = as_f(w); }
-    else { float t[8]; unpack_vec<T>(make_uint4(w, 0, 0, 0), t); o[0] = t[0]; o[1] = t[1]; }
-  } else if constexpr (BYTES == 8) {
-    const uint2 w = *reinterpret_cast<const uint2*>(p);
-    if constexpr (sizeof(T) == 4) { o[0] = as_f(w.x); o[1] = as_f(w.y); }
-    else { float t[8]; unpack_vec<T>(make_uint4(w.x, w.y, 0, 0), t); o[0] = t[0]; o[1] = t[1]; o[2] = t[2]; o[3] = t[3]; }
-  } else {
-    static_assert(BYTES == 16, "unsupported channels-per-lane");
-    const uint4 w = *reinterpret_cast<const uint4*>(p);
-    float t[8];
-    unpack_vec<T>(w, t);
-#pragma unroll
-    for (int i = 0; i < CPL; ++i) o[i] = t[i];
-  }
-}
+template <typename T> __device__ __forceinline__ float cvt_raw(typename raw_of<T>::type v);
+template <> __device__ __forceinline__ float cvt_raw<float>(uint32_t v) { return as_f(v); }
+template <> __device__ __forceinline__ float cvt_raw<bf16_t>(uint16_t v) { return as_f((uint32_t)v << 16); }
+template <> __device__ __forceinline__ float cvt_raw<f16_t>(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
 
-// Loads block `blk` (N rows x CPL channels starting at channel c0) and applies
-// the unnormalised FWHT along the row index, stages h = 1, 2, 4, ...
-template <typename T, int N, int CPL>
-__device__ __forceinline__ void load_transform(const T* in, int64_t C, int64_t blk, int64_t c0, float (&x)[N][CPL]) {
-  const T* p = in + (blk * N) * C + c0;
-#pragma unroll
-  for (int i = 0; i < N; ++i) load_cpl<T, CPL>(p + (int64_t)i * C, x[i]);
+// Unnormalised FWHT of the N-point groups of v[0..LEN), stages h = 1, 2, 4, ...
+template <int N, int LEN>
+__device__ __forceinline__ void fwht_regs(float (&v)[LEN]) {
 #pragma unroll
   for (int h = 1; h < N; h <<= 1) {
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
+    for (int i = 0; i < LEN; ++i) {
       if ((i & h) == 0) {
-#pragma unroll
-        for (int c = 0; c < CPL; ++c) {
-          const float a = x[i][c], b = x[i + h][c];
-          x[i][c] = a + b;
-          x[i + h][c] = a - b;
-        }
+        const float a = v[i], b = v[i + h];
+        v[i] = a + b;
+        v[i + h] = a - b;
       }
     }
   }
 }
 
-// ---- pass 1: statistics of the kept coefficients ------------------------------
+// rint(x / d) with rcp = 1 / d precomputed: the product x * rcp is within 1.5 * 2^-23 |x/d| of
+// the correctly rounded quotient, so it rounds to the same integer unless it lies within 2^-14 of
+// a half-integer (|x/d| <= 128); only then is the IEEE division carried out.
+__device__ __forceinline__ int quant_nearest_fast(float x, float d, float rcp) {
+  const float p = x * rcp;
+  float k = rintf(p);
+  if (__builtin_expect(fabsf(p - k) > 0.5f - 6.103515625e-05f, 0)) k = rintf(x / d);
+  return (int)k;
+}
 
-template <typename T, int N>
-__global__ void __launch_bounds__(COL_THREADS) colwise_stats_kernel(const ColArgs a) {
-  constexpr int CPL = cpl_of<N>::value;
-  __shared__ float s_max[COL_WAVES];
-  __shared__ double s_sum[2][COL_WAVES];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int64_t c0 = ((int64_t)blockIdx.x * 64 + lane) * CPL;
-  const bool active = c0 < a.C;
-  const int tb = COL_WAVES * a.bpw;
-  const int64_t b0 = (int64_t)blockIdx.y * tb + (int64_t)wave * a.bpw;
+// Streams the rows of the workgroup's tile through a ring of LDS buffers with
+// direct global -> LDS loads (16 bytes per lane, no registers in between).
+// Step s covers rows [row0 + 16 s, +16); a buffer holds them as [16][256] raw
+// elements.  A wave-wide load fills one contiguous KiB, i.e. 1024 / (256
+// sizeof(T)) rows; wave w issues KiB chunks w, w + 4, ...  Rows past the end
+// of the input and channels past C are redirected to valid addresses: what
+// they deliver is never consumed.
+constexpr int CW_DEPTH = 4;    // LDS buffers in the ring: three steps in flight behind the one in use
 
-  float cmax[CPL];
+template <typename T>
+struct RowStream {
+  static constexpr int RB = CW * (int)sizeof(T);                 // bytes per staged row
+  static constexpr int BUF_BYTES = CW_ROWS * RB;
+  static constexpr int LPW = BUF_BYTES / 1024 / (CW / 64);       // DMA instructions per wave per step
+  static constexpr int VPR = RB / 16;                            // 16-byte vectors per staged row
+  const uint8_t* base;   // &in[0][cg0]
+  uint32_t pitch;        // bytes per input row
+  int64_t rows_total;
+  int64_t row0;
+  int nvec_row;          // valid 16-byte vectors per row for this channel group
+};
+
+// s_waitcnt vmcnt(VM) lgkmcnt(0); vmcnt is split over bits 3:0 and 15:14
+template <int VM>
+__device__ __forceinline__ void wait_stream() {
+  __builtin_amdgcn_s_waitcnt((VM & 0xF) | ((VM >> 4) << 14) | (0x7 << 4) | (0x0 << 8));
+}
+
+__device__ __forceinline__ void dma16_to_lds(uint32_t lds_addr, uint32_t voff, const uint8_t* sbase) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+               :
+               : "s"(lds_addr), "v"(voff), "s"(sbase)
+               : "memory", "m0");
+}
+
+template <typename T>
+__device__ __forceinline__ void rs_issue(const RowStream<T>& rs, uint32_t buf_lds, int step, int wave, int lane) {
+  constexpr int VPR = RowStream<T>::VPR;
+  constexpr int RPC = 1024 / RowStream<T>::RB > 0 ? 1024 / RowStream<T>::RB : 1;   // rows per KiB chunk
+#pragma unroll
+  for (int i = 0; i < RowStream<T>::LPW; ++i) {
+    const int chunk = wave + (CW / 64) * i;
+    int64_t row = rs.row0 + (int64_t)step * CW_ROWS + chunk * RPC + lane / VPR;
+    if (row >= rs.rows_total) row = rs.rows_total - 1;
+    int vec = lane % VPR;
+    if (vec >= rs.nvec_row) vec = rs.nvec_row - 1;
+    dma16_to_lds(buf_lds + chunk * 1024, (uint32_t)row * rs.pitch + (uint32_t)vec * 16, rs.base);
+  }
+}
+
+template <typename T>
+__device__ __forceinline__ void rs_column(const uint8_t* buf, int tid, float* v) {
+  typedef typename raw_of<T>::type raw_t;
+  const raw_t* p = reinterpret_cast<const raw_t*>(buf) + tid;
+#pragma unroll
+  for (int i = 0; i < CW_ROWS; ++i) v[i] = cvt_raw<T>(p[i * CW]);
+}
+
+// ---- the kernel: PASS 0 = statistics, PASS 1 = quantise + transposed store ----
+
+template <typename T, int N, int PASS, int ROUND, bool SAWB>
+__global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
+  constexpr int SPB = N >= CW_ROWS ? N / CW_ROWS : 1;        // steps per token block
+  constexpr int BPS = N >= CW_ROWS ? 1 : CW_ROWS / N;        // token blocks per step
+  constexpr int XL = N >= CW_ROWS ? N : CW_ROWS;             // values a thread holds
+  constexpr int BUF = RowStream<T>::BUF_BYTES;
+  extern __shared__ __align__(16) uint8_t lds[];
+  __shared__ float s_max[CW / 64];
+  __shared__ double s_sum[2][CW / 64];
+  uint8_t* const stage = lds + CW_DEPTH * BUF;               // PASS 1: codes [channel][k]
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t cg0 = (int64_t)blockIdx.x * CW;
+  const int64_t c = cg0 + tid;
+  const bool active = c < a.C;
+  const int64_t blk0 = (int64_t)blockIdx.y * a.tb;
+  int nblk = (int)((a.NB - blk0) < a.tb ? (a.NB - blk0) : a.tb);
+  const int nsteps = (nblk * N + CW_ROWS - 1) / CW_ROWS;
+  const int qmax = (1 << (a.bits - 1)) - 1;
+  const int sb = a.tb * a.r;        // staged code bytes per channel
+  const int pitch = sb + 4;
+
+  RowStream<T> rs;
+  rs.base = reinterpret_cast<const uint8_t*>(a.in) + cg0 * (int64_t)sizeof(T);
+  rs.pitch = (uint32_t)(a.C * (int64_t)sizeof(T));
+  rs.rows_total = a.R;
+  rs.row0 = blk0 * N;
+  {
+    const int64_t chans = (a.C - cg0) < CW ? (a.C - cg0) : CW;
+    rs.nvec_row = (int)(chans * (int64_t)sizeof(T) / 16);
+  }
+
+  float d = 1.f, rcp = 1.f, clip = 0.f;
+  if constexpr (PASS == 1) {
+    uint32_t* l32 = reinterpret_cast<uint32_t*>(stage);
+    for (int i = tid; i < CW * pitch / 4; i += CW) l32[i] = 0u;   // gaps of partial groups must read as 0
+    __syncthreads();
+    if (a.mode == HOT_SCALE_ROW) {
+      d = active ? (a.colmax[c] / (float)qmax + 1e-11f) : 1.f;
+    } else {
+      d = a.stat[1] + 1e-11f;
+      clip = a.stat[2];
+    }
+    rcp = 1.0f / d;
+  }
+
+  float cmax = 0.f;
   double ssq = 0.0, sab = 0.0;
-#pragma unroll
-  for (int c = 0; c < CPL; ++c) cmax[c] = 0.f;
+  float x[XL];
 
-  for (int j = 0; j < a.bpw; ++j) {
-    const int64_t blk = b0 + j;
-    if (blk >= a.NB || !active) break;
-    float x[N][CPL];
-    load_transform<T, N, CPL>((const T*)a.in, a.C, blk, c0, x);
+  // Transforms and consumes the token blocks held in x; `bl` is the group-local index of the first.
+  auto consume = [&](int bl) {
+    fwht_regs<N, XL>(x);
 #pragma unroll
-    for (int i = 0; i < N; ++i) {
-      if (a.slot[i] >= 0) {
+    for (int g = 0; g < BPS; ++g) {
+      const int blk = bl + g;
+      if (blk < nblk) {
+        int visited = 0;      // kept coefficients of this block quantised so far (stochastic rounding)
+        float u[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int c = 0; c < CPL; ++c) {
-          cmax[c] = fmaxf(cmax[c], fabsf(x[i][c]));
-          if (a.mode == HOT_SCALE_SAWB) { ssq += (double)x[i][c] * (double)x[i][c]; sab += (double)fabsf(x[i][c]); }
+        for (int i = 0; i < N; ++i) {
+          const int sl = a.slot[i];
+          if (sl >= 0) {
+            float v = x[g * N + i];
+            if constexpr (PASS == 0) {
+              cmax = fmaxf(cmax, fabsf(v));
+              if constexpr (SAWB) { ssq += (double)v * (double)v; sab += (double)fabsf(v); }
+            } else {
+              if constexpr (SAWB) v = fminf(fmaxf(v, -clip), clip);
+              int q;
+              if constexpr (ROUND == HOT_ROUND_NEAREST) {
+                q = quant_nearest_fast(v, d, rcp);
+              } else {
+                // counter = ((channel * NB + block) * rpad + visit index) / 4, word = visit index % 4
+                if ((visited & 3) == 0) {
+                  const uint64_t quad = ((uint64_t)c * (uint64_t)a.NB + (uint64_t)(blk0 + blk)) * (uint64_t)(a.rpad >> 2) +
+                                        (uint64_t)(visited >> 2);
+                  sr_uniform4(quad, a.seed, a.stream, u);
+                }
+                const int w = visited & 3;
+                q = q_stoch(v / d, w == 0 ? u[0] : w == 1 ? u[1] : w == 2 ? u[2] : u[3]);
+                ++visited;
+              }
+              q = clampi(q, -qmax, qmax);
+              stage[tid * pitch + blk * a.r + sl] = (uint8_t)(q & 0xFF);
+            }
+          }
         }
       }
     }
+  };
+
+  // ring of CW_DEPTH LDS buffers: steps s+1 .. s+CW_DEPTH-1 are in flight while step s is consumed
+  constexpr int LPW = RowStream<T>::LPW;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t*)lds;
+#pragma unroll
+  for (int s = 0; s < CW_DEPTH - 1; ++s)
+    if (s < nsteps) rs_issue<T>(rs, lds0 + s * BUF, s, wave, lane);
+  // one step: wait for its rows, let the ring advance, pull this thread's 16 values into x[xo..]
+  auto step = [&](int s, float* dst) {
+    // this wave's share of step s has landed, and its own LDS reads of step s-1 are complete ...
+    if (s + 2 < nsteps) wait_stream<2 * LPW>(); else if (s + 1 < nsteps) wait_stream<LPW>(); else wait_stream<0>();
+    __builtin_amdgcn_s_barrier();   // ... and so for every wave: the buffer of step s-1 may be refilled
+    if (s + CW_DEPTH - 1 < nsteps) rs_issue<T>(rs, lds0 + ((s + CW_DEPTH - 1) % CW_DEPTH) * BUF, s + CW_DEPTH - 1, wave, lane);
+    rs_column<T>(lds + (s % CW_DEPTH) * BUF, tid, dst);
+  };
+  if constexpr (N >= CW_ROWS) {
+    for (int bl = 0; bl < nblk; ++bl) {
+#pragma unroll
+      for (int p = 0; p < SPB; ++p) step(bl * SPB + p, x + p * CW_ROWS);
+      consume(bl);
+    }
+  } else {
+    for (int s = 0; s < nsteps; ++s) {
+      step(s, x);
+      consume(s * BPS);
+    }
   }
 
-  if (a.mode == HOT_SCALE_ROW) {
-    if (active) {
-#pragma unroll
-      for (int c = 0; c < CPL; ++c) atomic_max_nonneg(a.colmax + c0 + c, cmax[c]);
+  if constexpr (PASS == 0) {
+    if (a.mode == HOT_SCALE_ROW) {
+      if (active) atomic_max_nonneg(a.colmax + c, cmax);
+      return;
     }
-    return;
-  }
-  if (a.mode == HOT_SCALE_TENSOR) {
-    float m = 0.f;
-#pragma unroll
-    for (int c = 0; c < CPL; ++c) m = fmaxf(m, cmax[c]);
-    m = wave_max(m);
-    if (lane == 0) s_max[wave] = m;
+    if (a.mode == HOT_SCALE_TENSOR) {
+      float m = wave_max(active ? cmax : 0.f);
+      if (lane == 0) s_max[wave] = m;
+      __syncthreads();
+      if (tid == 0) {
+        float mm = s_max[0];
+        for (int i = 1; i < CW / 64; ++i) mm = fmaxf(mm, s_max[i]);
+        atomic_max_nonneg(a.stat, mm);
+      }
+      return;
+    }
+    // SAWB: per-workgroup partial sums, reduced in a fixed order by the finalize kernel
+    ssq = wave_sum(active ? ssq : 0.0);
+    sab = wave_sum(active ? sab : 0.0);
+    if (lane == 0) { s_sum[0][wave] = ssq; s_sum[1][wave] = sab; }
     __syncthreads();
     if (tid == 0) {
-      float mm = s_max[0];
-      for (int i = 1; i < COL_WAVES; ++i) mm = fmaxf(mm, s_max[i]);
-      atomic_max_nonneg(a.stat, mm);
+      double q = 0.0, b = 0.0;
+      for (int i = 0; i < CW / 64; ++i) { q += s_sum[0][i]; b += s_sum[1][i]; }
+      const int64_t wg = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
+      a.partial[2 * wg] = q;
+      a.partial[2 * wg + 1] = b;
     }
-    return;
-  }
-  // SAWB: per-workgroup partial sums, reduced in a fixed order by the finalize kernel
-  ssq = wave_sum(ssq);
-  sab = wave_sum(sab);
-  if (lane == 0) { s_sum[0][wave] = ssq; s_sum[1][wave] = sab; }
-  __syncthreads();
-  if (tid == 0) {
-    double q = 0.0, b = 0.0;
-    for (int i = 0; i < COL_WAVES; ++i) { q += s_sum[0][i]; b += s_sum[1][i]; }
-    const int64_t wg = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
-    a.partial[2 * wg] = q;
-    a.partial[2 * wg + 1] = b;
+  } else {
+    __syncthreads();
+    // flush: each channel's staged run is one contiguous global segment
+    const bool last = blk0 + a.tb >= a.NB;
+    const int out_sb = a.store4 ? sb / 2 : sb;
+    const int64_t seg0 = (int64_t)blockIdx.y * out_sb;      // byte offset in the output row
+    const int64_t seg_end = last ? a.ld_out : seg0 + out_sb;
+    const int ndw = (int)((seg_end - seg0) / 4);            // output dwords per channel
+    const int sdw = out_sb / 4;                             // of which staged
+    const int nch = (int)((a.C - cg0) < CW ? (a.C - cg0) : CW);
+    // a wave walks along K of one channel: contiguous bytes of one output row per store
+    for (int ch = wave; ch < nch; ch += CW / 64) {
+      const uint32_t* row = reinterpret_cast<const uint32_t*>(stage + ch * pitch);
+      uint32_t* orow = reinterpret_cast<uint32_t*>(a.out + (cg0 + ch) * a.ld_out + seg0);
+      for (int jd = lane; jd < ndw; jd += 64) {
+        uint32_t w = 0u;
+        if (jd < sdw) {
+          if (a.store4) {
+            const uint32_t lo = row[2 * jd], hi = row[2 * jd + 1];
+            // bytes b0..b7 -> nibbles: byte j of the result = (b[2j+1] << 4) | (b[2j] & 15)
+            const uint32_t l = (lo & 0x0F) | ((lo >> 4) & 0xF0) | ((lo >> 8) & 0x0F00) | ((lo >> 12) & 0xF000);
+            const uint32_t h = (hi & 0x0F) | ((hi >> 4) & 0xF0) | ((hi >> 8) & 0x0F00) | ((hi >> 12) & 0xF000);
+            w = (l & 0xFFFF) | (h << 16);
+          } else {
+            w = row[jd];
+          }
+        }
+        orow[jd] = w;
+      }
+    }
   }
 }
 
@@ -200,104 +361,6 @@ __global__ void __launch_bounds__(256) colwise_finalize_kernel(const ColArgs a, 
   }
 }
 
-// ---- pass 2: transform again, quantise, transpose through LDS, store --------
-
-template <typename T, int N, int ROUND, bool SAWB>
-__global__ void __launch_bounds__(COL_THREADS) colwise_quant_kernel(const ColArgs a) {
-  constexpr int CPL = cpl_of<N>::value;
-  constexpr int CG = 64 * CPL;  // channels per workgroup
-  extern __shared__ __align__(16) uint8_t lds[];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int tb = COL_WAVES * a.bpw;
-  const int sb = tb * a.r;           // code bytes per channel in LDS
-  const int pitch = sb + 4;          // odd dword pitch for even sb/4 .. keeps byte writes spread over banks
-  const int64_t cg0 = (int64_t)blockIdx.x * CG;
-  const int64_t c0 = cg0 + (int64_t)lane * CPL;
-  const bool active = c0 < a.C;
-  const int64_t b0 = (int64_t)blockIdx.y * tb + (int64_t)wave * a.bpw;
-  const int qmax = (1 << (a.bits - 1)) - 1;
-
-  // zero the staging area (partial token-block groups leave gaps that must read as 0)
-  {
-    uint32_t* l32 = reinterpret_cast<uint32_t*>(lds);
-    const int n32 = CG * pitch / 4;
-    for (int i = tid; i < n32; i += COL_THREADS) l32[i] = 0u;
-  }
-  __syncthreads();
-
-  float d[CPL], clip = 0.f;
-  if (a.mode == HOT_SCALE_ROW) {
-#pragma unroll
-    for (int c = 0; c < CPL; ++c) d[c] = active ? (a.colmax[c0 + c] / (float)qmax + 1e-11f) : 1.f;
-  } else {
-    const float s = a.stat[1];
-    clip = a.stat[2];
-#pragma unroll
-    for (int c = 0; c < CPL; ++c) d[c] = s + 1e-11f;
-  }
-
-  for (int j = 0; j < a.bpw; ++j) {
-    const int64_t blk = b0 + j;
-    if (blk >= a.NB || !active) break;
-    float x[N][CPL];
-    load_transform<T, N, CPL>((const T*)a.in, a.C, blk, c0, x);
-    const int kl0 = (wave * a.bpw + j) * a.r;  // position of this block inside the staged run
-#pragma unroll
-    for (int i = 0; i < N; ++i) {
-      const int sl = a.slot[i];
-      if (sl >= 0) {
-        float u[4];
-        if constexpr (ROUND == HOT_ROUND_STOCH) {
-          // element index of coefficient (k, c) is k * C + c; c0 is a multiple of CPL, so the
-          // lane's channels share one (CPL = 4) or half of one (CPL = 2) counter value
-          const uint64_t e = (uint64_t)(blk * a.r + sl) * (uint64_t)a.C + (uint64_t)c0;
-          sr_uniform4(e >> 2, a.seed, a.stream, u);
-        }
-#pragma unroll
-        for (int c = 0; c < CPL; ++c) {
-          float v = x[i][c];
-          if constexpr (SAWB) v = fminf(fmaxf(v, -clip), clip);
-          const float y = v / d[c];
-          int q;
-          if constexpr (ROUND == HOT_ROUND_NEAREST) {
-            q = q_nearest(y);
-          } else {
-            q = q_stoch(y, CPL == 4 ? u[c] : ((c0 & 2) ? u[2 + c] : u[c]));
-          }
-          q = clampi(q, -qmax, qmax);
-          lds[(lane * CPL + c) * pitch + kl0 + sl] = (uint8_t)(q & 0xFF);
-        }
-      }
-    }
-  }
-  __syncthreads();
-
-  // flush: each channel's staged run is one contiguous global segment
-  const bool last = (int64_t)(blockIdx.y + 1) * tb >= a.NB;
-  const int64_t seg0 = (int64_t)blockIdx.y * (a.store4 ? sb / 2 : sb);  // byte offset in the output row
-  const int64_t seg_end = last ? a.ld_out : seg0 + (a.store4 ? sb / 2 : sb);
-  const int ndw = (int)((seg_end - seg0) / 4);  // output dwords per channel
-  const int sdw = (a.store4 ? sb / 2 : sb) / 4; // of which staged
-  const int64_t nch = (a.C - cg0) < CG ? (a.C - cg0) : CG;
-  for (int64_t p = tid; p < nch * ndw; p += COL_THREADS) {
-    const int ch = (int)(p / ndw), jd = (int)(p % ndw);
-    uint32_t w = 0u;
-    if (jd < sdw) {
-      const uint32_t* row = reinterpret_cast<const uint32_t*>(lds + ch * pitch);
-      if (a.store4) {
-        const uint32_t lo = row[2 * jd], hi = row[2 * jd + 1];
-        // bytes b0..b7 -> nibbles: byte j of the result = (b[2j+1] << 4) | (b[2j] & 15)
-        const uint32_t l = (lo & 0x0F) | ((lo >> 4) & 0xF0) | ((lo >> 8) & 0x0F00) | ((lo >> 12) & 0xF000);
-        const uint32_t h = (hi & 0x0F) | ((hi >> 4) & 0xF0) | ((hi >> 8) & 0x0F00) | ((hi >> 12) & 0xF000);
-        w = (l & 0xFFFF) | (h << 16);
-      } else {
-        w = row[jd];
-      }
-    }
-    *reinterpret_cast<uint32_t*>(a.out + (cg0 + ch) * a.ld_out + seg0 + (int64_t)jd * 4) = w;
-  }
-}
-
 __global__ void colwise_clear_kernel(float* stat, float* colmax, int64_t C) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < 4) stat[i] = 0.f;
@@ -309,37 +372,54 @@ __global__ void colwise_clear_kernel(float* stat, float* colmax, int64_t C) {
 static constexpr size_t COL_STAT_BYTES = 256;
 
 size_t colwise_workspace_bytes_impl(int64_t C) {
-  // stat | per-channel max | per-workgroup partial sums (worst-case count bounded on launch)
+  // stat | per-channel max | per-workgroup partial sums (at most 65536 workgroups)
   return COL_STAT_BYTES + (size_t)round_up(C * 4, 256) + (size_t)(2 * sizeof(double)) * 65536;
+}
+
+template <typename T, int N, int PASS, int ROUND, bool SAWB>
+static int launch_pass(const ColArgs& a, dim3 grid, size_t lds, hipStream_t st) {
+  static bool attr_done = false;  // one-time, read-only afterwards
+  if (!attr_done && lds > 48 * 1024) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&colwise_kernel<T, N, PASS, ROUND, SAWB>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    if (e != hipSuccess) return check_hip(e, "hipFuncSetAttribute(colwise_kernel)");
+    attr_done = true;
+  }
+  hipLaunchKernelGGL((colwise_kernel<T, N, PASS, ROUND, SAWB>), grid, dim3(CW), lds, st, a);
+  return HOT_OK;
 }
 
 template <typename T, int N>
 static int launch_colwise(ColArgs& a, hipStream_t st) {
-  constexpr int CPL = cpl_of<N>::value;
-  constexpr int CG = 64 * CPL;
-  // token blocks per wave: staged run of about 256 bytes per channel, LDS <= 48 KiB
-  int bpw = 8;
-  while (bpw > 1 && (COL_WAVES * bpw * a.r > 288 || (int64_t)CG * (COL_WAVES * bpw * a.r + 4) > 48 * 1024)) bpw >>= 1;
-  if ((int64_t)CG * (COL_WAVES * bpw * a.r + 4) > 64 * 1024) return fail(HOT_ERR_UNSUPPORTED, "colwise: staging does not fit LDS");
-  a.bpw = bpw;
-  const int tb = COL_WAVES * bpw;
-  const int64_t gx = (a.C + CG - 1) / CG, gy = (a.NB + tb - 1) / tb;
+  constexpr int BPS = N >= CW_ROWS ? 1 : CW_ROWS / N;
+  // token blocks per workgroup: a staged run of at least 128 code bytes per channel, a multiple of 4
+  // bytes (dword flush) and of the blocks that share a 16-row step
+  int tb = 4 > BPS ? 4 : BPS;
+  while (tb * a.r < 128) tb <<= 1;
+  a.tb = tb;
+  const size_t in_bytes = (size_t)CW_DEPTH * CW_ROWS * CW * sizeof(T);
+  const size_t lds_stats = in_bytes, lds_quant = in_bytes + (size_t)CW * (tb * a.r + 4);
+  if (lds_quant > 150 * 1024) return fail(HOT_ERR_UNSUPPORTED, "colwise: staging does not fit LDS");
+  const int64_t gx = (a.C + CW - 1) / CW, gy = (a.NB + tb - 1) / tb;
   if (gy > 65535 || gx * gy > 65536) return fail(HOT_ERR_UNSUPPORTED, "colwise: grid %lld x %lld too large", (long long)gx, (long long)gy);
-  const dim3 grid((unsigned)gx, (unsigned)gy), block(COL_THREADS);
-  const size_t lds = (size_t)CG * (tb * a.r + 4);
+  const dim3 grid((unsigned)gx, (unsigned)gy);
   const int64_t nclr = a.C > 4 ? a.C : 4;
   hipLaunchKernelGGL(colwise_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat,
                      a.mode == HOT_SCALE_ROW ? a.colmax : (float*)nullptr, a.C);
-  hipLaunchKernelGGL((colwise_stats_kernel<T, N>), grid, block, 0, st, a);
+  int rc;
+  if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 0, 0, true>(a, grid, lds_stats, st);
+  else rc = launch_pass<T, N, 0, 0, false>(a, grid, lds_stats, st);
+  if (rc) return rc;
   hipLaunchKernelGGL(colwise_finalize_kernel, dim3(1), dim3(256), 0, st, a, gx * gy);
   if (a.rounding == HOT_ROUND_STOCH) {
-    if (a.mode == HOT_SCALE_SAWB) hipLaunchKernelGGL((colwise_quant_kernel<T, N, 1, true>), grid, block, lds, st, a);
-    else hipLaunchKernelGGL((colwise_quant_kernel<T, N, 1, false>), grid, block, lds, st, a);
+    if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 1, 1, true>(a, grid, lds_quant, st);
+    else rc = launch_pass<T, N, 1, 1, false>(a, grid, lds_quant, st);
   } else {
-    if (a.mode == HOT_SCALE_SAWB) hipLaunchKernelGGL((colwise_quant_kernel<T, N, 0, true>), grid, block, lds, st, a);
-    else hipLaunchKernelGGL((colwise_quant_kernel<T, N, 0, false>), grid, block, lds, st, a);
+    if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 1, 0, true>(a, grid, lds_quant, st);
+    else rc = launch_pass<T, N, 1, 0, false>(a, grid, lds_quant, st);
   }
-  return check_launch("colwise_quant_kernel");
+  if (rc) return rc;
+  return check_launch("colwise_kernel");
 }
 
 template <typename T>
@@ -368,14 +448,15 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   if (bits != 4 && bits != 8) return fail(HOT_ERR_UNSUPPORTED, "%s: bits=%d (4 or 8)", who, bits);
   if (rounding != HOT_ROUND_NEAREST && rounding != HOT_ROUND_STOCH) return fail(HOT_ERR_INVALID, "%s: bad rounding %d", who, rounding);
   if (scale_mode < HOT_SCALE_TENSOR || scale_mode > HOT_SCALE_SAWB) return fail(HOT_ERR_INVALID, "%s: bad scale mode %d", who, scale_mode);
-  if (C % 4) return fail(HOT_ERR_UNSUPPORTED, "%s: channel count %lld must be a multiple of 4", who, (long long)C);
+  if (C % 8) return fail(HOT_ERR_UNSUPPORTED, "%s: channel count %lld must be a multiple of 8", who, (long long)C);
   if (((uintptr_t)in & 15) || ((uintptr_t)codes_out & 15)) return fail(HOT_ERR_INVALID, "%s: pointers must be 16-byte aligned", who);
+  if (R * C * 4 >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "%s: input of %lld x %lld elements exceeds the 32-bit offsets of the loader", who, (long long)R, (long long)C);
 
   ColArgs a;
   a.in = in; a.R = R; a.C = C; a.NB = R / n; a.Kout = a.NB * r;
   a.out = (int8_t*)codes_out; a.ld_out = ld_out;
   a.seed = seed; a.stream = rng_stream;
-  a.r = r; a.bits = bits; a.rounding = rounding; a.mode = scale_mode; a.bpw = 1;
+  a.r = r; a.rpad = (r + 3) & ~3; a.bits = bits; a.rounding = rounding; a.mode = scale_mode; a.tb = 4;
   for (int i = 0; i < HOT_MAX_HLA_N; ++i) a.slot[i] = -1;
   for (int k = 0; k < r; ++k) {
     if (rows[k] < 0 || rows[k] >= n) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d outside [0, %d)", who, k, rows[k], n);

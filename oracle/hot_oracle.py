@@ -394,15 +394,23 @@ def abc_forward(x: np.ndarray, cfg: HotConfig):
     x <- P x (HLA along tokens) then quantise to INT8.
     Returns (xq int8 [L', I], sx fp32 [1])."""
     xp = fwht_blocks_first(np.asarray(x, dtype=F32), cfg.hla_n, np.asarray(cfg.hla_rows))
-    return quant(xp, cfg.act_bits, cfg.act_scale, cfg.act_round, cfg.seed, STREAM_ACT)
+    idx = colwise_rng_index(xp.shape[1], xp.shape[0] // len(cfg.hla_rows), cfg.hla_rows).T
+    return quant(xp, cfg.act_bits, cfg.act_scale, cfg.act_round, cfg.seed, STREAM_ACT, index=idx)
 
 
-def _untransposed_index(shape) -> np.ndarray:
-    """RNG element index of entry (c, k) of a [C, K] matrix that is the
-    transpose of a row-major [K, C] one: the kernels number the coefficients of
-    the column-wise transforms by their position k * C + c before the transpose."""
-    C, K = shape
-    return (np.arange(K, dtype=np.int64)[None, :] * C + np.arange(C, dtype=np.int64)[:, None])
+def colwise_rng_index(C: int, NB: int, rows) -> np.ndarray:
+    """RNG element index of every coefficient of a column-wise transformed
+    matrix, laid out [C, NB * r] (K-major).  The kernels walk the kept
+    coefficients of a block in increasing natural-row order and number them
+    ((c * NB + block) * rpad + visit) with rpad = r rounded up to 4, so that one
+    Philox call serves four consecutive visits of a channel."""
+    rows = np.asarray(rows)
+    r = len(rows)
+    rpad = (r + 3) // 4 * 4
+    visit = np.argsort(np.argsort(rows))                      # rank of rows[k] among the kept rows
+    c = np.arange(C, dtype=np.int64)[:, None, None]
+    b = np.arange(NB, dtype=np.int64)[None, :, None]
+    return ((c * NB + b) * rpad + visit[None, None, :].astype(np.int64)).reshape(C, NB * r)
 
 
 @dataclass
@@ -433,7 +441,8 @@ def linear_backward(g_y: np.ndarray, w: np.ndarray, xq: np.ndarray, sx: np.ndarr
     tr.qG, tr.sG = quant(G, cfg.gx_bits, cfg.gx_scale, cfg.gx_round, cfg.seed, STREAM_GX)
     # :270  blkdiag(H) W ; :276-285 quantise
     Wh = fwht_blocks_first(w, cfg.n_o)
-    tr.qW, tr.sW = quant(Wh, cfg.w_bits, cfg.w_scale, cfg.w_round, cfg.seed, STREAM_W)
+    tr.qW, tr.sW = quant(Wh, cfg.w_bits, cfg.w_scale, cfg.w_round, cfg.seed, STREAM_W,
+                         index=colwise_rng_index(Wh.shape[1], Wh.shape[0] // cfg.n_o, np.arange(cfg.n_o)).T)
     # :288-290, :343
     tr.acc_x = int_gemm_nt(tr.qG, tr.qW.T)
     sg = tr.sG.reshape(-1, 1) if cfg.gx_scale == SCALE_ROW else tr.sG.reshape(1, 1)
@@ -441,7 +450,7 @@ def linear_backward(g_y: np.ndarray, w: np.ndarray, xq: np.ndarray, sx: np.ndarr
     # :301 (P g_y)^T ; :307-320 quantise
     GpT = np.ascontiguousarray(fwht_blocks_first(g_y, cfg.hla_n, np.asarray(cfg.hla_rows)).T)
     tr.qGp, tr.sGp = quant(GpT, cfg.gw_bits, cfg.gw_scale, cfg.gw_round, cfg.seed, STREAM_GW,
-                           index=_untransposed_index(GpT.shape))
+                           index=colwise_rng_index(GpT.shape[0], GpT.shape[1] // len(cfg.hla_rows), cfg.hla_rows))
     # :322-324, :344
     tr.acc_w = int_gemm_nt(tr.qGp, np.asarray(xq).T)
     sgw = tr.sGp.reshape(-1, 1) if cfg.gw_scale == SCALE_ROW else tr.sGp.reshape(1, 1)

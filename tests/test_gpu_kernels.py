@@ -180,7 +180,7 @@ def test_hla_tokenwise_stochastic_matches_oracle(gpu, scale):
     codes, s, kout = ops.hla_tokenwise(x.to(gpu), n, list(rows), bits=8, rounding="stoch", scale=scale, seed=77)
     t = np.ascontiguousarray(orc.fwht_blocks_first(xn, n, rows).T)
     mode = orc.SCALE_ROW if scale == "row" else orc.SCALE_TENSOR
-    q_ref, s_ref = orc.quant(t, 8, mode, orc.ROUND_STOCH, 77, orc.STREAM_GW, index=orc._untransposed_index(t.shape))
+    q_ref, s_ref = orc.quant(t, 8, mode, orc.ROUND_STOCH, 77, orc.STREAM_GW, index=orc.colwise_rng_index(C, L // n, rows))
     assert np.array_equal(s.cpu().numpy(), s_ref)
     assert np.array_equal(codes.cpu().numpy()[:, :kout], q_ref)
 
