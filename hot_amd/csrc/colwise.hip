@@ -48,6 +48,28 @@ struct ColArgs {
   int8_t slot[HOT_MAX_HLA_N];  // output position of natural row i, -1 = dropped
 };
 
+// Which coefficients of a block are kept and where they go.  The generic policy reads the table
+// from the kernel arguments; the presets make it a compile-time constant, which removes the
+// per-coefficient scalar branches and lets the compiler drop the butterflies that only feed
+// discarded coefficients.
+struct SelRuntime { static constexpr bool STATIC = false; };
+template <int N> struct SelFull {
+  static constexpr bool STATIC = true;
+  static constexpr int slot(int i) { return i; }
+};
+struct SelPy64 {  // make_WHT rule for n = 64: 36 coefficients, sequency order
+  static constexpr bool STATIC = true;
+  static constexpr int8_t TABLE[64] = {0,  35, 25, 26, 14, 33, 15, 32, 7,  -1, -1, -1, -1, -1, -1, -1, 3,  -1, 22, 29, 11, -1,
+                                       18, -1, 4,  -1, 21, -1, 10, -1, 19, -1, 1,  -1, 24, 27, 13, 34, 16, 31, 6,  -1, -1, -1,
+                                       8,  -1, -1, -1, 2,  -1, 23, 28, 12, -1, 17, 30, 5,  -1, -1, -1, 9,  -1, 20, -1};
+  static constexpr int slot(int i) { return TABLE[i]; }
+};
+struct SelPaper16 {  // the 8 lowest sequencies of a 16-block
+  static constexpr bool STATIC = true;
+  static constexpr int8_t TABLE[16] = {0, -1, 7, -1, 3, -1, 4, -1, 1, -1, 6, -1, 2, -1, 5, -1};
+  static constexpr int slot(int i) { return TABLE[i]; }
+};
+
 template <typename T> struct raw_of { typedef uint16_t type; };
 template <> struct raw_of<float> { typedef uint32_t type; };
 
@@ -70,16 +92,6 @@ __device__ __forceinline__ void fwht_regs(float (&v)[LEN]) {
       }
     }
   }
-}
-
-// rint(x / d) with rcp = 1 / d precomputed: the product x * rcp is within 1.5 * 2^-23 |x/d| of
-// the correctly rounded quotient, so it rounds to the same integer unless it lies within 2^-14 of
-// a half-integer (|x/d| <= 128); only then is the IEEE division carried out.
-__device__ __forceinline__ int quant_nearest_fast(float x, float d, float rcp) {
-  const float p = x * rcp;
-  float k = rintf(p);
-  if (__builtin_expect(fabsf(p - k) > 0.5f - 6.103515625e-05f, 0)) k = rintf(x / d);
-  return (int)k;
 }
 
 // Streams the rows of the workgroup's tile through a ring of LDS buffers with
@@ -142,7 +154,7 @@ __device__ __forceinline__ void rs_column(const uint8_t* buf, int tid, float* v)
 
 // ---- the kernel: PASS 0 = statistics, PASS 1 = quantise + transposed store ----
 
-template <typename T, int N, int PASS, int ROUND, bool SAWB>
+template <typename T, int N, int PASS, int ROUND, bool SAWB, typename SEL>
 __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   constexpr int SPB = N >= CW_ROWS ? N / CW_ROWS : 1;        // steps per token block
   constexpr int BPS = N >= CW_ROWS ? 1 : CW_ROWS / N;        // token blocks per step
@@ -204,7 +216,8 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
         float u[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < N; ++i) {
-          const int sl = a.slot[i];
+          int sl;
+          if constexpr (SEL::STATIC) sl = SEL::slot(i); else sl = a.slot[i];
           if (sl >= 0) {
             float v = x[g * N + i];
             if constexpr (PASS == 0) {
@@ -214,7 +227,9 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
               if constexpr (SAWB) v = fminf(fmaxf(v, -clip), clip);
               int q;
               if constexpr (ROUND == HOT_ROUND_NEAREST) {
-                q = quant_nearest_fast(v, d, rcp);
+                // |v / d| <= qmax (1 + 2^-22) by construction of d (absmax) or of the clip (SAWB):
+                // the rounded code cannot leave [-qmax, qmax]
+                q = (int)rint_div_fast(v, d, rcp);
               } else {
                 // counter = ((channel * NB + block) * rpad + visit index) / 4, word = visit index % 4
                 if ((visited & 3) == 0) {
@@ -225,8 +240,8 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
                 const int w = visited & 3;
                 q = q_stoch(v / d, w == 0 ? u[0] : w == 1 ? u[1] : w == 2 ? u[2] : u[3]);
                 ++visited;
+                q = clampi(q, -qmax, qmax);   // floor + 1 may step past qmax at the very top
               }
-              q = clampi(q, -qmax, qmax);
               stage[tid * pitch + blk * a.r + sl] = (uint8_t)(q & 0xFF);
             }
           }
@@ -300,25 +315,24 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     const int ndw = (int)((seg_end - seg0) / 4);            // output dwords per channel
     const int sdw = out_sb / 4;                             // of which staged
     const int nch = (int)((a.C - cg0) < CW ? (a.C - cg0) : CW);
-    // a wave walks along K of one channel: contiguous bytes of one output row per store
-    for (int ch = wave; ch < nch; ch += CW / 64) {
+    // consecutive threads walk along K within a channel, then on to the next channel
+    const int total = nch * ndw;
+    for (int p = tid; p < total; p += CW) {
+      const int ch = p / ndw, jd = p - ch * ndw;
       const uint32_t* row = reinterpret_cast<const uint32_t*>(stage + ch * pitch);
-      uint32_t* orow = reinterpret_cast<uint32_t*>(a.out + (cg0 + ch) * a.ld_out + seg0);
-      for (int jd = lane; jd < ndw; jd += 64) {
-        uint32_t w = 0u;
-        if (jd < sdw) {
-          if (a.store4) {
-            const uint32_t lo = row[2 * jd], hi = row[2 * jd + 1];
-            // bytes b0..b7 -> nibbles: byte j of the result = (b[2j+1] << 4) | (b[2j] & 15)
-            const uint32_t l = (lo & 0x0F) | ((lo >> 4) & 0xF0) | ((lo >> 8) & 0x0F00) | ((lo >> 12) & 0xF000);
-            const uint32_t h = (hi & 0x0F) | ((hi >> 4) & 0xF0) | ((hi >> 8) & 0x0F00) | ((hi >> 12) & 0xF000);
-            w = (l & 0xFFFF) | (h << 16);
-          } else {
-            w = row[jd];
-          }
+      uint32_t w = 0u;
+      if (jd < sdw) {
+        if (a.store4) {
+          const uint32_t lo = row[2 * jd], hi = row[2 * jd + 1];
+          // bytes b0..b7 -> nibbles: byte j of the result = (b[2j+1] << 4) | (b[2j] & 15)
+          const uint32_t l = (lo & 0x0F) | ((lo >> 4) & 0xF0) | ((lo >> 8) & 0x0F00) | ((lo >> 12) & 0xF000);
+          const uint32_t h = (hi & 0x0F) | ((hi >> 4) & 0xF0) | ((hi >> 8) & 0x0F00) | ((hi >> 12) & 0xF000);
+          w = (l & 0xFFFF) | (h << 16);
+        } else {
+          w = row[jd];
         }
-        orow[jd] = w;
       }
+      *reinterpret_cast<uint32_t*>(a.out + (cg0 + ch) * a.ld_out + seg0 + (int64_t)jd * 4) = w;
     }
   }
 }
@@ -376,26 +390,30 @@ size_t colwise_workspace_bytes_impl(int64_t C) {
   return COL_STAT_BYTES + (size_t)round_up(C * 4, 256) + (size_t)(2 * sizeof(double)) * 65536;
 }
 
-template <typename T, int N, int PASS, int ROUND, bool SAWB>
+template <typename T, int N, int PASS, int ROUND, bool SAWB, typename SEL>
 static int launch_pass(const ColArgs& a, dim3 grid, size_t lds, hipStream_t st) {
   static bool attr_done = false;  // one-time, read-only afterwards
   if (!attr_done && lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&colwise_kernel<T, N, PASS, ROUND, SAWB>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&colwise_kernel<T, N, PASS, ROUND, SAWB, SEL>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
     if (e != hipSuccess) return check_hip(e, "hipFuncSetAttribute(colwise_kernel)");
     attr_done = true;
   }
-  hipLaunchKernelGGL((colwise_kernel<T, N, PASS, ROUND, SAWB>), grid, dim3(CW), lds, st, a);
+  hipLaunchKernelGGL((colwise_kernel<T, N, PASS, ROUND, SAWB, SEL>), grid, dim3(CW), lds, st, a);
   return HOT_OK;
 }
 
-template <typename T, int N>
+template <typename T, int N, typename SEL>
 static int launch_colwise(ColArgs& a, hipStream_t st) {
   constexpr int BPS = N >= CW_ROWS ? 1 : CW_ROWS / N;
-  // token blocks per workgroup: a staged run of at least 128 code bytes per channel, a multiple of 4
-  // bytes (dword flush) and of the blocks that share a 16-row step
-  int tb = 4 > BPS ? 4 : BPS;
-  while (tb * a.r < 128) tb <<= 1;
+  // Token blocks per workgroup.  The staged run of a channel (tb * r codes) must be a whole number
+  // of output dwords and cover the blocks that share a 16-row step; beyond that, longer runs (up
+  // to 128 bytes) are taken only while they leave at least four workgroups per CU.
+  const int64_t gx0 = (a.C + CW - 1) / CW;
+  const int out_bytes_per_block = a.store4 ? a.r / 2 : a.r;   // r is even when store4
+  int tb = BPS;
+  while ((tb * a.r) % (a.store4 ? 8 : 4) != 0 || tb * out_bytes_per_block < 32) tb <<= 1;
+  while (tb * out_bytes_per_block < 128 && gx0 * ((a.NB + 2 * tb - 1) / (2 * tb)) >= 1024) tb <<= 1;
   a.tb = tb;
   const size_t in_bytes = (size_t)CW_DEPTH * CW_ROWS * CW * sizeof(T);
   const size_t lds_stats = in_bytes, lds_quant = in_bytes + (size_t)CW * (tb * a.r + 4);
@@ -407,31 +425,46 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   hipLaunchKernelGGL(colwise_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat,
                      a.mode == HOT_SCALE_ROW ? a.colmax : (float*)nullptr, a.C);
   int rc;
-  if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 0, 0, true>(a, grid, lds_stats, st);
-  else rc = launch_pass<T, N, 0, 0, false>(a, grid, lds_stats, st);
+  if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 0, 0, true, SEL>(a, grid, lds_stats, st);
+  else rc = launch_pass<T, N, 0, 0, false, SEL>(a, grid, lds_stats, st);
   if (rc) return rc;
   hipLaunchKernelGGL(colwise_finalize_kernel, dim3(1), dim3(256), 0, st, a, gx * gy);
   if (a.rounding == HOT_ROUND_STOCH) {
-    if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 1, 1, true>(a, grid, lds_quant, st);
-    else rc = launch_pass<T, N, 1, 1, false>(a, grid, lds_quant, st);
+    if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 1, 1, true, SEL>(a, grid, lds_quant, st);
+    else rc = launch_pass<T, N, 1, 1, false, SEL>(a, grid, lds_quant, st);
   } else {
-    if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 1, 0, true>(a, grid, lds_quant, st);
-    else rc = launch_pass<T, N, 1, 0, false>(a, grid, lds_quant, st);
+    if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 1, 0, true, SEL>(a, grid, lds_quant, st);
+    else rc = launch_pass<T, N, 1, 0, false, SEL>(a, grid, lds_quant, st);
   }
   if (rc) return rc;
   return check_launch("colwise_kernel");
 }
 
+template <typename SEL, int N>
+static bool matches(const ColArgs& a) {
+  for (int i = 0; i < N; ++i)
+    if (a.slot[i] != SEL::slot(i)) return false;
+  return true;
+}
+
 template <typename T>
 static int dispatch_colwise_n(int n, ColArgs& a, hipStream_t st) {
   switch (n) {
-    case 1: return launch_colwise<T, 1>(a, st);
-    case 2: return launch_colwise<T, 2>(a, st);
-    case 4: return launch_colwise<T, 4>(a, st);
-    case 8: return launch_colwise<T, 8>(a, st);
-    case 16: return launch_colwise<T, 16>(a, st);
-    case 32: return launch_colwise<T, 32>(a, st);
-    case 64: return launch_colwise<T, 64>(a, st);
+    case 1: return launch_colwise<T, 1, SelFull<1>>(a, st);   // r = 1 is the only choice
+    case 2: return launch_colwise<T, 2, SelRuntime>(a, st);
+    case 4: return launch_colwise<T, 4, SelRuntime>(a, st);
+    case 8: return launch_colwise<T, 8, SelRuntime>(a, st);
+    case 16:
+      if (a.r == 16 && matches<SelFull<16>, 16>(a)) return launch_colwise<T, 16, SelFull<16>>(a, st);
+      if (a.r == 8 && matches<SelPaper16, 16>(a)) return launch_colwise<T, 16, SelPaper16>(a, st);
+      return launch_colwise<T, 16, SelRuntime>(a, st);
+    case 32:
+      if (a.r == 32 && matches<SelFull<32>, 32>(a)) return launch_colwise<T, 32, SelFull<32>>(a, st);
+      return launch_colwise<T, 32, SelRuntime>(a, st);
+    case 64:
+      if (a.r == 36 && matches<SelPy64, 64>(a)) return launch_colwise<T, 64, SelPy64>(a, st);
+      if (a.r == 64 && matches<SelFull<64>, 64>(a)) return launch_colwise<T, 64, SelFull<64>>(a, st);
+      return launch_colwise<T, 64, SelRuntime>(a, st);
     default: return fail(HOT_ERR_UNSUPPORTED, "colwise: block size %d (power of two up to %d)", n, HOT_MAX_HLA_N);
   }
 }

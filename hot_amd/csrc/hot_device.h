@@ -160,9 +160,21 @@ __device__ __forceinline__ int q_stoch(float y, float u) {
 __device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
 
 // non-negative float max through an integer atomic (bit patterns of
-// non-negative floats are ordered like unsigned integers)
+// non-negative floats are ordered like unsigned integers).  The plain read
+// first keeps thousands of workgroups from queueing on one address: the value
+// only grows, so a stale read can at worst cause a redundant atomic.
 __device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) {
-  atomicMax(reinterpret_cast<unsigned int*>(addr), as_u(v));
+  if (v > *reinterpret_cast<volatile float*>(addr)) atomicMax(reinterpret_cast<unsigned int*>(addr), as_u(v));
+}
+
+// rint(x / d) with rcp = 1 / d precomputed: the product x * rcp is within 1.5 * 2^-23 |x/d| of
+// the correctly rounded quotient, so it rounds to the same integer unless it lies within 2^-14 of
+// a half-integer (|x/d| <= 128); only then is the IEEE division carried out.
+__device__ __forceinline__ float rint_div_fast(float x, float d, float rcp) {
+  const float p = x * rcp;
+  float k = rintf(p);
+  if (__builtin_expect(fabsf(p - k) > 0.5f - 6.103515625e-05f, 0)) k = rintf(x / d);
+  return k;
 }
 
 }  // namespace hot

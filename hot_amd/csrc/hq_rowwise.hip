@@ -68,13 +68,14 @@ __device__ __forceinline__ void fwht_lanes(float* x, int lane) {
 }
 
 template <int BITS, int ROUND>
-__device__ __forceinline__ void quant_store_chunk(const float* x, float d, uint64_t e0, uint64_t seed,
+__device__ __forceinline__ void quant_store_chunk(const float* x, float d, float rcp, uint64_t e0, uint64_t seed,
                                                   uint32_t stream, int8_t* out_row_chunk) {
   constexpr int QMAX = (1 << (BITS - 1)) - 1;
   int q[EPL];
   if constexpr (ROUND == 0) {
+    // |x / d| <= qmax (1 + 2^-22) because d comes from the absmax: no clamp needed
 #pragma unroll
-    for (int j = 0; j < EPL; ++j) q[j] = clampi(q_nearest(x[j] / d), -QMAX, QMAX);
+    for (int j = 0; j < EPL; ++j) q[j] = (int)rint_div_fast(x[j], d, rcp);
   } else {
     float u[EPL];
     sr_uniform4(e0 >> 2, seed, stream, u);
@@ -141,6 +142,7 @@ __global__ void hq_row_kernel(const T* __restrict__ in, int64_t K, int8_t* __res
   constexpr float QMAXF = (float)((1 << (BITS - 1)) - 1);
   const float s = mx / QMAXF;
   const float d = s + 1e-11f;
+  const float rcp = 1.0f / d;
   if (tid == 0) scales[row] = s;
 
   int8_t* orow = codes + row * ld;
@@ -148,7 +150,7 @@ __global__ void hq_row_kernel(const T* __restrict__ in, int64_t K, int8_t* __res
   for (int c = 0; c < C; ++c) {
     const int ch = tid + c * team;
     if (ch < nch) {
-      quant_store_chunk<BITS, ROUND>(x[c], d, (uint64_t)row * (uint64_t)K + (uint64_t)ch * EPL, seed,
+      quant_store_chunk<BITS, ROUND>(x[c], d, rcp, (uint64_t)row * (uint64_t)K + (uint64_t)ch * EPL, seed,
                                      stream, orow + (int64_t)ch * (EPL * BITS / 8));
     }
   }
@@ -189,6 +191,7 @@ __global__ void hq_tensor_kernel(const T* __restrict__ in, int64_t nchunks, int6
   constexpr float QMAXF = (float)((1 << (BITS - 1)) - 1);
   const float s = *absmax / QMAXF;
   const float d = s + 1e-11f;
+  const float rcp = 1.0f / d;
   if (blockIdx.x == 0 && threadIdx.x == 0) *scale_out = s;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t ch = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ch < nchunks; ch += stride) {
@@ -200,7 +203,7 @@ __global__ void hq_tensor_kernel(const T* __restrict__ in, int64_t nchunks, int6
       const int64_t row = ch / nch_row;
       off = row * ld + (ch - row * nch_row) * (EPL * BITS / 8);
     }
-    quant_store_chunk<BITS, ROUND>(x, d, (uint64_t)ch * EPL, seed, stream, codes + off);
+    quant_store_chunk<BITS, ROUND>(x, d, rcp, (uint64_t)ch * EPL, seed, stream, codes + off);
   }
 }
 
