@@ -205,7 +205,6 @@ gemm_i8_kernel(const GemmArgs g) {
 // DMA are explicit (vmcnt) and the barrier carries no fence.
 // ---------------------------------------------------------------------------
 
-constexpr int P_STAGES = 4;
 constexpr int P_ROWB = 64;  // bytes per row per stage
 
 // s_waitcnt vmcnt(VM) alone (expcnt and lgkmcnt untouched); vmcnt is split over bits 3:0 and 15:14
@@ -231,9 +230,10 @@ __device__ __forceinline__ uint32_t lds_offset(const uint8_t* p) {
   return (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t*)p;
 }
 
-template <int WM, int WN, int BITS, typename OutT>
-__global__ void __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(1, (WM * WN <= 4 ? 2 : 1))))
+template <int WM, int WN, int BITS, int S, typename OutT>
+__global__ void __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(1, (WM * WN <= 4 ? (S == 3 ? 3 : 2) : 1))))
 gemm_i8_pipe_kernel(const GemmArgs g) {
+  static_assert(S == 3 || S == 4, "three or four LDS stages");
   constexpr int BM = 64 * WM, BN = 64 * WN;
   constexpr int STAGE_BYTES = (BM + BN) * P_ROWB;
   constexpr int LPW = (BM + BN) / 64;           // DMA instructions per wave per stage (KiB chunks / 4 waves)
@@ -241,7 +241,7 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
   __shared__ __attribute__((aligned(1024))) uint8_t st0[STAGE_BYTES];
   __shared__ __attribute__((aligned(1024))) uint8_t st1[STAGE_BYTES];
   __shared__ __attribute__((aligned(1024))) uint8_t st2[STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t st3[STAGE_BYTES];
+  __shared__ __attribute__((aligned(1024))) uint8_t st3[S == 4 ? STAGE_BYTES : 1024];
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -335,17 +335,17 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
   };
 
   const int KT = g.ktiles * (G_BK / (BITS == 8 ? 64 : 128));   // stages of this kernel per G_BK-code tile
-  // prologue: up to three tiles in flight, tile 0 landed and visible, its first round in registers
+  // prologue: S - 1 tiles in flight, tile 0 landed and visible, its first round in registers
   issue(st0, 0);
   if (KT > 1) issue(st1, 1);
-  if (KT > 2) issue(st2, 2);
-  if (KT > 2) wait_dma<2 * LPW>(); else if (KT > 1) wait_dma<LPW>(); else wait_dma<0>();
+  if (S == 4 && KT > 2) issue(st2, 2);
+  if (S == 4 && KT > 2) wait_dma<2 * LPW>(); else if (KT > 1) wait_dma<LPW>(); else wait_dma<0>();
   __builtin_amdgcn_s_barrier();
   v4i a0[WM], b0[WN];
   read_round(st0, 0, a0, b0);
 
   // One K-tile.  `cur` holds tile kt, `nxt` tile kt+1 (in flight or landed), `fre` held tile kt-1
-  // and receives tile kt+3.  The barrier sits in the middle of the tile, behind a block of MFMAs,
+  // and receives tile kt+S-1.  The barrier sits in the middle of the tile, behind a block of MFMAs,
   // and the first fragments of tile kt+1 are fetched before the last MFMA block of tile kt starts,
   // so the matrix pipe keeps running across the tile boundary.
   auto ktile = [&](auto steady, const uint8_t* cur, const uint8_t* nxt, const uint8_t* fre, int kt) {
@@ -358,14 +358,14 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (decltype(steady)::value) {
       // steady state (kt + 3 < KT): straight-line code, so the compiler's LDS wait counts are exact
-      wait_dma<LPW>();                                        // this wave's share of tile kt+1 has landed
+      wait_dma<(S - 3) * LPW>();                              // this wave's share of tile kt+1 has landed
       __builtin_amdgcn_s_barrier();                           // ... and everybody's; nobody reads tile kt-1 any more
-      issue(fre, kt + 3);
+      issue(fre, kt + S - 1);
       read_round(nxt, 0, a0, b0);
     } else if (kt + 1 < KT) {
-      if (kt + 2 < KT) wait_dma<LPW>(); else wait_dma<0>();
+      if (S == 4 && kt + 2 < KT) wait_dma<LPW>(); else wait_dma<0>();
       __builtin_amdgcn_s_barrier();
-      if (kt + 3 < KT) issue(fre, kt + 3);
+      if (kt + S - 1 < KT) issue(fre, kt + S - 1);
       read_round(nxt, 0, a0, b0);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -373,17 +373,30 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
     __builtin_amdgcn_sched_barrier(0);
   };
   int kt0 = 0;
-  for (; kt0 + 6 < KT; kt0 += P_STAGES) {
-    ktile(std::true_type{}, st0, st1, st3, kt0);
-    ktile(std::true_type{}, st1, st2, st0, kt0 + 1);
-    ktile(std::true_type{}, st2, st3, st1, kt0 + 2);
-    ktile(std::true_type{}, st3, st0, st2, kt0 + 3);
-  }
-  for (; kt0 < KT; kt0 += P_STAGES) {
-    ktile(std::false_type{}, st0, st1, st3, kt0);
-    if (kt0 + 1 < KT) ktile(std::false_type{}, st1, st2, st0, kt0 + 1);
-    if (kt0 + 2 < KT) ktile(std::false_type{}, st2, st3, st1, kt0 + 2);
-    if (kt0 + 3 < KT) ktile(std::false_type{}, st3, st0, st2, kt0 + 3);
+  if constexpr (S == 4) {
+    for (; kt0 + 6 < KT; kt0 += 4) {
+      ktile(std::true_type{}, st0, st1, st3, kt0);
+      ktile(std::true_type{}, st1, st2, st0, kt0 + 1);
+      ktile(std::true_type{}, st2, st3, st1, kt0 + 2);
+      ktile(std::true_type{}, st3, st0, st2, kt0 + 3);
+    }
+    for (; kt0 < KT; kt0 += 4) {
+      ktile(std::false_type{}, st0, st1, st3, kt0);
+      if (kt0 + 1 < KT) ktile(std::false_type{}, st1, st2, st0, kt0 + 1);
+      if (kt0 + 2 < KT) ktile(std::false_type{}, st2, st3, st1, kt0 + 2);
+      if (kt0 + 3 < KT) ktile(std::false_type{}, st3, st0, st2, kt0 + 3);
+    }
+  } else {
+    for (; kt0 + 4 < KT; kt0 += 3) {
+      ktile(std::true_type{}, st0, st1, st2, kt0);
+      ktile(std::true_type{}, st1, st2, st0, kt0 + 1);
+      ktile(std::true_type{}, st2, st0, st1, kt0 + 2);
+    }
+    for (; kt0 < KT; kt0 += 3) {
+      ktile(std::false_type{}, st0, st1, st2, kt0);
+      if (kt0 + 1 < KT) ktile(std::false_type{}, st1, st2, st0, kt0 + 1);
+      if (kt0 + 2 < KT) ktile(std::false_type{}, st2, st0, st1, kt0 + 2);
+    }
   }
 
   const float sb = g.scale_b[0];
@@ -410,7 +423,7 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
   }
 }
 
-template <int WM, int WN, int BITS, typename OutT>
+template <int WM, int WN, int BITS, int S, typename OutT>
 static int launch_gemm_pipe(GemmArgs& g, hipStream_t st) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
   g.tiles_m = (int)((g.M + BM - 1) / BM);
@@ -418,7 +431,7 @@ static int launch_gemm_pipe(GemmArgs& g, hipStream_t st) {
   const int64_t total = (int64_t)g.tiles_m * g.tiles_n;
   if (total > (1 << 30)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: too many tiles");
   if (g.M * g.lda >= (1ll << 32) || g.N * g.ldb >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: operand larger than 4 GiB");
-  hipLaunchKernelGGL((gemm_i8_pipe_kernel<WM, WN, BITS, OutT>), dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
+  hipLaunchKernelGGL((gemm_i8_pipe_kernel<WM, WN, BITS, S, OutT>), dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
   return check_launch("gemm_i8_pipe_kernel");
 }
 
@@ -446,19 +459,25 @@ static int pick_tile(GemmArgs& g, hipStream_t st) {
   static int forced = -1;
   if (forced < 0) { const char* e = getenv("HOT_GEMM_TILE"); forced = e ? atoi(e) : 0; }
   switch (forced) {
-    case 144: return launch_gemm_pipe<4, 4, BITS, OutT>(g, st);
-    case 142: return launch_gemm_pipe<4, 2, BITS, OutT>(g, st);
-    case 124: return launch_gemm_pipe<2, 4, BITS, OutT>(g, st);
-    case 122: return launch_gemm_pipe<2, 2, BITS, OutT>(g, st);
+    case 144: return launch_gemm_pipe<4, 4, BITS, 4, OutT>(g, st);
+    case 142: return launch_gemm_pipe<4, 2, BITS, 4, OutT>(g, st);
+    case 124: return launch_gemm_pipe<2, 4, BITS, 4, OutT>(g, st);
+    case 122: return launch_gemm_pipe<2, 2, BITS, 4, OutT>(g, st);
+    case 322: return launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st);
     case 44: return launch_gemm<4, 4, BITS, OutT>(g, st);
     case 42: return launch_gemm<4, 2, BITS, OutT>(g, st);
     case 24: return launch_gemm<2, 4, BITS, OutT>(g, st);
     case 22: return launch_gemm<2, 2, BITS, OutT>(g, st);
     default: break;
   }
-  // 128 x 128 tiles, two workgroups per CU: best on every graded shape so far.  The DMA kernel
-  // addresses operands with 32-bit offsets; larger operands take the register-staged kernel.
-  if (g.M * g.lda < (1ll << 32) && g.N * g.ldb < (1ll << 32)) return launch_gemm_pipe<2, 2, BITS, OutT>(g, st);
+  // 128 x 128 tiles.  With more tiles than CUs, three LDS stages let three workgroups share a CU
+  // and hide each other's stalls; with fewer, a lone workgroup per CU prefers the deeper prefetch of
+  // four stages.  The DMA kernel addresses operands with 32-bit offsets; larger operands take the
+  // register-staged kernel.
+  if (g.M * g.lda < (1ll << 32) && g.N * g.ldb < (1ll << 32)) {
+    const int64_t tiles = ((g.M + 127) / 128) * ((g.N + 127) / 128);
+    return tiles > 256 ? launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st) : launch_gemm_pipe<2, 2, BITS, 4, OutT>(g, st);
+  }
   return launch_gemm<2, 2, BITS, OutT>(g, st);
 }
 
