@@ -171,14 +171,21 @@ int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq
     (void)hipEventRecord(ev[0], st);
   }
   int rc;
-  // g_y: Hadamard along O + quantise (g_x operand); HLA along tokens + quantise, transposed (g_W operand)
-  rc = hq_rowwise_impl(gy, dtype, L, O, cfg->n_o, cfg->gx_bits, cfg->gx_round, cfg->seed, HOT_STREAM_GX,
-                       cfg->gx_scale, ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, 256, st);
-  if (rc) goto done;
-  rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->gw_bits, cfg->gw_round,
-                          cfg->seed, HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp,
-                          ws + b.off_colg, colwise_workspace_bytes_impl(O), st, who);
-  if (rc) goto done;
+  // g_y: HLA along tokens + quantise, transposed (g_W operand); Hadamard along O + quantise (g_x
+  // operand).  With one step per tensor both quantisers need the absmax of their transform first:
+  // the statistics pass of the token-wise kernel delivers both from a single read of g_y.
+  {
+    const bool fuse = cfg->gx_scale == HOT_SCALE_TENSOR && cfg->n_o == 16 && O % 16 == 0 &&
+                      cfg->gw_scale != HOT_SCALE_SAWB;
+    rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->gw_bits, cfg->gw_round,
+                            cfg->seed, HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp,
+                            ws + b.off_colg, colwise_workspace_bytes_impl(O), st, who,
+                            fuse ? (float*)(ws + b.off_hq) : nullptr);
+    if (rc) goto done;
+    rc = hq_rowwise_impl(gy, dtype, L, O, cfg->n_o, cfg->gx_bits, cfg->gx_round, cfg->seed, HOT_STREAM_GX,
+                         cfg->gx_scale, ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, 256, st, fuse);
+    if (rc) goto done;
+  }
   if (times4) (void)hipEventRecord(ev[1], st);
   // W: Hadamard along O + quantise, stored [I, O]
   rc = colwise_quant_impl(w, dtype, O, I, cfg->n_o, identity_rows(), cfg->n_o, cfg->w_bits, cfg->w_round, cfg->seed,

@@ -42,6 +42,7 @@ struct ColArgs {
   double* partial;    // SAWB: 2 doubles per workgroup
   float* colmax;      // ROW: per-channel absmax
   float* scales_out;
+  float* row_absmax;  // statistics pass with RS != 0: absmax of the row-wise block Hadamard
   uint64_t seed;
   uint32_t stream;
   int32_t r, rpad, bits, store4, rounding, mode, tb;
@@ -154,7 +155,11 @@ __device__ __forceinline__ void rs_column(const uint8_t* buf, int tid, float* v)
 
 // ---- the kernel: PASS 0 = statistics, PASS 1 = quantise + transposed store ----
 
-template <typename T, int N, int PASS, int ROUND, bool SAWB, typename SEL>
+// RS (statistics pass only): when non-zero the pass also tracks the absmax of the ROW-wise block
+// Hadamard (block RS along the channels) of the same input, so that the row-wise quantiser of g_y
+// needs no statistics pass of its own.  Adjacent lanes hold adjacent channels, hence the row-wise
+// butterflies run across lanes.
+template <typename T, int N, int PASS, int ROUND, bool SAWB, typename SEL, int RS = 0>
 __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   constexpr int SPB = N >= CW_ROWS ? N / CW_ROWS : 1;        // steps per token block
   constexpr int BPS = N >= CW_ROWS ? 1 : CW_ROWS / N;        // token blocks per step
@@ -201,7 +206,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     rcp = 1.0f / d;
   }
 
-  float cmax = 0.f;
+  float cmax = 0.f, rmax = 0.f;
   double ssq = 0.0, sab = 0.0;
   float x[XL];
 
@@ -263,6 +268,20 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     __builtin_amdgcn_s_barrier();   // ... and so for every wave: the buffer of step s-1 may be refilled
     if (s + CW_DEPTH - 1 < nsteps) rs_issue<T>(rs, lds0 + ((s + CW_DEPTH - 1) % CW_DEPTH) * BUF, s + CW_DEPTH - 1, wave, lane);
     rs_column<T>(lds + (s % CW_DEPTH) * BUF, tid, dst);
+    if constexpr (PASS == 0 && RS != 0) {
+#pragma unroll
+      for (int i = 0; i < CW_ROWS; ++i) {
+        float t = dst[i];
+        // lower lane: own + partner ; upper lane: partner - own == partner + (-own)
+        t = as_f(as_u(t) ^ ((lane & 1) ? 0x80000000u : 0u)) + lane_xor<1>(t);
+        t = as_f(as_u(t) ^ ((lane & 2) ? 0x80000000u : 0u)) + lane_xor<2>(t);
+        t = as_f(as_u(t) ^ ((lane & 4) ? 0x80000000u : 0u)) + lane_xor<4>(t);
+        t = as_f(as_u(t) ^ ((lane & 8) ? 0x80000000u : 0u)) + lane_xor<8>(t);
+        if constexpr (RS >= 32) t = as_f(as_u(t) ^ ((lane & 16) ? 0x80000000u : 0u)) + lane_xor<16>(t);
+        if constexpr (RS >= 64) t = as_f(as_u(t) ^ ((lane & 32) ? 0x80000000u : 0u)) + lane_xor<32>(t);
+        rmax = fmaxf(rmax, fabsf(t));
+      }
+    }
   };
   if constexpr (N >= CW_ROWS) {
     for (int bl = 0; bl < nblk; ++bl) {
@@ -278,6 +297,19 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   }
 
   if constexpr (PASS == 0) {
+    if constexpr (RS != 0) {
+      // rows past the end of the input were redirected to real rows and channels past C form whole
+      // inactive blocks, so only the latter need masking
+      float m = wave_max(active ? rmax : 0.f);
+      if (lane == 0) s_max[wave] = m;
+      __syncthreads();
+      if (tid == 0) {
+        float mm = s_max[0];
+        for (int i = 1; i < CW / 64; ++i) mm = fmaxf(mm, s_max[i]);
+        atomic_max_nonneg(a.row_absmax, mm);
+      }
+      __syncthreads();
+    }
     if (a.mode == HOT_SCALE_ROW) {
       if (active) atomic_max_nonneg(a.colmax + c, cmax);
       return;
@@ -375,9 +407,10 @@ __global__ void __launch_bounds__(256) colwise_finalize_kernel(const ColArgs a, 
   }
 }
 
-__global__ void colwise_clear_kernel(float* stat, float* colmax, int64_t C) {
+__global__ void colwise_clear_kernel(float* stat, float* colmax, int64_t C, float* row_absmax) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < 4) stat[i] = 0.f;
+  if (i == 0 && row_absmax) *row_absmax = 0.f;
   if (colmax && i < C) colmax[i] = 0.f;
 }
 
@@ -390,16 +423,16 @@ size_t colwise_workspace_bytes_impl(int64_t C) {
   return COL_STAT_BYTES + (size_t)round_up(C * 4, 256) + (size_t)(2 * sizeof(double)) * 65536;
 }
 
-template <typename T, int N, int PASS, int ROUND, bool SAWB, typename SEL>
+template <typename T, int N, int PASS, int ROUND, bool SAWB, typename SEL, int RS = 0>
 static int launch_pass(const ColArgs& a, dim3 grid, size_t lds, hipStream_t st) {
   static bool attr_done = false;  // one-time, read-only afterwards
   if (!attr_done && lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&colwise_kernel<T, N, PASS, ROUND, SAWB, SEL>),
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&colwise_kernel<T, N, PASS, ROUND, SAWB, SEL, RS>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
     if (e != hipSuccess) return check_hip(e, "hipFuncSetAttribute(colwise_kernel)");
     attr_done = true;
   }
-  hipLaunchKernelGGL((colwise_kernel<T, N, PASS, ROUND, SAWB, SEL>), grid, dim3(CW), lds, st, a);
+  hipLaunchKernelGGL((colwise_kernel<T, N, PASS, ROUND, SAWB, SEL, RS>), grid, dim3(CW), lds, st, a);
   return HOT_OK;
 }
 
@@ -423,9 +456,10 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   const dim3 grid((unsigned)gx, (unsigned)gy);
   const int64_t nclr = a.C > 4 ? a.C : 4;
   hipLaunchKernelGGL(colwise_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat,
-                     a.mode == HOT_SCALE_ROW ? a.colmax : (float*)nullptr, a.C);
+                     a.mode == HOT_SCALE_ROW ? a.colmax : (float*)nullptr, a.C, a.row_absmax);
   int rc;
   if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 0, 0, true, SEL>(a, grid, lds_stats, st);
+  else if (a.row_absmax) rc = launch_pass<T, N, 0, 0, false, SEL, 16>(a, grid, lds_stats, st);
   else rc = launch_pass<T, N, 0, 0, false, SEL>(a, grid, lds_stats, st);
   if (rc) return rc;
   hipLaunchKernelGGL(colwise_finalize_kernel, dim3(1), dim3(256), 0, st, a, gx * gy);
@@ -472,7 +506,7 @@ static int dispatch_colwise_n(int n, ColArgs& a, hipStream_t st) {
 int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r,
                        int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
                        void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,
-                       size_t workspace_bytes, hipStream_t st, const char* who) {
+                       size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out) {
   if (!in || !codes_out || !scales_out || !rows) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
   if (R <= 0 || C <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape R=%lld C=%lld", who, (long long)R, (long long)C);
   if (n < 1 || n > HOT_MAX_HLA_N || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (power of two up to %d)", who, n, HOT_MAX_HLA_N);
@@ -507,6 +541,9 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   a.colmax = (float*)(ws + COL_STAT_BYTES);
   a.partial = (double*)(ws + COL_STAT_BYTES + round_up(C * 4, 256));
   a.scales_out = scales_out;
+  // the fused row-wise statistic exists for block 16 and absmax steps, and needs whole 16-blocks of channels
+  a.row_absmax = (row16_absmax_out && scale_mode != HOT_SCALE_SAWB && C % 16 == 0) ? row16_absmax_out : nullptr;
+  if (row16_absmax_out && !a.row_absmax) return fail(HOT_ERR_UNSUPPORTED, "%s: fused row statistic unavailable for this configuration", who);
   switch (dtype) {
     case HOT_F32: return dispatch_colwise_n<float>(n, a, st);
     case HOT_BF16: return dispatch_colwise_n<bf16_t>(n, a, st);

@@ -24,12 +24,13 @@ constexpr int64_t GEMM_KTILE = 128;  // codes per K-tile of the int8 GEMM
 
 int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, int rounding,
                     uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_codes,
-                    float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st);
+                    float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st,
+                    bool absmax_ready = false);
 
 int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r,
                        int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
                        void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,
-                       size_t workspace_bytes, hipStream_t st, const char* who);
+                       size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out = nullptr);
 size_t colwise_workspace_bytes_impl(int64_t C);
 
 int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bits, int64_t M, int64_t N,

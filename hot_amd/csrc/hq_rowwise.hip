@@ -249,15 +249,17 @@ static int launch_row(const void* in, int64_t M, int64_t K, void* codes, int64_t
 
 template <typename T, int N, int BITS, int ROUND>
 static int launch_tensor(const void* in, int64_t M, int64_t K, void* codes, int64_t ld, float* scales, float* absmax,
-                         uint64_t seed, uint32_t stream_id, hipStream_t st) {
+                         uint64_t seed, uint32_t stream_id, hipStream_t st, bool absmax_ready) {
   const int64_t nch = M * K / EPL;
   const int block = 256;
   int64_t blocks = (nch + block - 1) / block;
   const int64_t cap = 256 * 16;  // 16 workgroups per CU, grid-stride beyond
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
-  hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, (uint32_t*)absmax, 0u, 1);
-  hipLaunchKernelGGL((hq_absmax_kernel<T, N>), dim3((unsigned)blocks), dim3(block), 0, st, (const T*)in, nch, absmax);
+  if (!absmax_ready) {
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, (uint32_t*)absmax, 0u, 1);
+    hipLaunchKernelGGL((hq_absmax_kernel<T, N>), dim3((unsigned)blocks), dim3(block), 0, st, (const T*)in, nch, absmax);
+  }
   hipLaunchKernelGGL((hq_tensor_kernel<T, N, BITS, ROUND>), dim3((unsigned)blocks), dim3(block), 0, st,
                      (const T*)in, nch, K / EPL, ld, absmax, (int8_t*)codes, scales, seed, stream_id);
   return check_launch("hq_tensor_kernel");
@@ -265,44 +267,44 @@ static int launch_tensor(const void* in, int64_t M, int64_t K, void* codes, int6
 
 template <typename T, int N, int BITS, int ROUND>
 static int dispatch_mode(int scale_mode, const void* in, int64_t M, int64_t K, void* codes, int64_t ld, float* scales,
-                         float* absmax, uint64_t seed, uint32_t stream_id, hipStream_t st) {
+                         float* absmax, uint64_t seed, uint32_t stream_id, hipStream_t st, bool absmax_ready) {
   const int64_t row_bytes = K * BITS / 8;
   if (ld > row_bytes) {
     const int64_t n = M * ((ld - row_bytes) / 4);
     hipLaunchKernelGGL(zero_pad_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (int8_t*)codes, M, row_bytes, ld);
   }
   if (scale_mode == HOT_SCALE_ROW) return launch_row<T, N, BITS, ROUND>(in, M, K, codes, ld, scales, seed, stream_id, st);
-  return launch_tensor<T, N, BITS, ROUND>(in, M, K, codes, ld, scales, absmax, seed, stream_id, st);
+  return launch_tensor<T, N, BITS, ROUND>(in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready);
 }
 
 template <typename T, int N>
 static int dispatch_bits(int bits, int rounding, int scale_mode, const void* in, int64_t M, int64_t K,
                          void* codes, int64_t ld, float* scales, float* absmax, uint64_t seed, uint32_t stream_id,
-                         hipStream_t st) {
+                         hipStream_t st, bool absmax_ready) {
   if (bits == 4) {
     return rounding == HOT_ROUND_NEAREST
-               ? dispatch_mode<T, N, 4, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st)
-               : dispatch_mode<T, N, 4, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st);
+               ? dispatch_mode<T, N, 4, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready)
+               : dispatch_mode<T, N, 4, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready);
   }
   return rounding == HOT_ROUND_NEAREST
-             ? dispatch_mode<T, N, 8, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st)
-             : dispatch_mode<T, N, 8, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st);
+             ? dispatch_mode<T, N, 8, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready)
+             : dispatch_mode<T, N, 8, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready);
 }
 
 template <typename T>
 static int dispatch_n(int n, int bits, int rounding, int scale_mode, const void* in, int64_t M, int64_t K,
                       void* codes, int64_t ld, float* scales, float* absmax, uint64_t seed, uint32_t stream_id,
-                      hipStream_t st) {
+                      hipStream_t st, bool absmax_ready) {
   switch (n) {
-    case 16: return dispatch_bits<T, 16>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st);
-    case 32: return dispatch_bits<T, 32>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st);
-    default: return dispatch_bits<T, 64>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st);
+    case 16: return dispatch_bits<T, 16>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready);
+    case 32: return dispatch_bits<T, 32>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready);
+    default: return dispatch_bits<T, 64>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready);
   }
 }
 
 int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, int rounding,
                     uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_codes,
-                    float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st) {
+                    float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st, bool absmax_ready) {
   if (M != 0 && (!in || !codes_out || !scales_out)) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: null pointer");
   if (M < 0 || K <= 0) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: bad shape M=%lld K=%lld", (long long)M, (long long)K);
   if (n != 16 && n != 32 && n != 64) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: Hadamard block %d (16, 32 or 64)", n);
@@ -320,9 +322,9 @@ int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int 
   }
   if (M == 0) return HOT_OK;
   switch (dtype) {
-    case HOT_F32: return dispatch_n<float>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st);
-    case HOT_BF16: return dispatch_n<bf16_t>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st);
-    case HOT_F16: return dispatch_n<f16_t>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st);
+    case HOT_F32: return dispatch_n<float>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st, absmax_ready);
+    case HOT_BF16: return dispatch_n<bf16_t>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st, absmax_ready);
+    case HOT_F16: return dispatch_n<f16_t>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st, absmax_ready);
     default: return fail(HOT_ERR_INVALID, "hot_hq_rowwise: bad dtype %d", dtype);
   }
 }
