@@ -68,6 +68,15 @@ static BwdLayout bwd_layout(int64_t L, int64_t O, int64_t I, const hot_config* c
   return b;
 }
 
+__global__ void clear3_kernel(uint32_t* p0, int n0, uint32_t* p1, int n1, uint32_t* p2, int n2) {
+  int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n0) { p0[i] = 0u; return; }
+  i -= n0;
+  if (i < n1) { p1[i] = 0u; return; }
+  i -= n1;
+  if (i < n2) p2[i] = 0u;
+}
+
 static const int32_t* identity_rows() {
   static int32_t rows[HOT_MAX_HLA_N];
   static bool init = false;
@@ -171,6 +180,13 @@ int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq
     (void)hipEventRecord(ev[0], st);
   }
   int rc;
+  // one launch zeroes every statistic of the call (absmax slots, per-channel maxima)
+  {
+    const int n0 = 64, n1 = (int)(colwise_stats_bytes_impl(I) / 4), n2 = (int)(colwise_stats_bytes_impl(O) / 4);
+    const int total = n0 + n1 + n2;
+    hipLaunchKernelGGL(clear3_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                       (uint32_t*)(ws + b.off_hq), n0, (uint32_t*)(ws + b.off_colw), n1, (uint32_t*)(ws + b.off_colg), n2);
+  }
   // g_y: HLA along tokens + quantise, transposed (g_W operand); Hadamard along O + quantise (g_x
   // operand).  With one step per tensor both quantisers need the absmax of their transform first:
   // the statistics pass of the token-wise kernel delivers both from a single read of g_y.
@@ -180,7 +196,7 @@ int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq
     rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->gw_bits, cfg->gw_round,
                             cfg->seed, HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp,
                             ws + b.off_colg, colwise_workspace_bytes_impl(O), st, who,
-                            fuse ? (float*)(ws + b.off_hq) : nullptr);
+                            fuse ? (float*)(ws + b.off_hq) : nullptr, /*stats_cleared=*/true);
     if (rc) goto done;
     rc = hq_rowwise_impl(gy, dtype, L, O, cfg->n_o, cfg->gx_bits, cfg->gx_round, cfg->seed, HOT_STREAM_GX,
                          cfg->gx_scale, ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, 256, st, fuse);
@@ -190,7 +206,7 @@ int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq
   // W: Hadamard along O + quantise, stored [I, O]
   rc = colwise_quant_impl(w, dtype, O, I, cfg->n_o, identity_rows(), cfg->n_o, cfg->w_bits, cfg->w_round, cfg->seed,
                           HOT_STREAM_W, cfg->w_scale, ws + b.off_qw, b.ld_w, cfg->w_bits == 4, sw,
-                          ws + b.off_colw, colwise_workspace_bytes_impl(I), st, who);
+                          ws + b.off_colw, colwise_workspace_bytes_impl(I), st, who, nullptr, /*stats_cleared=*/true);
   if (rc) goto done;
   if (times4) (void)hipEventRecord(ev[2], st);
   // g_x = (qG . qW^T) sG sW / n_o

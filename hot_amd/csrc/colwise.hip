@@ -45,7 +45,7 @@ struct ColArgs {
   float* row_absmax;  // statistics pass with RS != 0: absmax of the row-wise block Hadamard
   uint64_t seed;
   uint32_t stream;
-  int32_t r, rpad, bits, store4, rounding, mode, tb;
+  int32_t r, rpad, bits, store4, rounding, mode, tb, stats_cleared;
   int8_t slot[HOT_MAX_HLA_N];  // output position of natural row i, -1 = dropped
 };
 
@@ -197,8 +197,15 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     uint32_t* l32 = reinterpret_cast<uint32_t*>(stage);
     for (int i = tid; i < CW * pitch / 4; i += CW) l32[i] = 0u;   // gaps of partial groups must read as 0
     __syncthreads();
+    // absmax modes read the statistic itself (no finalize kernel in between) and publish the step
     if (a.mode == HOT_SCALE_ROW) {
-      d = active ? (a.colmax[c] / (float)qmax + 1e-11f) : 1.f;
+      const float sc = active ? a.colmax[c] / (float)qmax : 0.f;
+      d = active ? sc + 1e-11f : 1.f;
+      if (active && blockIdx.y == 0) a.scales_out[c] = sc;
+    } else if (a.mode == HOT_SCALE_TENSOR) {
+      const float sc = a.stat[0] / (float)qmax;
+      d = sc + 1e-11f;
+      if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) a.scales_out[0] = sc;
     } else {
       d = a.stat[1] + 1e-11f;
       clip = a.stat[2];
@@ -418,6 +425,8 @@ __global__ void colwise_clear_kernel(float* stat, float* colmax, int64_t C, floa
 
 static constexpr size_t COL_STAT_BYTES = 256;
 
+size_t colwise_stats_bytes_impl(int64_t C) { return COL_STAT_BYTES + (size_t)round_up(C * 4, 256); }
+
 size_t colwise_workspace_bytes_impl(int64_t C) {
   // stat | per-channel max | per-workgroup partial sums (at most 65536 workgroups)
   return COL_STAT_BYTES + (size_t)round_up(C * 4, 256) + (size_t)(2 * sizeof(double)) * 65536;
@@ -454,15 +463,17 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   const int64_t gx = (a.C + CW - 1) / CW, gy = (a.NB + tb - 1) / tb;
   if (gy > 65535 || gx * gy > 65536) return fail(HOT_ERR_UNSUPPORTED, "colwise: grid %lld x %lld too large", (long long)gx, (long long)gy);
   const dim3 grid((unsigned)gx, (unsigned)gy);
-  const int64_t nclr = a.C > 4 ? a.C : 4;
-  hipLaunchKernelGGL(colwise_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat,
-                     a.mode == HOT_SCALE_ROW ? a.colmax : (float*)nullptr, a.C, a.row_absmax);
+  if (!a.stats_cleared) {
+    const int64_t nclr = a.C > 4 ? a.C : 4;
+    hipLaunchKernelGGL(colwise_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat,
+                       a.mode == HOT_SCALE_ROW ? a.colmax : (float*)nullptr, a.C, a.row_absmax);
+  }
   int rc;
   if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 0, 0, true, SEL>(a, grid, lds_stats, st);
   else if (a.row_absmax) rc = launch_pass<T, N, 0, 0, false, SEL, 16>(a, grid, lds_stats, st);
   else rc = launch_pass<T, N, 0, 0, false, SEL>(a, grid, lds_stats, st);
   if (rc) return rc;
-  hipLaunchKernelGGL(colwise_finalize_kernel, dim3(1), dim3(256), 0, st, a, gx * gy);
+  if (a.mode == HOT_SCALE_SAWB) hipLaunchKernelGGL(colwise_finalize_kernel, dim3(1), dim3(256), 0, st, a, gx * gy);
   if (a.rounding == HOT_ROUND_STOCH) {
     if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 1, 1, true, SEL>(a, grid, lds_quant, st);
     else rc = launch_pass<T, N, 1, 1, false, SEL>(a, grid, lds_quant, st);
@@ -506,7 +517,8 @@ static int dispatch_colwise_n(int n, ColArgs& a, hipStream_t st) {
 int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r,
                        int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
                        void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,
-                       size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out) {
+                       size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out,
+                       bool stats_cleared) {
   if (!in || !codes_out || !scales_out || !rows) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
   if (R <= 0 || C <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape R=%lld C=%lld", who, (long long)R, (long long)C);
   if (n < 1 || n > HOT_MAX_HLA_N || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (power of two up to %d)", who, n, HOT_MAX_HLA_N);
@@ -536,6 +548,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   if (!workspace || workspace_bytes < colwise_workspace_bytes_impl(C)) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed", who, colwise_workspace_bytes_impl(C));
   if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
   a.store4 = store4;
+  a.stats_cleared = stats_cleared ? 1 : 0;
   uint8_t* ws = (uint8_t*)workspace;
   a.stat = (float*)ws;
   a.colmax = (float*)(ws + COL_STAT_BYTES);

@@ -30,8 +30,10 @@ int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int 
 int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r,
                        int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
                        void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,
-                       size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out = nullptr);
+                       size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out = nullptr,
+                       bool stats_cleared = false);
 size_t colwise_workspace_bytes_impl(int64_t C);
+size_t colwise_stats_bytes_impl(int64_t C);  // leading part of the workspace that must be zero before the statistics pass
 
 int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bits, int64_t M, int64_t N,
                  int64_t K, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
