@@ -12,8 +12,9 @@ written beforehand by the forward-side kernel.  Four input sets (> 256 MiB in
 total) are rotated so that g_y is not served from the Infinity Cache.
 
 Prints ONE JSON line.  Besides the contract fields it carries
-  roofline      the dominant kernel of the step, timed live with HIP events on
-                the launch stream, against the chip's published peak
+  roofline      the dominant kernel of the step, timed live inside the fused
+                step with HIP events on the launch stream
+                (hot_linear_backward_kernels), against the chip's published peak
   cpu_baseline  the op-for-op CPU port of the reference's fake-quant path
                 (oracle/fakequant_port.py) on the same layer, on the host cores
   kernels       per-kernel microseconds and achieved rates for this layer
@@ -65,47 +66,95 @@ def make_layer(L, O, I, dtype, dev, nsets, seed=0):
     return w, sets
 
 
-def kernel_table(gy, w, x, opt, iters, warm):
-    """Times every kernel group of the step on its own (same operands, same
-    stream) and prices it with its algorithmic bytes / operations."""
+# HBM bytes per launch of each kernel of the step at the bench workload, from two `rocprofv3 --pmc`
+# runs of this file (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same
+# counter reads for a 512 MiB device copy (FETCH_SIZE reads half the bytes, WRITE_SIZE all of them).
+# Summary and commands: profiles/hot_linear_backward_vit_b_fc1_bf16.hbm_traffic.txt
+MEASURED_TRAFFIC_BYTES = {
+    "gy_stats": (2 * 37910.4 + 0.0) * 1024,
+    "gy_hla_quant": (2 * 34001.4 + 26036.4) * 1024,
+    "gy_hq_quant": (2 * 37854.6 + 18912.0) * 1024,
+    "w_stats": (2 * 2331.5 + 0.0) * 1024,
+    "w_quant": (2 * 2352.0 + 1152.0) * 1024,
+    "gemm_gx": (2 * 14742.1 + 18912.0) * 1024,
+    "gemm_gw": (2 * 32420.1 + 4608.0) * 1024,
+}
+
+
+def kernel_table(w, sets, bufs, opt, ws, iters, warm, traffic=None):
+    """Per-kernel durations INSIDE the fused step: hot_linear_backward_kernels records a HIP event
+    on the launch stream after every kernel; the table prices each kernel with its algorithmic
+    bytes (sizeof(in) read once + codes written) or operations (2 M N K)."""
     import torch
     from hot_amd import ops
-    L, O = gy.shape
+    L, O = sets[0][1].shape
     I = w.shape[1]
-    e = gy.element_size()
+    e = sets[0][1].element_size()
     lp = opt.lprime(L)
+    acc = [0.0] * 8
+    for it in range(warm + iters):
+        i = it % len(sets)
+        _, _, t = ops.linear_backward(sets[i][1], w, bufs[i][0], bufs[i][1], opt, timing="kernels", workspace=ws)
+        if it >= warm:
+            acc = [a + b for a, b in zip(acc, t)]
+    us = [a / iters * 1e6 for a in acc]
+    spec = [
+        ("clear", "hot::clear3_kernel", us[0], "hbm", 0.0),
+        ("gy_stats", "hot::colwise_kernel<.., PASS 0, RS 16> (g_y: token-wise + row-wise absmax)", us[1], "hbm", L * O * e),
+        ("gy_hla_quant", "hot::colwise_kernel<.., PASS 1> (g_y: HLA + INT8, transposed)", us[2], "hbm", L * O * e + lp * O),
+        ("gy_hq_quant", "hot::hq_tensor_kernel (g_y: Hadamard-16 + INT%d)" % opt.gx_bits, us[3], "hbm",
+         L * O * e + L * O * opt.gx_bits // 8),
+        ("w_stats", "hot::colwise_kernel<.., PASS 0> (W)", us[4], "hbm", O * I * e),
+        ("w_quant", "hot::colwise_kernel<.., PASS 1> (W: Hadamard-16 + INT%d, transposed)" % opt.w_bits, us[5], "hbm",
+         O * I * e + O * I * opt.w_bits // 8),
+        ("gemm_gx", "hot::gemm_i8_pipe_kernel<2, 2, %d, ..> (g_x)" % opt.gx_bits, us[6], "mfma", 2.0 * L * O * I),
+        ("gemm_gw", "hot::gemm_i8_pipe_kernel<2, 2, 8, ..> (g_W)", us[7], "mfma", 2.0 * O * I * lp),
+    ]
     rows = []
-
-    def add(name, us, bound, alg):
+    for key, name, t, bound, alg in spec:
         peak = HBM_PEAK_GBS if bound == "hbm" else INT8_PEAK_TOPS
-        ach = alg / us / 1e3 if bound == "hbm" else alg / us / 1e6      # GB/s | TOP/s
-        rows.append(dict(kernel=name, us=round(us, 2), bound=bound, achieved=round(ach, 1),
-                         peak=peak, unit="GB/s" if bound == "hbm" else "TOP/s", frac=round(ach / peak, 4)))
-
-    us = _events(lambda: ops.hq_rowwise(gy, n=opt.n_o, bits=opt.gx_bits, rounding=opt.gx_round, scale=opt.gx_scale),
-                 iters, warm)
-    add("hq_rowwise(g_y)", us, "hbm", L * O * e + L * O * opt.gx_bits // 8 + 4 * (L if opt.gx_scale == ops.SCALE_ROW else 1))
-    us = _events(lambda: ops.hla_tokenwise(gy, opt.hla_n, opt.hla_rows, bits=opt.gw_bits, rounding=opt.gw_round,
-                                           scale=opt.gw_scale), iters, warm)
-    add("hla_tokenwise(g_y)", us, "hbm", L * O * e + lp * O)
-    us = _events(lambda: ops.wq_colwise(w, n=opt.n_o, bits=opt.w_bits, rounding=opt.w_round, scale=opt.w_scale),
-                 iters, warm)
-    add("wq_colwise(W)", us, "hbm", O * I * e + O * I * opt.w_bits // 8)
-    us = _events(lambda: ops.abc_forward(x, opt), iters, warm)
-    add("abc_forward(x) [forward side, not in the step]", us, "hbm", L * I * e + lp * I)
-    qg, sg = ops.hq_rowwise(gy, n=opt.n_o, bits=opt.gx_bits, scale=opt.gx_scale)
-    qw, sw = ops.wq_colwise(w, n=opt.n_o, bits=opt.w_bits)
-    qgp, sgp, _ = ops.hla_tokenwise(gy, opt.hla_n, opt.hla_rows, bits=opt.gw_bits, scale=opt.gw_scale)
-    xq, sx = ops.abc_forward(x, opt)
-    if qg.shape[1] != qw.shape[1]:       # O not a multiple of the K tile: pad the packed g_y codes
-        pad = torch.zeros((L, qw.shape[1]), dtype=torch.int8, device=gy.device)
-        pad[:, :qg.shape[1]] = qg
-        qg = pad
-    us = _events(lambda: ops.gemm_i8(qg, qw, O, opt.gx_bits, sg, sw, 1.0 / opt.n_o, out_dtype=gy.dtype), iters, warm)
-    add("gemm_i8(g_x)", us, "mfma", 2.0 * L * O * I)
-    us = _events(lambda: ops.gemm_i8(qgp, xq, lp, 8, sgp, sx, 1.0 / opt.hla_n, out_dtype=gy.dtype), iters, warm)
-    add("gemm_i8(g_W)", us, "mfma", 2.0 * O * I * lp)
+        ach = (alg / t / 1e3 if bound == "hbm" else alg / t / 1e6) if t > 0 else 0.0      # GB/s | TOP/s
+        rows.append(dict(key=key, kernel=name, us=round(t, 2), bound=bound, achieved=round(ach, 1), peak=peak,
+                         unit="GB/s" if bound == "hbm" else "TOP/s", frac=round(ach / peak, 4),
+                         traffic=(round(traffic[key]) if traffic and key in traffic else None),
+                         work=("%.0f bytes" % alg if bound == "hbm" else "%.0f ops" % alg)))
     return rows
+
+
+def gemm_launch_times(w, sets, bufs, opt, iters=20, warm=4):
+    """Average launch duration of the two GEMM kernels of the step, each timed over `iters`
+    back-to-back launches between two HIP events on the launch stream, on the step's real
+    operands (produced by the transform kernels), rotating the input sets."""
+    import torch
+    from hot_amd import ops
+    L, O = sets[0][1].shape
+    I = w.shape[1]
+    lp = opt.lprime(L)
+    qw, sw = ops.wq_colwise(w, n=opt.n_o, bits=opt.w_bits, rounding=opt.w_round, scale=opt.w_scale)
+    gx_ops, gw_ops = [], []
+    for (x, gy), (xq, sx) in zip(sets, bufs):
+        qg, sg = ops.hq_rowwise(gy, n=opt.n_o, bits=opt.gx_bits, rounding=opt.gx_round, scale=opt.gx_scale)
+        if qg.shape[1] != qw.shape[1]:       # O not a multiple of the K tile: pad the packed g_y codes
+            pad = torch.zeros((L, qw.shape[1]), dtype=torch.int8, device=gy.device)
+            pad[:, :qg.shape[1]] = qg
+            qg = pad
+        qgp, sgp, _ = ops.hla_tokenwise(gy, opt.hla_n, opt.hla_rows, bits=opt.gw_bits, rounding=opt.gw_round,
+                                        scale=opt.gw_scale)
+        gx_ops.append((qg, sg))
+        gw_ops.append((qgp, sgp, xq, sx))
+    state = {"i": 0}
+
+    def run_gx():
+        qg, sg = gx_ops[state["i"] % len(gx_ops)]
+        state["i"] += 1
+        ops.gemm_i8(qg, qw, O, opt.gx_bits, sg, sw, 1.0 / opt.n_o, out_dtype=sets[0][1].dtype)
+
+    def run_gw():
+        qgp, sgp, xq, sx = gw_ops[state["i"] % len(gw_ops)]
+        state["i"] += 1
+        ops.gemm_i8(qgp, xq, lp, 8, sgp, sx, 1.0 / opt.hla_n, out_dtype=sets[0][1].dtype)
+
+    return _events(run_gx, iters, warm), _events(run_gw, iters, warm)
 
 
 def step_time(w, sets, opt, steps, warmup):
@@ -133,7 +182,7 @@ def step_time(w, sets, opt, steps, warmup):
     for _ in range(steps):
         one()
     torch.cuda.synchronize()
-    return (time.perf_counter() - t0) / steps
+    return (time.perf_counter() - t0) / steps, bufs, ws
 
 
 def cpu_baseline(reps=5):
@@ -166,6 +215,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-extras", action="store_true", help="skip the per-kernel table and the Llama shape")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run three 512 MiB device-to-device copies (a kernel of known traffic, for scaling "
+                         "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)"
@@ -181,11 +233,19 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
 
+    if a.copy_calibration:
+        src = torch.empty(512 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+
     L, O, I = 12608, 3072, 768
     n, rows = hla_rows(L)
     opt = ops.HotOptions(n_o=16, hla_n=int(n), hla_rows=tuple(int(v) for v in rows))
     w, sets = make_layer(L, O, I, torch.bfloat16, dev, nsets=4)
-    sec = step_time(w, sets, opt, a.steps, a.warmup)
+    sec, bufs, ws = step_time(w, sets, opt, a.steps, a.warmup)
 
     out = {
         "metric": "hot_linear_backward_us_per_layer", "value": round(sec * 1e6, 2), "unit": "us/layer",
@@ -198,19 +258,25 @@ def main():
                    "L": L, "O": O, "I": I, "input_sets_rotated": len(sets)},
     }
     if not a.no_extras:
-        table = kernel_table(sets[0][1], w, sets[0][0], opt, iters=20, warm=3)
+        table = kernel_table(w, sets, bufs, opt, ws, iters=20, warm=4, traffic=MEASURED_TRAFFIC_BYTES)
         out["kernels"] = table
-        step_rows = [r for r in table if "not in the step" not in r["kernel"]]
-        dom = max(step_rows, key=lambda r: r["us"])
+        # Roofline entry: the kernel with the longest in-step duration (HIP events recorded on the
+        # launch stream around every kernel of the timed steps); the same two GEMMs launched back
+        # to back, without the neighbouring kernels, are reported beside it.
+        rows = {r["key"]: r for r in table}
+        key = max(rows, key=lambda k: rows[k]["us"])
+        dom = rows[key]
+        us_gx, us_gw = gemm_launch_times(w, sets, bufs, opt)
         out["roofline"] = {"kernel": dom["kernel"], "bound": dom["bound"], "achieved": dom["achieved"],
-                           "peak": dom["peak"], "unit": dom["unit"], "frac": dom["frac"], "traffic": None,
-                           "us_per_launch": dom["us"]}
+                           "peak": dom["peak"], "unit": dom["unit"], "frac": dom["frac"], "traffic": dom["traffic"],
+                           "us_per_launch": dom["us"], "per_launch": dom["work"],
+                           "back_to_back_us": {"gemm_gx": round(us_gx, 2), "gemm_gw": round(us_gw, 2)}}
         # Llama-7B gate/up at 8192 tokens, bf16, paper HLA setting (n = 16, 8 lowest sequencies)
         Ll, Ol, Il = 8192, 11008, 4096
         pn, prow = paper_rows(16, 8)
         lopt = ops.HotOptions(n_o=16, hla_n=int(pn), hla_rows=tuple(int(v) for v in prow))
         lw, lsets = make_layer(Ll, Ol, Il, torch.bfloat16, dev, nsets=2, seed=1)
-        lsec = step_time(lw, lsets, lopt, max(5, a.steps // 5), max(2, a.warmup // 5))
+        lsec, _, _ = step_time(lw, lsets, lopt, max(5, a.steps // 5), max(2, a.warmup // 5))
         out["llama_gate_up"] = {"us_per_layer": round(lsec * 1e6, 1), "L": Ll, "O": Ol, "I": Il,
                                 "hla": "n=16 r=8", "int8_tops": round((2.0 * Ll * Ol * Il + 2.0 * Ol * Il * (Ll // 2)) / lsec / 1e12, 1)}
         del lw, lsets

@@ -150,9 +150,23 @@ size_t hot_backward_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_c
   return bwd_layout(L, O, I, cfg).total;
 }
 
-int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,
+// Slots of the per-kernel timing of one backward (hot_linear_backward_kernels).
+enum {
+  K_CLEAR = 0,      // statistics cleared
+  K_GY_STATS = 1,   // token-wise statistics pass over g_y (also the row-wise absmax when fused)
+  K_GY_HLA = 2,     // token-wise quantise pass over g_y  -> g_W operand
+  K_GY_HQ = 3,      // row-wise pass(es) over g_y          -> g_x operand
+  K_W_STATS = 4,    // statistics pass over W
+  K_W_QUANT = 5,    // quantise pass over W
+  K_GEMM_GX = 6,
+  K_GEMM_GW = 7,
+  K_COUNT = 8
+};
+
+static int run_backward(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,
                         int64_t O, int64_t I, const hot_config* cfg, void* gx, void* gw, int out_dtype,
-                        void* workspace, size_t workspace_bytes, float* times4, void* hip_stream) {
+                        void* workspace, size_t workspace_bytes, hipEvent_t* ev /* K_COUNT + 1 or null */,
+                        hipStream_t st) {
   const char* who = "hot_linear_backward";
   if (int e = check_cfg(cfg, who)) return e;
   if (!gy || !w || !xq || !sx || !gx || !gw) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
@@ -166,20 +180,14 @@ int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq
   const BwdLayout b = bwd_layout(L, O, I, cfg);
   if (!workspace || workspace_bytes < b.total) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, b.total, workspace_bytes);
   if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
-  hipStream_t st = (hipStream_t)hip_stream;
   uint8_t* ws = (uint8_t*)workspace;
   float* sg = (float*)(ws + b.off_sg);
   float* sw = (float*)(ws + b.off_sw);
   float* sgp = (float*)(ws + b.off_sgp);
   const int64_t lp = (L / cfg->hla_n) * cfg->hla_r;
+  auto mark = [&](int slot) { if (ev) (void)hipEventRecord(ev[slot], st); };
 
-  hipEvent_t ev[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
-  if (times4) {
-    for (int i = 0; i < 5; ++i)
-      if (int e = check_hip(hipEventCreate(&ev[i]), "hipEventCreate")) return e;
-    (void)hipEventRecord(ev[0], st);
-  }
-  int rc;
+  mark(0);
   // one launch zeroes every statistic of the call (absmax slots, per-channel maxima)
   {
     const int n0 = 64, n1 = (int)(colwise_stats_bytes_impl(I) / 4), n2 = (int)(colwise_stats_bytes_impl(O) / 4);
@@ -187,52 +195,87 @@ int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq
     hipLaunchKernelGGL(clear3_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
                        (uint32_t*)(ws + b.off_hq), n0, (uint32_t*)(ws + b.off_colw), n1, (uint32_t*)(ws + b.off_colg), n2);
   }
+  mark(K_CLEAR + 1);
   // g_y: HLA along tokens + quantise, transposed (g_W operand); Hadamard along O + quantise (g_x
   // operand).  With one step per tensor both quantisers need the absmax of their transform first:
   // the statistics pass of the token-wise kernel delivers both from a single read of g_y.
-  {
-    const bool fuse = cfg->gx_scale == HOT_SCALE_TENSOR && cfg->n_o == 16 && O % 16 == 0 &&
-                      cfg->gw_scale != HOT_SCALE_SAWB;
-    rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->gw_bits, cfg->gw_round,
-                            cfg->seed, HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp,
-                            ws + b.off_colg, colwise_workspace_bytes_impl(O), st, who,
-                            fuse ? (float*)(ws + b.off_hq) : nullptr, /*stats_cleared=*/true);
-    if (rc) goto done;
-    rc = hq_rowwise_impl(gy, dtype, L, O, cfg->n_o, cfg->gx_bits, cfg->gx_round, cfg->seed, HOT_STREAM_GX,
-                         cfg->gx_scale, ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, 256, st, fuse);
-    if (rc) goto done;
-  }
-  if (times4) (void)hipEventRecord(ev[1], st);
+  const bool fuse = cfg->gx_scale == HOT_SCALE_TENSOR && cfg->n_o == 16 && O % 16 == 0 && cfg->gw_scale != HOT_SCALE_SAWB;
+  int rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->gw_bits, cfg->gw_round,
+                              cfg->seed, HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp,
+                              ws + b.off_colg, colwise_workspace_bytes_impl(O), st, who,
+                              fuse ? (float*)(ws + b.off_hq) : nullptr, /*stats_cleared=*/true,
+                              ev ? ev[K_GY_STATS + 1] : nullptr);
+  if (rc) return rc;
+  mark(K_GY_HLA + 1);
+  rc = hq_rowwise_impl(gy, dtype, L, O, cfg->n_o, cfg->gx_bits, cfg->gx_round, cfg->seed, HOT_STREAM_GX,
+                       cfg->gx_scale, ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, 256, st, fuse);
+  if (rc) return rc;
+  mark(K_GY_HQ + 1);
   // W: Hadamard along O + quantise, stored [I, O]
   rc = colwise_quant_impl(w, dtype, O, I, cfg->n_o, identity_rows(), cfg->n_o, cfg->w_bits, cfg->w_round, cfg->seed,
                           HOT_STREAM_W, cfg->w_scale, ws + b.off_qw, b.ld_w, cfg->w_bits == 4, sw,
-                          ws + b.off_colw, colwise_workspace_bytes_impl(I), st, who, nullptr, /*stats_cleared=*/true);
-  if (rc) goto done;
-  if (times4) (void)hipEventRecord(ev[2], st);
+                          ws + b.off_colw, colwise_workspace_bytes_impl(I), st, who, nullptr, /*stats_cleared=*/true,
+                          ev ? ev[K_W_STATS + 1] : nullptr);
+  if (rc) return rc;
+  mark(K_W_QUANT + 1);
   // g_x = (qG . qW^T) sG sW / n_o
   rc = gemm_i8_impl(ws + b.off_qg, b.ld_g, ws + b.off_qw, b.ld_w, cfg->gx_bits, L, I, O, sg,
                     cfg->gx_scale == HOT_SCALE_ROW, sw, 1.0f / (float)cfg->n_o, gx, out_dtype, I, nullptr, st);
-  if (rc) goto done;
-  if (times4) (void)hipEventRecord(ev[3], st);
+  if (rc) return rc;
+  mark(K_GEMM_GX + 1);
   // g_W = (qGp . xq^T) sGp sx / hla_n
   rc = gemm_i8_impl(ws + b.off_qgp, b.ld_gp, xq, b.ld_gp, 8, O, I, lp, sgp, cfg->gw_scale == HOT_SCALE_ROW, sx,
                     1.0f / (float)cfg->hla_n, gw, out_dtype, I, nullptr, st);
-  if (rc) goto done;
-  if (times4) {
-    (void)hipEventRecord(ev[4], st);
-    rc = check_hip(hipEventSynchronize(ev[4]), "hipEventSynchronize");
-    if (!rc) {
-      for (int i = 0; i < 4; ++i) {
-        float ms = 0.f;
-        (void)hipEventElapsedTime(&ms, ev[i], ev[i + 1]);
-        times4[i] = ms * 1e-3f;
-      }
+  if (rc) return rc;
+  mark(K_GEMM_GW + 1);
+  return HOT_OK;
+}
+
+// Runs the backward with an event after every kernel group and returns the K_COUNT durations (s).
+static int run_backward_timed(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,
+                              int64_t O, int64_t I, const hot_config* cfg, void* gx, void* gw, int out_dtype,
+                              void* workspace, size_t workspace_bytes, float* secs, hipStream_t st) {
+  hipEvent_t ev[K_COUNT + 1];
+  for (int i = 0; i <= K_COUNT; ++i) ev[i] = nullptr;
+  int rc = HOT_OK;
+  for (int i = 0; i <= K_COUNT && !rc; ++i) rc = check_hip(hipEventCreate(&ev[i]), "hipEventCreate");
+  if (!rc) rc = run_backward(gy, w, dtype, xq, sx, L, O, I, cfg, gx, gw, out_dtype, workspace, workspace_bytes, ev, st);
+  if (!rc) rc = check_hip(hipEventSynchronize(ev[K_COUNT]), "hipEventSynchronize");
+  if (!rc) {
+    for (int i = 0; i < K_COUNT; ++i) {
+      float ms = 0.f;
+      (void)hipEventElapsedTime(&ms, ev[i], ev[i + 1]);
+      secs[i] = ms * 1e-3f;
     }
   }
-done:
-  for (int i = 0; i < 5; ++i)
+  for (int i = 0; i <= K_COUNT; ++i)
     if (ev[i]) (void)hipEventDestroy(ev[i]);
   return rc;
+}
+
+int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,
+                        int64_t O, int64_t I, const hot_config* cfg, void* gx, void* gw, int out_dtype,
+                        void* workspace, size_t workspace_bytes, float* times4, void* hip_stream) {
+  if (!times4)
+    return run_backward(gy, w, dtype, xq, sx, L, O, I, cfg, gx, gw, out_dtype, workspace, workspace_bytes, nullptr,
+                        (hipStream_t)hip_stream);
+  float k[K_COUNT];
+  const int rc = run_backward_timed(gy, w, dtype, xq, sx, L, O, I, cfg, gx, gw, out_dtype, workspace, workspace_bytes,
+                                    k, (hipStream_t)hip_stream);
+  if (rc) return rc;
+  times4[0] = k[K_CLEAR] + k[K_GY_STATS] + k[K_GY_HLA] + k[K_GY_HQ];
+  times4[1] = k[K_W_STATS] + k[K_W_QUANT];
+  times4[2] = k[K_GEMM_GX];
+  times4[3] = k[K_GEMM_GW];
+  return HOT_OK;
+}
+
+int hot_linear_backward_kernels(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,
+                                int64_t O, int64_t I, const hot_config* cfg, void* gx, void* gw, int out_dtype,
+                                void* workspace, size_t workspace_bytes, float* times8, void* hip_stream) {
+  if (!times8) return fail(HOT_ERR_INVALID, "hot_linear_backward_kernels: null times8");
+  return run_backward_timed(gy, w, dtype, xq, sx, L, O, I, cfg, gx, gw, out_dtype, workspace, workspace_bytes, times8,
+                            (hipStream_t)hip_stream);
 }
 
 }  // extern "C"

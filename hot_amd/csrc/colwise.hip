@@ -46,6 +46,7 @@ struct ColArgs {
   uint64_t seed;
   uint32_t stream;
   int32_t r, rpad, bits, store4, rounding, mode, tb, stats_cleared;
+  hipEvent_t after_stats;  // host only: recorded between the statistics and the quantise pass
   int8_t slot[HOT_MAX_HLA_N];  // output position of natural row i, -1 = dropped
 };
 
@@ -474,6 +475,7 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   else rc = launch_pass<T, N, 0, 0, false, SEL>(a, grid, lds_stats, st);
   if (rc) return rc;
   if (a.mode == HOT_SCALE_SAWB) hipLaunchKernelGGL(colwise_finalize_kernel, dim3(1), dim3(256), 0, st, a, gx * gy);
+  if (a.after_stats) (void)hipEventRecord(a.after_stats, st);
   if (a.rounding == HOT_ROUND_STOCH) {
     if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 1, 1, true, SEL>(a, grid, lds_quant, st);
     else rc = launch_pass<T, N, 1, 1, false, SEL>(a, grid, lds_quant, st);
@@ -518,7 +520,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
                        int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
                        void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,
                        size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out,
-                       bool stats_cleared) {
+                       bool stats_cleared, hipEvent_t after_stats) {
   if (!in || !codes_out || !scales_out || !rows) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
   if (R <= 0 || C <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape R=%lld C=%lld", who, (long long)R, (long long)C);
   if (n < 1 || n > HOT_MAX_HLA_N || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (power of two up to %d)", who, n, HOT_MAX_HLA_N);
@@ -549,6 +551,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
   a.store4 = store4;
   a.stats_cleared = stats_cleared ? 1 : 0;
+  a.after_stats = after_stats;
   uint8_t* ws = (uint8_t*)workspace;
   a.stat = (float*)ws;
   a.colmax = (float*)(ws + COL_STAT_BYTES);

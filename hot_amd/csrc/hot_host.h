@@ -31,7 +31,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
                        int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
                        void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,
                        size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out = nullptr,
-                       bool stats_cleared = false);
+                       bool stats_cleared = false, hipEvent_t after_stats = nullptr);
 size_t colwise_workspace_bytes_impl(int64_t C);
 size_t colwise_stats_bytes_impl(int64_t C);  // leading part of the workspace that must be zero before the statistics pass
 

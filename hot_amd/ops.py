@@ -182,7 +182,8 @@ def abc_forward(x: torch.Tensor, opt: HotOptions):
 
 def linear_backward(gy: torch.Tensor, w: torch.Tensor, xq: torch.Tensor, sx: torch.Tensor, opt: HotOptions,
                     out_dtype=None, timing: bool = False, workspace: Optional[torch.Tensor] = None):
-    """g_x [L, I], g_W [O, I] (and the four stage times in seconds when timing)."""
+    """g_x [L, I], g_W [O, I]; with timing=True also the four stage times (s), with
+    timing="kernels" the eight per-kernel times of hot_linear_backward_kernels."""
     _need_gpu_2d(gy, "Go")
     _need_gpu_2d(w, "Wt")
     L, O = gy.shape
@@ -203,11 +204,12 @@ def linear_backward(gy: torch.Tensor, w: torch.Tensor, xq: torch.Tensor, sx: tor
         workspace = _ws(need, gy.device)
     gx = torch.empty((L, I), dtype=out_dtype, device=gy.device)
     gw = torch.empty((O, I), dtype=out_dtype, device=gy.device)
-    times = (C.c_float * 4)() if timing else None
-    _lib.check(_lib.lib().hot_linear_backward(gy.data_ptr(), w.data_ptr(), _dt(gy), xq.data_ptr(), sx.data_ptr(),
-                                              L, O, I, C.byref(cfg), gx.data_ptr(), gw.data_ptr(),
-                                              _DTYPES[out_dtype], workspace.data_ptr(), workspace.numel(), times,
-                                              _stream()))
+    per_kernel = timing == "kernels"
+    times = (C.c_float * (8 if per_kernel else 4))() if timing else None
+    entry = _lib.lib().hot_linear_backward_kernels if per_kernel else _lib.lib().hot_linear_backward
+    _lib.check(entry(gy.data_ptr(), w.data_ptr(), _dt(gy), xq.data_ptr(), sx.data_ptr(), L, O, I, C.byref(cfg),
+                     gx.data_ptr(), gw.data_ptr(), _DTYPES[out_dtype], workspace.data_ptr(), workspace.numel(),
+                     times, _stream()))
     if timing:
         return gx, gw, [float(t) for t in times]
     return gx, gw

@@ -163,6 +163,23 @@ HOT_API int hot_linear_backward(const void* gy, const void* w, int dtype, const 
                         void* workspace, size_t workspace_bytes, float* times4,
                         void* hip_stream);
 
+/*
+ * hot_linear_backward with a HIP event after every kernel group; synchronises
+ * the stream.  times8 (host) receives the seconds of
+ *   [0] clearing the statistics          [1] token-wise statistics pass over g_y
+ *   [2] token-wise quantise pass (g_y)   [3] row-wise quantise pass(es) (g_y)
+ *   [4] statistics pass over W           [5] quantise pass over W
+ *   [6] g_x GEMM                         [7] g_W GEMM
+ * The reference has no counterpart beyond the four clock() stage timers its op
+ * returns (cuda_measure/HLQ_backward_kernel.cu:717-733); this is the
+ * measurement hook of bench.py.
+ */
+HOT_API int hot_linear_backward_kernels(const void* gy, const void* w, int dtype, const void* xq,
+                                const float* sx, int64_t L, int64_t O, int64_t I,
+                                const hot_config* cfg, void* gx, void* gw, int out_dtype,
+                                void* workspace, size_t workspace_bytes, float* times8,
+                                void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif
