@@ -1,6 +1,7 @@
 """Builds libhot_gfx950.so (the C-ABI library with the gfx950 kernels) in-tree.
 
-    python -m hot_amd.build
+    python -m hot_amd.build                 # everything
+    python -m hot_amd.build gemm_i8.hip     # recompile one source, relink
 
 hipcc cross-compiles for gfx950 without a GPU.  Packed-FP32 instruction
 selection is switched off for all device code.
@@ -46,9 +47,14 @@ def _compile(src: str) -> str:
     return obj
 
 
-def build(verbose: bool = True) -> str:
+def build(verbose: bool = True, only=None) -> str:
+    """Compiles every source and links the library.  `only` (a list of source names) recompiles just
+    those and reuses the other object files of an earlier full build: a developer shortcut."""
+    todo = [s for s in SOURCES if not only or s in only
+            or not os.path.exists(os.path.join(CSRC, s.replace(".hip", ".o")))]
     with ThreadPoolExecutor(max_workers=min(4, len(SOURCES))) as ex:
-        objs = list(ex.map(_compile, SOURCES))
+        list(ex.map(_compile, todo))
+    objs = [os.path.join(CSRC, s.replace(".hip", ".o")) for s in SOURCES]
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
     if r.returncode != 0:
@@ -59,4 +65,4 @@ def build(verbose: bool = True) -> str:
 
 
 if __name__ == "__main__":
-    build()
+    build(only=[a for a in sys.argv[1:] if a.endswith(".hip")] or None)

@@ -22,6 +22,7 @@
 #include <stdlib.h>
 
 #include <type_traits>
+#include <utility>
 
 #include "hot_device.h"
 #include "hot_host.h"
@@ -46,7 +47,108 @@ struct GemmArgs {
   int64_t ldo;
   int32_t* acc_out;
   int32_t tiles_m, tiles_n;
+  int32_t group_m;   // tile rows per group of the launch order (tile_of)
+  int32_t vec_out;   // out and ldo allow aligned four-element stores
 };
+
+// Workgroup -> tile.  Hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with
+// its own L2.  XCD x takes a contiguous chunk of the launch order, and the launch order walks the
+// tile grid in groups of group_m tile rows, row index fastest inside a group, so the workgroups that
+// are resident in one XCD at the same time form a compact block of tiles: they stream few distinct
+// A and B row panels, and most of their loads hit in that XCD's L2.
+__device__ __forceinline__ void tile_of(const GemmArgs& g, int wg, int& tm, int& tn) {
+  const int total = g.tiles_m * g.tiles_n;
+  const int x = wg & 7, idx = wg >> 3;
+  const int q = total >> 3, rem = total & 7;
+  const int t = x * q + (x < rem ? x : rem) + idx;
+  const int per_group = g.group_m * g.tiles_n;
+  const int grp = t / per_group, j = t - grp * per_group;
+  const int rows = min(g.group_m, g.tiles_m - grp * g.group_m);
+  tm = grp * g.group_m + j % rows;
+  tn = j / rows;
+}
+
+// Rows per group: about the square root of the tiles one XCD holds at a time.
+static int pick_group_m(int tiles_m, int tiles_n, int wgs_per_cu) {
+  static int forced = -1;   // experiments: HOT_GEMM_GROUP_M overrides the rule
+  if (forced < 0) { const char* e = getenv("HOT_GEMM_GROUP_M"); forced = e ? atoi(e) : 0; }
+  if (forced > 0) return forced < tiles_m ? forced : tiles_m;
+  const int64_t total = (int64_t)tiles_m * tiles_n;
+  int64_t conc = total / 8 < 32 * wgs_per_cu ? total / 8 : 32 * wgs_per_cu;
+  if (conc < 1) conc = 1;
+  int gm = 1;
+  while ((int64_t)(gm + 1) * (gm + 1) <= conc) ++gm;
+  if (gm > tiles_m) gm = tiles_m;
+  return gm;
+}
+
+
+// Fused dequantisation epilogue, shared by both kernels.  The MFMAs are issued with the operands
+// swapped (B fragment first), so a 32x32 accumulator tile holds the TRANSPOSED product: lane l owns
+// output row l % 32 and, in registers 4 q .. 4 q + 3, the four adjacent output columns
+// 8 q + 4 (l / 32) .. + 3.  Each lane therefore stores four adjacent outputs at a time (8 bytes of
+// bf16 / f16, 16 bytes of fp32), and lanes l and l + 32 fill neighbouring quads of one row.
+template <typename OutT> struct Quad;
+template <> struct Quad<float> { typedef float type __attribute__((ext_vector_type(4))); };
+template <> struct Quad<bf16_t> { typedef uint16_t type __attribute__((ext_vector_type(4))); };
+template <> struct Quad<f16_t> { typedef _Float16 type __attribute__((ext_vector_type(4))); };
+template <typename OutT> __device__ __forceinline__ void quad_set(typename Quad<OutT>::type& q, int t, float v);
+template <> __device__ __forceinline__ void quad_set<float>(Quad<float>::type& q, int t, float v) { q[t] = v; }
+template <> __device__ __forceinline__ void quad_set<bf16_t>(Quad<bf16_t>::type& q, int t, float v) { q[t] = f32_to_bf16_rne(v); }
+template <> __device__ __forceinline__ void quad_set<f16_t>(Quad<f16_t>::type& q, int t, float v) { q[t] = (_Float16)v; }
+
+// The quantisation steps of this lane's output rows; loaded before the K loop so that the loads'
+// latency is hidden behind it.
+template <int WM>
+__device__ __forceinline__ void load_row_scales(const GemmArgs& g, int64_t row_base, int lane, float (&sa_row)[WM]) {
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const int64_t row = row_base + i * 32 + (lane & 31);
+    sa_row[i] = g.a_per_row ? g.scale_a[row < g.M ? row : g.M - 1] : g.scale_a[0];
+  }
+}
+
+template <int WM, int WN, int BITS, typename OutT>
+__device__ __forceinline__ void gemm_epilogue(const v16i (&acc)[WM][WN], const GemmArgs& g, int64_t row_base,
+                                              int64_t col_base, int lane, const float (&sa_row)[WM], float sb) {
+  OutT* out = reinterpret_cast<OutT*>(g.out);
+  const int half = lane >> 5;
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const int64_t row = row_base + i * 32 + (lane & 31);
+    if (row >= g.M) continue;
+    const float sa = sa_row[i];
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t col = col_base + j * 32 + 8 * q + 4 * half;
+        if (col >= g.N) continue;
+        int a[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          a[t] = acc[i][j][4 * q + t];
+          if constexpr (BITS == 4) a[t] >>= 8;
+        }
+        if (g.acc_out) {
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (col + t < g.N) g.acc_out[row * g.N + col + t] = a[t];
+        }
+        if (g.vec_out && col + 3 < g.N) {
+          typename Quad<OutT>::type v;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) quad_set<OutT>(v, t, (((float)a[t] * sa) * sb) * g.post_scale);
+          *reinterpret_cast<typename Quad<OutT>::type*>(out + row * g.ldo + col) = v;
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (col + t < g.N) store_scalar<OutT>(out + row * g.ldo + col + t, (((float)a[t] * sa) * sb) * g.post_scale);
+        }
+      }
+    }
+  }
+}
 
 // Global -> register prefetch of one operand tile (ROWS x G_BK codes), and the
 // register -> LDS store that expands packed INT4 on the way.
@@ -101,19 +203,12 @@ gemm_i8_kernel(const GemmArgs g) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave >> 1, wn = wave & 1;
 
-  // Workgroup -> tile.  Hardware deals consecutive workgroup ids round-robin
-  // to the 8 XCDs; give each XCD a contiguous range of tiles (N fastest) so
-  // the tiles sharing an A row panel meet in one L2.
-  int tile;
-  {
-    const int total = g.tiles_m * g.tiles_n;
-    const int wg = blockIdx.x;
-    const int x = wg & 7, idx = wg >> 3;
-    const int q = total >> 3, rem = total & 7;
-    tile = x * q + (x < rem ? x : rem) + idx;
-  }
-  const int tm = tile / g.tiles_n, tn = tile % g.tiles_n;
+  int tm, tn;
+  tile_of(g, blockIdx.x, tm, tn);
   const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
+  float sa_row[WM];
+  load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
+  const float sb = g.scale_b[0];
 
   constexpr int PTA = TileShape<BM, BITS>::PER_THREAD, PTB = TileShape<BN, BITS>::PER_THREAD;
   v4i ra[PTA], rb[PTB];
@@ -152,7 +247,7 @@ gemm_i8_kernel(const GemmArgs g) {
       for (int i = 0; i < WM; ++i)
 #pragma unroll
         for (int j = 0; j < WN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[j], fa[i], acc[i][j], 0, 0, 0);
     }
     if (kt + 1 < g.ktiles) {
       tile_store<BM, BITS, PTA>(ra, lds + (cur ^ 1) * STAGE_BYTES, tid);
@@ -161,30 +256,7 @@ gemm_i8_kernel(const GemmArgs g) {
     __syncthreads();
   }
 
-  // Epilogue.  In a 32x32 accumulator tile lane l, register e holds
-  // row 8 (e / 4) + 4 (l / 32) + (e % 4), column l % 32.
-  const float sb = g.scale_b[0];
-  const float sa0 = g.a_per_row ? 0.f : g.scale_a[0];
-  OutT* out = reinterpret_cast<OutT*>(g.out);
-#pragma unroll
-  for (int i = 0; i < WM; ++i) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int64_t row = row0 + (wm * WM + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-      if (row >= g.M) continue;
-      const float sa = g.a_per_row ? g.scale_a[row] : sa0;
-#pragma unroll
-      for (int j = 0; j < WN; ++j) {
-        const int64_t col = col0 + (wn * WN + j) * 32 + (lane & 31);
-        if (col >= g.N) continue;
-        int a = acc[i][j][e];
-        if constexpr (BITS == 4) a >>= 8;
-        if (g.acc_out) g.acc_out[row * g.N + col] = a;
-        const float v = (((float)a * sa) * sb) * g.post_scale;
-        store_scalar<OutT>(out + row * g.ldo + col, v);
-      }
-    }
-  }
+  gemm_epilogue<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb);
 }
 
 // ---------------------------------------------------------------------------
@@ -195,10 +267,11 @@ gemm_i8_kernel(const GemmArgs g) {
 // right after the fragment read.
 //
 // LDS stage layout: rows of 64 bytes = four 16-byte slots; slot s of row r is
-// stored at slot s ^ ((r >> 1) & 3), which spreads the 16-byte fragment reads
-// of 8 consecutive rows over all banks.  A wave-wide DMA instruction fills one
+// stored at slot s ^ ((r >> 2) & 3), so the 16-byte fragment reads of 16
+// consecutive rows (same logical slot) land in 16 different 16-byte bank groups
+// of the 256-byte bank row.  A wave-wide DMA instruction fills one
 // contiguous KiB (16 rows); lane l fills physical slot l of that KiB and so
-// fetches row l >> 2, logical slot (l & 3) ^ ((l >> 3) & 3) from global memory.
+// fetches row l >> 2, logical slot (l & 3) ^ ((l >> 4) & 3) from global memory.
 //
 // Each stage is its own __shared__ array and the K loop is unrolled by the
 // stage count, so every LDS access names its stage statically; waits on the
@@ -212,6 +285,24 @@ template <int VM>
 __device__ __forceinline__ void wait_dma() {
   __builtin_amdgcn_s_waitcnt((VM & 0xF) | ((VM >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
+
+// vmcnt wait that lets `tiles` (0 .. MAXT) groups of LPW loads stay in flight
+template <int MAXT, int LPW>
+__device__ __forceinline__ void wait_dma_upto(int tiles) {
+  if constexpr (MAXT <= 0) {
+    wait_dma<0>();
+  } else {
+    if (tiles >= MAXT) wait_dma<MAXT * LPW>();
+    else wait_dma_upto<MAXT - 1, LPW>(tiles);
+  }
+}
+
+template <int... I, class F>
+__device__ __forceinline__ void static_for_impl(std::integer_sequence<int, I...>, F&& f) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) { static_for_impl(std::make_integer_sequence<int, N>{}, f); }
 
 // One wave-wide 16-byte-per-lane load from global memory straight into LDS:
 // lane l's 16 bytes land at lds_addr + 16 l.  `lds_addr` and `sbase` must be
@@ -233,29 +324,22 @@ __device__ __forceinline__ uint32_t lds_offset(const uint8_t* p) {
 template <int WM, int WN, int BITS, int S, typename OutT>
 __global__ void __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(1, (WM * WN <= 4 ? (S == 3 ? 3 : 2) : 1))))
 gemm_i8_pipe_kernel(const GemmArgs g) {
-  static_assert(S == 3 || S == 4, "three or four LDS stages");
+  static_assert(S >= 3 && S * (WM + WN) * 4096 <= 160 * 1024, "three or more LDS stages within 160 KiB");
   constexpr int BM = 64 * WM, BN = 64 * WN;
   constexpr int STAGE_BYTES = (BM + BN) * P_ROWB;
   constexpr int LPW = (BM + BN) / 64;           // DMA instructions per wave per stage (KiB chunks / 4 waves)
   constexpr int GSTEP = P_ROWB;                 // global bytes per stage and row: 64 int8 codes or 128 packed INT4 codes
-  __shared__ __attribute__((aligned(1024))) uint8_t st0[STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t st1[STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t st2[STAGE_BYTES];
-  __shared__ __attribute__((aligned(1024))) uint8_t st3[S == 4 ? STAGE_BYTES : 1024];
+  __shared__ __attribute__((aligned(1024))) uint8_t ring[S * STAGE_BYTES];   // stage k at k * STAGE_BYTES
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
-  int tile;
-  {
-    const int total = g.tiles_m * g.tiles_n;
-    const int wg = blockIdx.x;
-    const int x = wg & 7, idx = wg >> 3;
-    const int q = total >> 3, rem = total & 7;
-    tile = x * q + (x < rem ? x : rem) + idx;
-  }
-  const int tm = tile / g.tiles_n, tn = tile % g.tiles_n;
+  int tm, tn;
+  tile_of(g, blockIdx.x, tm, tn);
   const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
+  float sa_row[WM];
+  load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
+  const float sb = g.scale_b[0];
 
   // DMA instruction i of this wave fills KiB chunk 4 i + wave of the stage (A rows first, then B
   // rows; BM / 16 is a multiple of 4, so instruction i serves A for i < BM / 64 and B otherwise).
@@ -263,7 +347,7 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
 #pragma unroll
   for (int i = 0; i < LPW; ++i) {
     const int r = (4 * i + wave) * 16 + (lane >> 2);
-    const int slot = (lane & 3) ^ ((lane >> 3) & 3);
+    const int slot = (lane & 3) ^ ((lane >> 4) & 3);
     if (i < BM / 64) {
       int64_t gr = row0 + r;
       if (gr >= g.M) gr = g.M - 1;
@@ -294,7 +378,7 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
   // slot 2 d + h of their row: 16 int8 codes (one MFMA) or 32 packed INT4 codes (two MFMAs: the
   // low nibbles, then the high nibbles; both operands alike, so every product pairs equal k).
   const int frow = lane & 31, fhalf = lane >> 5;
-  const int sw = (frow >> 1) & 3;                              // same for rows r and r + 32 k
+  const int sw = (frow >> 2) & 3;                              // same for rows r and r + 32 k
   const int offA = (wm * 32 * WM + frow) * P_ROWB, offB = (BM + wn * 32 * WN + frow) * P_ROWB;
   auto read_round = [&](const uint8_t* stage, int d, v4i (&fa)[WM], v4i (&fb)[WN]) {
     const int so = ((2 * d + fhalf) ^ sw) * 16;
@@ -309,7 +393,7 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
       for (int i = 0; i < WM; ++i)
 #pragma unroll
         for (int j = 0; j < WN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fb[j], fa[i], acc[i][j], 0, 0, 0);
     } else {
       const v4i m = {(int)0xF0F0F0F0, (int)0xF0F0F0F0, (int)0xF0F0F0F0, (int)0xF0F0F0F0};
       v4i ea[WM], eb[WN];
@@ -321,7 +405,7 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
       for (int i = 0; i < WM; ++i)
 #pragma unroll
         for (int j = 0; j < WN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ea[i], eb[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(eb[j], ea[i], acc[i][j], 0, 0, 0);
 #pragma unroll
       for (int i = 0; i < WM; ++i) ea[i] = fa[i] & m;
 #pragma unroll
@@ -330,97 +414,80 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
       for (int i = 0; i < WM; ++i)
 #pragma unroll
         for (int j = 0; j < WN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ea[i], eb[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(eb[j], ea[i], acc[i][j], 0, 0, 0);
     }
   };
 
   const int KT = g.ktiles * (G_BK / (BITS == 8 ? 64 : 128));   // stages of this kernel per G_BK-code tile
   // prologue: S - 1 tiles in flight, tile 0 landed and visible, its first round in registers
-  issue(st0, 0);
-  if (KT > 1) issue(st1, 1);
-  if (S == 4 && KT > 2) issue(st2, 2);
-  if (S == 4 && KT > 2) wait_dma<2 * LPW>(); else if (KT > 1) wait_dma<LPW>(); else wait_dma<0>();
+  static_for<S - 1>([&](auto k) {
+    if (k.value < KT) issue(ring + k.value * STAGE_BYTES, k.value);
+  });
+  wait_dma_upto<S - 2, LPW>((KT < S - 1 ? KT : S - 1) - 1);   // all but the youngest tiles: tile 0 is in
   __builtin_amdgcn_s_barrier();
   v4i a0[WM], b0[WN];
-  read_round(st0, 0, a0, b0);
+  read_round(ring, 0, a0, b0);
 
   // One K-tile.  `cur` holds tile kt, `nxt` tile kt+1 (in flight or landed), `fre` held tile kt-1
   // and receives tile kt+S-1.  The barrier sits in the middle of the tile, behind a block of MFMAs,
   // and the first fragments of tile kt+1 are fetched before the last MFMA block of tile kt starts,
   // so the matrix pipe keeps running across the tile boundary.
   auto ktile = [&](auto steady, const uint8_t* cur, const uint8_t* nxt, const uint8_t* fre, int kt) {
-    // The scheduling fences keep each burst of fragment reads ahead of the MFMA block that
-    // hides its latency; without them the scheduler sinks the reads next to their first use.
+    // Scheduling: the fragment reads of the NEXT MFMA block are interleaved with the MFMAs of the
+    // current one (one LDS read after every MPR MFMAs), so the reads issue while the matrix pipe
+    // is busy instead of after the whole block; the fences keep the blocks themselves in order.
+    constexpr int NREAD = WM + WN;                              // fragment reads per round
+    constexpr int NMFMA = WM * WN * (BITS == 8 ? 1 : 2);        // MFMAs per round
+    constexpr int MPR = NMFMA / NREAD > 0 ? NMFMA / NREAD : 1;  // MFMAs per read
+    auto interleave = [&]() {
+#pragma unroll
+      for (int i = 0; i < NREAD; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x008, MPR, 0);    // MFMA
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);      // DS read
+      }
+      __builtin_amdgcn_sched_group_barrier(0x008, NMFMA - MPR * NREAD, 0);
+    };
     v4i a1[WM], b1[WN];
     read_round(cur, 1, a1, b1);
-    __builtin_amdgcn_sched_barrier(0);
     mma_round(a0, b0);
+    interleave();
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (decltype(steady)::value) {
       // steady state (kt + 3 < KT): straight-line code, so the compiler's LDS wait counts are exact
       wait_dma<(S - 3) * LPW>();                              // this wave's share of tile kt+1 has landed
       __builtin_amdgcn_s_barrier();                           // ... and everybody's; nobody reads tile kt-1 any more
       issue(fre, kt + S - 1);
+      __builtin_amdgcn_sched_barrier(0);
       read_round(nxt, 0, a0, b0);
-    } else if (kt + 1 < KT) {
-      if (S == 4 && kt + 2 < KT) wait_dma<LPW>(); else wait_dma<0>();
-      __builtin_amdgcn_s_barrier();
-      if (kt + S - 1 < KT) issue(fre, kt + S - 1);
-      read_round(nxt, 0, a0, b0);
+      mma_round(a1, b1);
+      interleave();
+    } else {
+      if (kt + 1 < KT) {
+        // tiles kt+2 .. min(kt+S-2, KT-1) may stay in flight
+        wait_dma_upto<S - 3, LPW>((kt + S - 2 < KT - 1 ? kt + S - 2 : KT - 1) - (kt + 1));
+        __builtin_amdgcn_s_barrier();
+        if (kt + S - 1 < KT) issue(fre, kt + S - 1);
+        read_round(nxt, 0, a0, b0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      mma_round(a1, b1);
     }
-    __builtin_amdgcn_sched_barrier(0);
-    mma_round(a1, b1);
     __builtin_amdgcn_sched_barrier(0);
   };
+  // The loop is unrolled by the stage count, so every LDS address is a compile-time offset.
+  auto rotation = [&](auto steady, int kt0) {
+    static_for<S>([&](auto k) {
+      constexpr int K = decltype(k)::value;
+      if (decltype(steady)::value || kt0 + K < KT)
+        ktile(steady, ring + K * STAGE_BYTES, ring + ((K + 1) % S) * STAGE_BYTES, ring + ((K + S - 1) % S) * STAGE_BYTES,
+              kt0 + K);
+    });
+  };
   int kt0 = 0;
-  if constexpr (S == 4) {
-    for (; kt0 + 6 < KT; kt0 += 4) {
-      ktile(std::true_type{}, st0, st1, st3, kt0);
-      ktile(std::true_type{}, st1, st2, st0, kt0 + 1);
-      ktile(std::true_type{}, st2, st3, st1, kt0 + 2);
-      ktile(std::true_type{}, st3, st0, st2, kt0 + 3);
-    }
-    for (; kt0 < KT; kt0 += 4) {
-      ktile(std::false_type{}, st0, st1, st3, kt0);
-      if (kt0 + 1 < KT) ktile(std::false_type{}, st1, st2, st0, kt0 + 1);
-      if (kt0 + 2 < KT) ktile(std::false_type{}, st2, st3, st1, kt0 + 2);
-      if (kt0 + 3 < KT) ktile(std::false_type{}, st3, st0, st2, kt0 + 3);
-    }
-  } else {
-    for (; kt0 + 4 < KT; kt0 += 3) {
-      ktile(std::true_type{}, st0, st1, st2, kt0);
-      ktile(std::true_type{}, st1, st2, st0, kt0 + 1);
-      ktile(std::true_type{}, st2, st0, st1, kt0 + 2);
-    }
-    for (; kt0 < KT; kt0 += 3) {
-      ktile(std::false_type{}, st0, st1, st2, kt0);
-      if (kt0 + 1 < KT) ktile(std::false_type{}, st1, st2, st0, kt0 + 1);
-      if (kt0 + 2 < KT) ktile(std::false_type{}, st2, st0, st1, kt0 + 2);
-    }
-  }
+  for (; kt0 + 2 * S - 2 < KT; kt0 += S) rotation(std::true_type{}, kt0);   // every issue inside is in range
+  for (; kt0 < KT; kt0 += S) rotation(std::false_type{}, kt0);
 
-  const float sb = g.scale_b[0];
-  const float sa0 = g.a_per_row ? 0.f : g.scale_a[0];
-  OutT* out = reinterpret_cast<OutT*>(g.out);
-#pragma unroll
-  for (int i = 0; i < WM; ++i) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-      const int64_t row = row0 + (wm * WM + i) * 32 + 8 * (e >> 2) + 4 * (lane >> 5) + (e & 3);
-      if (row >= g.M) continue;
-      const float sa = g.a_per_row ? g.scale_a[row] : sa0;
-#pragma unroll
-      for (int j = 0; j < WN; ++j) {
-        const int64_t col = col0 + (wn * WN + j) * 32 + (lane & 31);
-        if (col >= g.N) continue;
-        int a = acc[i][j][e];
-        if constexpr (BITS == 4) a >>= 8;
-        if (g.acc_out) g.acc_out[row * g.N + col] = a;
-        const float v = (((float)a * sa) * sb) * g.post_scale;
-        store_scalar<OutT>(out + row * g.ldo + col, v);
-      }
-    }
-  }
+  gemm_epilogue<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb);
 }
 
 template <int WM, int WN, int BITS, int S, typename OutT>
@@ -428,6 +495,7 @@ static int launch_gemm_pipe(GemmArgs& g, hipStream_t st) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
   g.tiles_m = (int)((g.M + BM - 1) / BM);
   g.tiles_n = (int)((g.N + BN - 1) / BN);
+  g.group_m = pick_group_m(g.tiles_m, g.tiles_n, S == 3 && WM * WN <= 4 ? 3 : 1);
   const int64_t total = (int64_t)g.tiles_m * g.tiles_n;
   if (total > (1 << 30)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: too many tiles");
   if (g.M * g.lda >= (1ll << 32) || g.N * g.ldb >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: operand larger than 4 GiB");
@@ -440,6 +508,7 @@ static int launch_gemm(GemmArgs& g, hipStream_t st) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
   g.tiles_m = (int)((g.M + BM - 1) / BM);
   g.tiles_n = (int)((g.N + BN - 1) / BN);
+  g.group_m = pick_group_m(g.tiles_m, g.tiles_n, 1);
   const size_t lds = (size_t)2 * (BM + BN) * G_PITCH;
   static bool attr_done = false;  // one-time, read-only afterwards
   if (!attr_done) {
@@ -470,12 +539,15 @@ static int pick_tile(GemmArgs& g, hipStream_t st) {
     case 22: return launch_gemm<2, 2, BITS, OutT>(g, st);
     default: break;
   }
-  // 128 x 128 tiles.  With more tiles than CUs, three LDS stages let three workgroups share a CU
-  // and hide each other's stalls; with fewer, a lone workgroup per CU prefers the deeper prefetch of
-  // four stages.  The DMA kernel addresses operands with 32-bit offsets; larger operands take the
-  // register-staged kernel.
+  // 128 x 128 tiles by default.  With more tiles than CUs, three LDS stages let three workgroups
+  // share a CU and hide each other's stalls; with fewer, a lone workgroup per CU prefers the deeper
+  // prefetch of four stages.  Problems with at least two full rounds of 256 x 256 tiles take those:
+  // half the operand traffic per multiply-add.  The DMA kernel addresses operands with 32-bit
+  // offsets; larger operands take the register-staged kernel.
   if (g.M * g.lda < (1ll << 32) && g.N * g.ldb < (1ll << 32)) {
     const int64_t tiles = ((g.M + 127) / 128) * ((g.N + 127) / 128);
+    const int64_t big = ((g.M + 255) / 256) * ((g.N + 255) / 256);
+    if (big >= 512) return launch_gemm_pipe<4, 4, BITS, 4, OutT>(g, st);
     return tiles > 256 ? launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st) : launch_gemm_pipe<2, 2, BITS, 4, OutT>(g, st);
   }
   return launch_gemm<2, 2, BITS, OutT>(g, st);
@@ -511,6 +583,7 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
   g.ktiles = (int)(kpad / G_BK);
   g.scale_a = scale_a; g.scale_b = scale_b; g.post_scale = post_scale; g.a_per_row = a_per_row;
   g.out = out; g.ldo = ldo; g.acc_out = acc_out;
+  g.vec_out = ((ldo & 3) == 0 && ((uintptr_t)out & 15) == 0) ? 1 : 0;
   return bits == 4 ? dispatch_out<4>(out_dtype, g, st) : dispatch_out<8>(out_dtype, g, st);
 }
 
