@@ -8,6 +8,8 @@
 // forward-side activation buffer of FLinearQ.setup_context (:178-212).
 #include <string.h>
 
+#include <mutex>
+
 #include "hot_device.h"
 #include "hot_host.h"
 
@@ -43,7 +45,8 @@ static int check_cfg(const hot_config* c, const char* who) {
 
 struct BwdLayout {
   int64_t ld_g, ld_w, ld_gp;                       // code pitches in bytes
-  size_t off_hq, off_colw, off_colg, off_sg, off_sw, off_sgp, off_qg, off_qw, off_qgp, total;
+  size_t off_hq, off_colw, off_colg, off_sg, off_sw, off_sgp, off_qg, off_qw, off_qgp, off_split, total;
+  size_t split_bytes;                            // split-K workspace shared by the two GEMMs
 };
 
 static size_t align256(size_t v) { return (v + 255) & ~(size_t)255; }
@@ -64,6 +67,9 @@ static BwdLayout bwd_layout(int64_t L, int64_t O, int64_t I, const hot_config* c
   b.off_qg = o;   o += align256((size_t)L * b.ld_g);
   b.off_qw = o;   o += align256((size_t)I * b.ld_w);
   b.off_qgp = o;  o += align256((size_t)O * b.ld_gp);
+  const GemmSplit px = gemm_split_plan(L, I, O, c->gx_bits), pw = gemm_split_plan(O, I, lp, 8);
+  b.split_bytes = px.ws_bytes > pw.ws_bytes ? px.ws_bytes : pw.ws_bytes;
+  b.off_split = o; o += align256(b.split_bytes);
   b.total = o;
   return b;
 }
@@ -163,6 +169,31 @@ enum {
   K_COUNT = 8
 };
 
+// The two W kernels are small (a few MB) and cannot fill the chip; they run on a side stream beside
+// the g_y kernels.  One side stream and two events per device, created on first use (default
+// priority) and kept for the life of the process; a mutex keeps the fork / join of one call together.
+struct SideLane {
+  hipStream_t stream = nullptr;
+  hipEvent_t fork = nullptr, join = nullptr;
+  bool tried = false, ok = false;
+};
+static std::mutex g_side_mutex;
+static SideLane g_side[64];
+
+static SideLane* side_lane_locked() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  SideLane& s = g_side[dev];
+  if (!s.tried) {
+    s.tried = true;
+    s.ok = hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) == hipSuccess &&
+           hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) == hipSuccess &&
+           hipEventCreateWithFlags(&s.join, hipEventDisableTiming) == hipSuccess;
+    if (!s.ok) (void)hipGetLastError();
+  }
+  return s.ok ? &s : nullptr;
+}
+
 static int run_backward(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,
                         int64_t O, int64_t I, const hot_config* cfg, void* gx, void* gw, int out_dtype,
                         void* workspace, size_t workspace_bytes, hipEvent_t* ev /* K_COUNT + 1 or null */,
@@ -196,11 +227,34 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
                        (uint32_t*)(ws + b.off_hq), n0, (uint32_t*)(ws + b.off_colw), n1, (uint32_t*)(ws + b.off_colg), n2);
   }
   mark(K_CLEAR + 1);
+  // W: Hadamard along O + quantise, stored [I, O]
+  auto quantise_w = [&](hipStream_t s2) {
+    return colwise_quant_impl(w, dtype, O, I, cfg->n_o, identity_rows(), cfg->n_o, cfg->w_bits, cfg->w_round, cfg->seed,
+                              HOT_STREAM_W, cfg->w_scale, ws + b.off_qw, b.ld_w, cfg->w_bits == 4, sw,
+                              ws + b.off_colw, colwise_workspace_bytes_impl(I), s2, who, nullptr, /*stats_cleared=*/true,
+                              ev ? ev[K_W_STATS + 1] : nullptr);
+  };
+  // Without per-kernel timing the W kernels overlap the g_y kernels on the side stream.
+  std::unique_lock<std::mutex> side_guard(g_side_mutex, std::defer_lock);
+  SideLane* side = nullptr;
+  if (!ev) {
+    side_guard.lock();
+    side = side_lane_locked();
+    if (!side) side_guard.unlock();
+  }
+  int rc = HOT_OK;
+  if (side) {
+    rc = check_hip(hipEventRecord(side->fork, st), "hipEventRecord");
+    if (!rc) rc = check_hip(hipStreamWaitEvent(side->stream, side->fork, 0), "hipStreamWaitEvent");
+    if (!rc) rc = quantise_w(side->stream);
+    if (!rc) rc = check_hip(hipEventRecord(side->join, side->stream), "hipEventRecord");
+    if (rc) return rc;
+  }
   // g_y: HLA along tokens + quantise, transposed (g_W operand); Hadamard along O + quantise (g_x
   // operand).  With one step per tensor both quantisers need the absmax of their transform first:
   // the statistics pass of the token-wise kernel delivers both from a single read of g_y.
   const bool fuse = cfg->gx_scale == HOT_SCALE_TENSOR && cfg->n_o == 16 && O % 16 == 0 && cfg->gw_scale != HOT_SCALE_SAWB;
-  int rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->gw_bits, cfg->gw_round,
+  rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->gw_bits, cfg->gw_round,
                               cfg->seed, HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp,
                               ws + b.off_colg, colwise_workspace_bytes_impl(O), st, who,
                               fuse ? (float*)(ws + b.off_hq) : nullptr, /*stats_cleared=*/true,
@@ -211,21 +265,24 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
                        cfg->gx_scale, ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, 256, st, fuse);
   if (rc) return rc;
   mark(K_GY_HQ + 1);
-  // W: Hadamard along O + quantise, stored [I, O]
-  rc = colwise_quant_impl(w, dtype, O, I, cfg->n_o, identity_rows(), cfg->n_o, cfg->w_bits, cfg->w_round, cfg->seed,
-                          HOT_STREAM_W, cfg->w_scale, ws + b.off_qw, b.ld_w, cfg->w_bits == 4, sw,
-                          ws + b.off_colw, colwise_workspace_bytes_impl(I), st, who, nullptr, /*stats_cleared=*/true,
-                          ev ? ev[K_W_STATS + 1] : nullptr);
-  if (rc) return rc;
+  if (side) {
+    rc = check_hip(hipStreamWaitEvent(st, side->join, 0), "hipStreamWaitEvent");
+    if (rc) return rc;
+  } else {
+    rc = quantise_w(st);
+    if (rc) return rc;
+  }
   mark(K_W_QUANT + 1);
   // g_x = (qG . qW^T) sG sW / n_o
   rc = gemm_i8_impl(ws + b.off_qg, b.ld_g, ws + b.off_qw, b.ld_w, cfg->gx_bits, L, I, O, sg,
-                    cfg->gx_scale == HOT_SCALE_ROW, sw, 1.0f / (float)cfg->n_o, gx, out_dtype, I, nullptr, st);
+                    cfg->gx_scale == HOT_SCALE_ROW, sw, 1.0f / (float)cfg->n_o, gx, out_dtype, I, nullptr, st,
+                    b.split_bytes ? ws + b.off_split : nullptr, b.split_bytes);
   if (rc) return rc;
   mark(K_GEMM_GX + 1);
   // g_W = (qGp . xq^T) sGp sx / hla_n
   rc = gemm_i8_impl(ws + b.off_qgp, b.ld_gp, xq, b.ld_gp, 8, O, I, lp, sgp, cfg->gw_scale == HOT_SCALE_ROW, sx,
-                    1.0f / (float)cfg->hla_n, gw, out_dtype, I, nullptr, st);
+                    1.0f / (float)cfg->hla_n, gw, out_dtype, I, nullptr, st,
+                    b.split_bytes ? ws + b.off_split : nullptr, b.split_bytes);
   if (rc) return rc;
   mark(K_GEMM_GW + 1);
   return HOT_OK;

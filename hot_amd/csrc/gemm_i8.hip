@@ -49,6 +49,8 @@ struct GemmArgs {
   int32_t tiles_m, tiles_n;
   int32_t group_m;   // tile rows per group of the launch order (tile_of)
   int32_t vec_out;   // out and ldo allow aligned four-element stores
+  int32_t splits;    // K is cut into this many ranges, one workgroup each (1 = no split)
+  v4i* partials;     // [tile][range][wave][fragment quad][lane]: raw accumulators of the ranges
 };
 
 // Workgroup -> tile.  Hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with
@@ -334,8 +336,10 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
+  const int tiles_total = g.tiles_m * g.tiles_n;
+  const int split = (int)blockIdx.x / tiles_total, tile_id = (int)blockIdx.x - split * tiles_total;
   int tm, tn;
-  tile_of(g, blockIdx.x, tm, tn);
+  tile_of(g, tile_id, tm, tn);
   const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
   float sa_row[WM];
   load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
@@ -358,10 +362,15 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
       goff[i] = (uint32_t)(gr * g.ldb + slot * 16);
     }
   }
+  // stages of this workgroup: its K range of the G_BK-code tiles, in 64-byte steps
+  const int kt_all = g.ktiles * (G_BK / (BITS == 8 ? 64 : 128));
+  const int kt_per = (kt_all + g.splits - 1) / g.splits;
+  const int kt_begin = split * kt_per;
+  const int KT = kt_all - kt_begin < kt_per ? kt_all - kt_begin : kt_per;
   auto issue = [&](const uint8_t* stage, int kt) {
     const uint32_t l0 = lds_offset(stage) + wave * 1024;
-    const uint8_t* ga = g.A + (int64_t)kt * GSTEP;
-    const uint8_t* gb = g.B + (int64_t)kt * GSTEP;
+    const uint8_t* ga = g.A + (int64_t)(kt_begin + kt) * GSTEP;
+    const uint8_t* gb = g.B + (int64_t)(kt_begin + kt) * GSTEP;
 #pragma unroll
     for (int i = 0; i < LPW; ++i) dma16(l0 + i * 4096, goff[i], i < BM / 64 ? ga : gb);
   };
@@ -418,7 +427,6 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
     }
   };
 
-  const int KT = g.ktiles * (G_BK / (BITS == 8 ? 64 : 128));   // stages of this kernel per G_BK-code tile
   // prologue: S - 1 tiles in flight, tile 0 landed and visible, its first round in registers
   static_for<S - 1>([&](auto k) {
     if (k.value < KT) issue(ring + k.value * STAGE_BYTES, k.value);
@@ -487,6 +495,61 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
   for (; kt0 + 2 * S - 2 < KT; kt0 += S) rotation(std::true_type{}, kt0);   // every issue inside is in range
   for (; kt0 < KT; kt0 += S) rotation(std::false_type{}, kt0);
 
+  if (g.splits > 1) {
+    // Split K: every range leaves its raw accumulators in the workspace (lane-major, so each store
+    // is one contiguous KiB per wave); gemm_i8_reduce_kernel adds them up and runs the epilogue.
+    constexpr int QUADS = WM * WN * 4;
+    v4i* mine = g.partials + (((int64_t)tile_id * g.splits + split) * 4 + wave) * (QUADS * 64) + lane;
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          v4i c = {acc[i][j][4 * q], acc[i][j][4 * q + 1], acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]};
+          mine[((i * WN + j) * 4 + q) * 64] = c;
+        }
+    return;
+  }
+
+  gemm_epilogue<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb);
+}
+
+// Second kernel of a split-K product: one workgroup per output tile, thread for thread the layout
+// of the pipelined kernel, so each thread adds up the accumulators its twins left in the workspace
+// (integer sums: any order gives the same result) and runs the same epilogue.
+template <int WM, int WN, int BITS, typename OutT>
+__global__ void __launch_bounds__(G_THREADS) gemm_i8_reduce_kernel(const GemmArgs g) {
+  constexpr int BM = 64 * WM, BN = 64 * WN, QUADS = WM * WN * 4;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int tile_id = blockIdx.x;
+  int tm, tn;
+  tile_of(g, tile_id, tm, tn);
+  const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
+  float sa_row[WM];
+  load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
+  const float sb = g.scale_b[0];
+  v16i acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+  for (int s2 = 0; s2 < g.splits; ++s2) {
+    const v4i* part = g.partials + (((int64_t)tile_id * g.splits + s2) * 4 + wave) * (QUADS * 64) + lane;
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const v4i c = part[((i * WN + j) * 4 + q) * 64];
+#pragma unroll
+          for (int t = 0; t < 4; ++t) acc[i][j][4 * q + t] += c[t];
+        }
+  }
   gemm_epilogue<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb);
 }
 
@@ -499,7 +562,12 @@ static int launch_gemm_pipe(GemmArgs& g, hipStream_t st) {
   const int64_t total = (int64_t)g.tiles_m * g.tiles_n;
   if (total > (1 << 30)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: too many tiles");
   if (g.M * g.lda >= (1ll << 32) || g.N * g.ldb >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: operand larger than 4 GiB");
-  hipLaunchKernelGGL((gemm_i8_pipe_kernel<WM, WN, BITS, S, OutT>), dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
+  hipLaunchKernelGGL((gemm_i8_pipe_kernel<WM, WN, BITS, S, OutT>), dim3((unsigned)(total * g.splits)), dim3(G_THREADS), 0, st, g);
+  if (g.splits > 1) {
+    if (int rc = check_launch("gemm_i8_pipe_kernel")) return rc;
+    hipLaunchKernelGGL((gemm_i8_reduce_kernel<WM, WN, BITS, OutT>), dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
+    return check_launch("gemm_i8_reduce_kernel");
+  }
   return check_launch("gemm_i8_pipe_kernel");
 }
 
@@ -523,10 +591,41 @@ static int launch_gemm(GemmArgs& g, hipStream_t st) {
   return check_launch("gemm_i8_kernel");
 }
 
-template <int BITS, typename OutT>
-static int pick_tile(GemmArgs& g, hipStream_t st) {
+static int forced_tile() {   // experiments: HOT_GEMM_TILE picks one kernel variant for every problem
   static int forced = -1;
   if (forced < 0) { const char* e = getenv("HOT_GEMM_TILE"); forced = e ? atoi(e) : 0; }
+  return forced;
+}
+
+// Split K when the 128 x 128 tiles cannot fill the chip: up to two workgroups per CU, at least 16
+// stages of 64 bytes per range.
+GemmSplit gemm_split_plan(int64_t M, int64_t N, int64_t K, int bits) {
+  GemmSplit p; p.splits = 1; p.ws_bytes = 0;
+  if (M <= 0 || N <= 0 || K <= 0) return p;
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+  const int64_t stages = round_up(K, GEMM_KTILE) / (bits == 8 ? 64 : 128);
+  static int forced = -1;   // experiments: HOT_GEMM_SPLITK overrides the rule (1 = never split)
+  if (forced < 0) { const char* e = getenv("HOT_GEMM_SPLITK"); forced = e ? atoi(e) : 0; }
+  int64_t sk = 1;
+  if (tiles < 256) {
+    sk = 512 / tiles;                        // about two workgroups per CU
+    if (sk > stages / 16) sk = stages / 16;
+    if (sk > 8) sk = 8;
+    if (forced > 0) sk = forced;
+  }
+  if (sk > stages) sk = stages;
+  if (sk < 2) return p;
+  const int64_t per = (stages + sk - 1) / sk;
+  sk = (stages + per - 1) / per;            // no empty range
+  if (sk < 2) return p;
+  p.splits = (int)sk;
+  p.ws_bytes = (size_t)tiles * (size_t)sk * (128 * 128 * 4);
+  return p;
+}
+
+template <int BITS, typename OutT>
+static int pick_tile(GemmArgs& g, hipStream_t st) {
+  const int forced = forced_tile();
   switch (forced) {
     case 144: return launch_gemm_pipe<4, 4, BITS, 4, OutT>(g, st);
     case 142: return launch_gemm_pipe<4, 2, BITS, 4, OutT>(g, st);
@@ -545,6 +644,7 @@ static int pick_tile(GemmArgs& g, hipStream_t st) {
   // half the operand traffic per multiply-add.  The DMA kernel addresses operands with 32-bit
   // offsets; larger operands take the register-staged kernel.
   if (g.M * g.lda < (1ll << 32) && g.N * g.ldb < (1ll << 32)) {
+    if (g.splits > 1) return launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st);
     const int64_t tiles = ((g.M + 127) / 128) * ((g.N + 127) / 128);
     const int64_t big = ((g.M + 255) / 256) * ((g.N + 255) / 256);
     if (big >= 512) return launch_gemm_pipe<4, 4, BITS, 4, OutT>(g, st);
@@ -565,7 +665,8 @@ static int dispatch_out(int out_dtype, GemmArgs& g, hipStream_t st) {
 
 int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bits, int64_t M, int64_t N,
                  int64_t K, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
-                 void* out, int out_dtype, int64_t ldo, int32_t* acc_out, hipStream_t st) {
+                 void* out, int out_dtype, int64_t ldo, int32_t* acc_out, hipStream_t st, void* split_ws,
+                 size_t split_ws_bytes) {
   if (!A || !B || !scale_a || !scale_b || !out) return fail(HOT_ERR_INVALID, "hot_gemm_i8: null pointer");
   if (M < 0 || N < 0 || K <= 0) return fail(HOT_ERR_INVALID, "hot_gemm_i8: bad shape %lld x %lld x %lld", (long long)M, (long long)N, (long long)K);
   if (bits != 4 && bits != 8) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: bits=%d (4 or 8)", bits);
@@ -584,6 +685,13 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
   g.scale_a = scale_a; g.scale_b = scale_b; g.post_scale = post_scale; g.a_per_row = a_per_row;
   g.out = out; g.ldo = ldo; g.acc_out = acc_out;
   g.vec_out = ((ldo & 3) == 0 && ((uintptr_t)out & 15) == 0) ? 1 : 0;
+  g.splits = 1; g.partials = nullptr;
+  const GemmSplit plan = gemm_split_plan(M, N, K, bits);
+  if (plan.splits > 1 && split_ws && split_ws_bytes >= plan.ws_bytes && M * lda < (1ll << 32) && N * ldb < (1ll << 32) &&
+      forced_tile() == 0) {
+    g.splits = plan.splits;
+    g.partials = (v4i*)split_ws;
+  }
   return bits == 4 ? dispatch_out<4>(out_dtype, g, st) : dispatch_out<8>(out_dtype, g, st);
 }
 

@@ -37,6 +37,12 @@ size_t colwise_stats_bytes_impl(int64_t C);  // leading part of the workspace th
 
 int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bits, int64_t M, int64_t N,
                  int64_t K, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
-                 void* out, int out_dtype, int64_t ldo, int32_t* acc_out, hipStream_t st);
+                 void* out, int out_dtype, int64_t ldo, int32_t* acc_out, hipStream_t st, void* split_ws = nullptr,
+                 size_t split_ws_bytes = 0);
+
+// Split-K plan of gemm_i8_impl for a problem: `splits` K ranges (1 = none) and the bytes of workspace
+// that hold their partial accumulators (16-byte aligned; contents need no initialisation).
+struct GemmSplit { int splits; size_t ws_bytes; };
+GemmSplit gemm_split_plan(int64_t M, int64_t N, int64_t K, int bits);
 
 }  // namespace hot

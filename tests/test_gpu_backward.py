@@ -87,6 +87,24 @@ def test_backward_matches_oracle(gpu, dtype, shape, variant):
         assert torch.equal(gw.cpu(), torch.from_numpy(tr.g_w).to(dtype))
 
 
+@pytest.mark.parametrize("variant", [dict(), dict(gw_scale=orc.SCALE_ROW, gx_bits=8, w_bits=8)])
+def test_backward_split_k(gpu, variant):
+    """Few output tiles and a long reduction (L' = 2304): the g_W GEMM cuts K into ranges that meet
+    in the workspace and a second kernel adds up.  Run twice on one (dirty) workspace."""
+    from hot_amd import ops
+    L, O, I = 4096, 256, 256
+    x, w, gy = make_case(L, O, I, seed=5)
+    ocfg, opt = both_configs(L, **variant)
+    assert opt.lprime(L) >= 2048
+    gx, gw, tr = run_both(x, w, gy, ocfg, opt, gpu)
+    assert np.array_equal(gx.cpu().numpy(), tr.g_x) and np.array_equal(gw.cpu().numpy(), tr.g_w)
+    xq, sx = ops.abc_forward(x.to(gpu), opt)
+    ws = torch.empty(1 << 26, dtype=torch.uint8, device=gpu)
+    for _ in range(2):
+        gx2, gw2 = ops.linear_backward(gy.to(gpu), w.to(gpu), xq, sx, opt, workspace=ws)
+        assert np.array_equal(gx2.cpu().numpy(), tr.g_x) and np.array_equal(gw2.cpu().numpy(), tr.g_w)
+
+
 def test_backward_paper_rule(gpu):
     L, O, I = 512, 256, 128
     x, w, gy = make_case(L, O, I, seed=1)
