@@ -17,8 +17,11 @@ actQuantBit = 8      # P x              (g_W path, B operand; the saved buffer)
 
 eps = 1e-11
 
+precisionScheduling = False   # utils.precision_scheduler drives the bit widths per epoch
+milestone = " "
+
 quantAuto = False
-quantBWDGogi = "int"   # int | stoch | nq
+quantBWDGogi = "int"   # int | stoch | nq      ("no" on all four + Transform* off = plain layer)
 quantBWDWgt = "int"    # int | stoch | sawb
 quantBWDGogw = "int"   # int | stoch | nq
 quantBWDAct = "int"    # int | stoch | sawb

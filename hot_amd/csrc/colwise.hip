@@ -272,7 +272,10 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   // one step: wait for its rows, let the ring advance, pull this thread's 16 values into x[xo..]
   auto step = [&](int s, float* dst) {
     // this wave's share of step s has landed, and its own LDS reads of step s-1 are complete ...
-    if (s + 2 < nsteps) wait_stream<2 * LPW>(); else if (s + 1 < nsteps) wait_stream<LPW>(); else wait_stream<0>();
+    // steps s+1 .. s+CW_DEPTH-2 may still be in flight
+    if (CW_DEPTH >= 4 && s + 2 < nsteps) wait_stream<2 * LPW>();
+    else if (CW_DEPTH >= 3 && s + 1 < nsteps) wait_stream<LPW>();
+    else wait_stream<0>();
     __builtin_amdgcn_s_barrier();   // ... and so for every wave: the buffer of step s-1 may be refilled
     if (s + CW_DEPTH - 1 < nsteps) rs_issue<T>(rs, lds0 + ((s + CW_DEPTH - 1) % CW_DEPTH) * BUF, s + CW_DEPTH - 1, wave, lane);
     rs_column<T>(lds + (s % CW_DEPTH) * BUF, tid, dst);

@@ -6,7 +6,13 @@ utils/quant_matmul.py:169-422, so that
 unchanged.  Forward stays full precision (:173-175); ``setup_context`` writes
 the INT8 Hadamard-compressed activation buffer (:178-212) with the native
 kernel and ``backward`` (:215-348, scheme gih_gwlr) calls the fused native op.
-There is no eager fallback: on a CPU tensor the native path raises.
+``HQ_Conv2d`` (:426-488) lowers a convolution to the same Function by im2col.
+
+With every Transform* flag off and every quantBWD* flag "no" the reference's
+Function is an ordinary full-precision linear layer (its branches all fall
+through); that setting is kept, because the layer-wise quantizer selection
+calibrates in it.  Any other partial setting raises: there is no eager
+stand-in for the HOT path, and on a CPU tensor the native path raises.
 """
 from __future__ import annotations
 
@@ -55,6 +61,14 @@ def token_rule(tokens: int):
     return n, rows
 
 
+def hot_switched_off() -> bool:
+    """True when args describes the reference's plain full-precision layer: no transform, no
+    quantiser (the state of args.py:40-49 before a recipe is applied)."""
+    off = (False, "no", None)
+    return (not (args.TransformGogi or args.TransformWgt or args.TransformGogw or args.TransformInput)
+            and all(getattr(args, k) in off for k in ("quantBWDGogi", "quantBWDWgt", "quantBWDGogw", "quantBWDAct")))
+
+
 def options_for(tokens: int, layer_name: str = " ") -> ops.HotOptions:
     """args.* -> HotOptions, following the branch structure of FLinearQ."""
     if args.transform_scheme != "gih_gwlr":
@@ -94,6 +108,10 @@ class FLinearQ(Function):
         x, w, _h_out, _h_bs, name = inputs
         ctx.name = name
         ctx.x_shape = tuple(x.shape)
+        ctx.full_precision = hot_switched_off()
+        if ctx.full_precision:
+            ctx.save_for_backward(x, w)
+            return
         if x.dim() == 3 and args.batched_mode == "per_sample":
             tokens = x.shape[1]
             opt = options_for(tokens, name)
@@ -110,6 +128,13 @@ class FLinearQ(Function):
 
     @staticmethod
     def backward(ctx, grad_output):
+        if ctx.full_precision:
+            x, w = ctx.saved_tensors
+            go = grad_output.to(w.dtype)
+            grad_w = go.mT @ x.to(w.dtype)
+            if grad_w.dim() == 3:                    # [B, O, I]: the sum over samples autograd would take
+                grad_w = grad_w.sum(dim=0)
+            return go @ w, grad_w, None, None, None
         xq, w, sx = ctx.saved_tensors
         opt = ctx.opt
         go = grad_output
@@ -170,4 +195,33 @@ class HQ_Linear(nn.Linear):
         output = FLinearQ.apply(input, self.weight, self.hadamard_out, self.hadamard_bs, self.layer_name)
         if self.bias is not None:
             output = output + self.bias.to(output.device)
+        return output
+
+
+class HQ_Conv2d(nn.Conv2d):
+    """nn.Conv2d (groups = 1) whose backward runs the HOT path: unfold to [B, H'W', C k k], the
+    same Function as HQ_Linear with the weight viewed as [O, C k k], fold back
+    (utils/quant_matmul.py:426-488).  Tokens are the output positions of one sample."""
+
+    def __init__(self, in_channels, out_channels, kernel_size, stride=1, padding=0, dilation=1, groups=1,
+                 bias=True, padding_mode="zeros") -> None:
+        super().__init__(in_channels, out_channels, kernel_size, stride, padding, dilation, groups, bias, padding_mode)
+        self.register_buffer("hadamard_out", torch.tensor(TD.get_or_register("hadamard", self.out_channels),
+                                                          dtype=self.weight.dtype), persistent=False)
+        self.register_buffer("hadamard_bs", torch.zeros((1, 1), dtype=self.weight.dtype), persistent=False)
+        self.layer_name = " "
+
+    def forward(self, input: Tensor) -> Tensor:
+        if self.groups > 1:                          # depth-wise convolution
+            raise NotImplementedError
+        B, _, H, W = input.shape
+        cols = F.unfold(input, self.kernel_size, dilation=self.dilation, padding=self.padding,
+                        stride=self.stride).transpose(1, 2)              # [B, H'W', C k k]
+        weight = self.weight.view(self.weight.size(0), -1)
+        output = FLinearQ.apply(cols, weight, self.hadamard_out, self.hadamard_bs, self.layer_name)
+        ho = (H + 2 * self.padding[0] - self.dilation[0] * (self.kernel_size[0] - 1) - 1) // self.stride[0] + 1
+        wo = (W + 2 * self.padding[1] - self.dilation[1] * (self.kernel_size[1] - 1) - 1) // self.stride[1] + 1
+        output = output.transpose(1, 2).reshape(B, self.out_channels, ho, wo)
+        if self.bias is not None:
+            output = output + self.bias.view(1, -1, 1, 1)
         return output

@@ -269,6 +269,67 @@ def test_hq_linear_3d_input(gpu, fresh_args, mode):
         assert np.array_equal(lin.weight.grad.cpu().numpy(), tr.g_w)
 
 
+def test_hq_conv2d_matches_oracle(gpu, fresh_args):
+    """HQ_Conv2d = im2col + the linear path per sample (utils/quant_matmul.py:426-488): the weight
+    gradient is the sum of the per-sample oracle results, the input gradient their fold."""
+    from hot_amd.quant_matmul import HQ_Conv2d
+    B, C, H, W, O, k = 2, 8, 16, 16, 32, 2
+    torch.manual_seed(2)
+    conv = HQ_Conv2d(C, O, kernel_size=k, stride=k).to(gpu)
+    ref = torch.nn.Conv2d(C, O, kernel_size=k, stride=k).to(gpu)
+    ref.load_state_dict({n: p for n, p in conv.state_dict().items() if n in ("weight", "bias")})
+    x = torch.randn(B, C, H, W, device=gpu, requires_grad=True)
+    y = conv(x)
+    assert torch.allclose(y, ref(x), atol=1e-5, rtol=1e-5)
+    G = torch.randn_like(y) * 1e-3
+    y.backward(G)
+    L = (H // k) * (W // k)
+    ocfg, _ = both_configs(L)
+    cols = torch.nn.functional.unfold(x.detach().cpu(), k, stride=k).transpose(1, 2)       # [B, L, C k k]
+    gy = G.cpu().flatten(2).transpose(1, 2)                                                # [B, L, O]
+    wn = conv.weight.detach().cpu().reshape(O, -1).numpy()
+    gw, gcols = 0, []
+    for b in range(B):
+        xq_ref, sx_ref = orc.abc_forward(cols[b].contiguous().numpy(), ocfg)
+        tr = orc.linear_backward(gy[b].contiguous().numpy(), wn, xq_ref, sx_ref, ocfg)
+        gw = gw + tr.g_w
+        gcols.append(torch.from_numpy(tr.g_x))
+    # stride == kernel: the patches do not overlap, so the fold only moves values
+    gx = torch.nn.functional.fold(torch.stack(gcols).transpose(1, 2), (H, W), k, stride=k)
+    assert np.array_equal(x.grad.cpu().numpy(), gx.numpy())
+    assert rel(conv.weight.grad.cpu().reshape(O, -1).numpy(), gw) < 1e-6
+    assert torch.allclose(conv.bias.grad.cpu(), G.cpu().sum((0, 2, 3)), rtol=1e-4, atol=1e-7)
+
+
+def test_lqs_then_hot_training_step(gpu, fresh_args):
+    """Calibrate in the plain setting, then take a HOT step with the selected quantisers."""
+    from hot_amd import lqs, utils as hutils
+    from hot_amd.quant_matmul import HQ_Linear
+    torch.manual_seed(3)
+    model = torch.nn.Sequential(torch.nn.Linear(64, 128), torch.nn.GELU(), torch.nn.Linear(128, 32)).to(gpu)
+    hutils.replace_layers(model, torch.nn.Linear, HQ_Linear)
+    hutils.name_layers(model)
+    fresh_args.layer_quant_dict.clear()
+    batches = [(torch.randn(256, 64, device=gpu), torch.randint(0, 32, (256,), device=gpu))]
+    chosen = lqs.calibrate(model, batches, torch.nn.CrossEntropyLoss())
+    assert set(chosen) == {"0_gx", "0_gw", "2_gx", "2_gw"}
+    fresh_args.quantAuto = True
+    model.zero_grad()
+    x, t = batches[0]
+    torch.nn.functional.cross_entropy(model(x), t).backward()
+    hot = [p.grad.clone() for p in model.parameters()]
+    # the same step in the plain setting: the HOT gradients approximate it
+    for k_ in ("TransformGogi", "TransformWgt", "TransformGogw", "TransformInput"):
+        setattr(fresh_args, k_, False)
+    for k_ in ("quantBWDGogi", "quantBWDWgt", "quantBWDGogw", "quantBWDAct"):
+        setattr(fresh_args, k_, "no")
+    model.zero_grad()
+    torch.nn.functional.cross_entropy(model(x), t).backward()
+    for h, p in zip(hot, model.parameters()):
+        cos = torch.nn.functional.cosine_similarity(h.flatten(), p.grad.flatten(), dim=0)
+        assert float(cos) > 0.7, float(cos)
+
+
 def test_backward_errors(gpu):
     from hot_amd import ops
     from hot_amd._lib import HotError
