@@ -197,7 +197,7 @@ static SideLane* side_lane_locked() {
 static int run_backward(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,
                         int64_t O, int64_t I, const hot_config* cfg, void* gx, void* gw, int out_dtype,
                         void* workspace, size_t workspace_bytes, hipEvent_t* ev /* K_COUNT + 1 or null */,
-                        hipStream_t st) {
+                        int* slot_of /* K_COUNT: kernel group measured by event pair i, i + 1 */, hipStream_t st) {
   const char* who = "hot_linear_backward";
   if (int e = check_cfg(cfg, who)) return e;
   if (!gy || !w || !xq || !sx || !gx || !gw) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
@@ -216,9 +216,20 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   float* sw = (float*)(ws + b.off_sw);
   float* sgp = (float*)(ws + b.off_sgp);
   const int64_t lp = (L / cfg->hla_n) * cfg->hla_r;
-  auto mark = [&](int slot) { if (ev) (void)hipEventRecord(ev[slot], st); };
-
-  mark(0);
+  // timing: event i + 1 is recorded after the i-th kernel group of the launch order; slot_of[i] names it
+  int seq = 0;
+  auto mark = [&](int slot) {
+    if (!ev) return;
+    slot_of[seq] = slot;
+    (void)hipEventRecord(ev[++seq], st);
+  };
+  // event to record between the two kernels of a token-wise call (statistics pass, quantise pass)
+  auto mid = [&](int slot) -> hipEvent_t {
+    if (!ev) return nullptr;
+    slot_of[seq] = slot;
+    return ev[++seq];
+  };
+  if (ev) (void)hipEventRecord(ev[0], st);
   // one launch zeroes every statistic of the call (absmax slots, per-channel maxima)
   {
     const int n0 = 64, n1 = (int)(colwise_stats_bytes_impl(I) / 4), n2 = (int)(colwise_stats_bytes_impl(O) / 4);
@@ -226,13 +237,13 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
     hipLaunchKernelGGL(clear3_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
                        (uint32_t*)(ws + b.off_hq), n0, (uint32_t*)(ws + b.off_colw), n1, (uint32_t*)(ws + b.off_colg), n2);
   }
-  mark(K_CLEAR + 1);
+  mark(K_CLEAR);
   // W: Hadamard along O + quantise, stored [I, O]
   auto quantise_w = [&](hipStream_t s2) {
     return colwise_quant_impl(w, dtype, O, I, cfg->n_o, identity_rows(), cfg->n_o, cfg->w_bits, cfg->w_round, cfg->seed,
                               HOT_STREAM_W, cfg->w_scale, ws + b.off_qw, b.ld_w, cfg->w_bits == 4, sw,
                               ws + b.off_colw, colwise_workspace_bytes_impl(I), s2, who, nullptr, /*stats_cleared=*/true,
-                              ev ? ev[K_W_STATS + 1] : nullptr);
+                              mid(K_W_STATS));
   };
   // Without per-kernel timing the W kernels overlap the g_y kernels on the side stream.
   std::unique_lock<std::mutex> side_guard(g_side_mutex, std::defer_lock);
@@ -255,36 +266,36 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   // the statistics pass of the token-wise kernel delivers both from a single read of g_y.
   const bool fuse = cfg->gx_scale == HOT_SCALE_TENSOR && cfg->n_o == 16 && O % 16 == 0 && cfg->gw_scale != HOT_SCALE_SAWB;
   rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->gw_bits, cfg->gw_round,
-                              cfg->seed, HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp,
-                              ws + b.off_colg, colwise_workspace_bytes_impl(O), st, who,
-                              fuse ? (float*)(ws + b.off_hq) : nullptr, /*stats_cleared=*/true,
-                              ev ? ev[K_GY_STATS + 1] : nullptr);
+                          cfg->seed, HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp,
+                          ws + b.off_colg, colwise_workspace_bytes_impl(O), st, who,
+                          fuse ? (float*)(ws + b.off_hq) : nullptr, /*stats_cleared=*/true, mid(K_GY_STATS));
   if (rc) return rc;
-  mark(K_GY_HLA + 1);
+  mark(K_GY_HLA);
+  // Each GEMM follows the kernel that wrote its large operand, while that operand is still in the
+  // last-level cache.  g_W = (qGp . xq^T) sGp sx / hla_n
+  rc = gemm_i8_impl(ws + b.off_qgp, b.ld_gp, xq, b.ld_gp, 8, O, I, lp, sgp, cfg->gw_scale == HOT_SCALE_ROW, sx,
+                    1.0f / (float)cfg->hla_n, gw, out_dtype, I, nullptr, st,
+                    b.split_bytes ? ws + b.off_split : nullptr, b.split_bytes);
+  if (rc) return rc;
+  mark(K_GEMM_GW);
   rc = hq_rowwise_impl(gy, dtype, L, O, cfg->n_o, cfg->gx_bits, cfg->gx_round, cfg->seed, HOT_STREAM_GX,
                        cfg->gx_scale, ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, 256, st, fuse);
   if (rc) return rc;
-  mark(K_GY_HQ + 1);
+  mark(K_GY_HQ);
   if (side) {
     rc = check_hip(hipStreamWaitEvent(st, side->join, 0), "hipStreamWaitEvent");
     if (rc) return rc;
   } else {
     rc = quantise_w(st);
     if (rc) return rc;
+    mark(K_W_QUANT);
   }
-  mark(K_W_QUANT + 1);
   // g_x = (qG . qW^T) sG sW / n_o
   rc = gemm_i8_impl(ws + b.off_qg, b.ld_g, ws + b.off_qw, b.ld_w, cfg->gx_bits, L, I, O, sg,
                     cfg->gx_scale == HOT_SCALE_ROW, sw, 1.0f / (float)cfg->n_o, gx, out_dtype, I, nullptr, st,
                     b.split_bytes ? ws + b.off_split : nullptr, b.split_bytes);
   if (rc) return rc;
-  mark(K_GEMM_GX + 1);
-  // g_W = (qGp . xq^T) sGp sx / hla_n
-  rc = gemm_i8_impl(ws + b.off_qgp, b.ld_gp, xq, b.ld_gp, 8, O, I, lp, sgp, cfg->gw_scale == HOT_SCALE_ROW, sx,
-                    1.0f / (float)cfg->hla_n, gw, out_dtype, I, nullptr, st,
-                    b.split_bytes ? ws + b.off_split : nullptr, b.split_bytes);
-  if (rc) return rc;
-  mark(K_GEMM_GW + 1);
+  mark(K_GEMM_GX);
   return HOT_OK;
 }
 
@@ -293,16 +304,18 @@ static int run_backward_timed(const void* gy, const void* w, int dtype, const vo
                               int64_t O, int64_t I, const hot_config* cfg, void* gx, void* gw, int out_dtype,
                               void* workspace, size_t workspace_bytes, float* secs, hipStream_t st) {
   hipEvent_t ev[K_COUNT + 1];
+  int slot_of[K_COUNT];
   for (int i = 0; i <= K_COUNT; ++i) ev[i] = nullptr;
+  for (int i = 0; i < K_COUNT; ++i) { slot_of[i] = -1; secs[i] = 0.f; }
   int rc = HOT_OK;
   for (int i = 0; i <= K_COUNT && !rc; ++i) rc = check_hip(hipEventCreate(&ev[i]), "hipEventCreate");
-  if (!rc) rc = run_backward(gy, w, dtype, xq, sx, L, O, I, cfg, gx, gw, out_dtype, workspace, workspace_bytes, ev, st);
+  if (!rc) rc = run_backward(gy, w, dtype, xq, sx, L, O, I, cfg, gx, gw, out_dtype, workspace, workspace_bytes, ev, slot_of, st);
   if (!rc) rc = check_hip(hipEventSynchronize(ev[K_COUNT]), "hipEventSynchronize");
   if (!rc) {
     for (int i = 0; i < K_COUNT; ++i) {
       float ms = 0.f;
       (void)hipEventElapsedTime(&ms, ev[i], ev[i + 1]);
-      secs[i] = ms * 1e-3f;
+      if (slot_of[i] >= 0) secs[slot_of[i]] = ms * 1e-3f;
     }
   }
   for (int i = 0; i <= K_COUNT; ++i)
@@ -315,7 +328,7 @@ int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq
                         void* workspace, size_t workspace_bytes, float* times4, void* hip_stream) {
   if (!times4)
     return run_backward(gy, w, dtype, xq, sx, L, O, I, cfg, gx, gw, out_dtype, workspace, workspace_bytes, nullptr,
-                        (hipStream_t)hip_stream);
+                        nullptr, (hipStream_t)hip_stream);
   float k[K_COUNT];
   const int rc = run_backward_timed(gy, w, dtype, xq, sx, L, O, I, cfg, gx, gw, out_dtype, workspace, workspace_bytes,
                                     k, (hipStream_t)hip_stream);

@@ -515,42 +515,35 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
   gemm_epilogue<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb);
 }
 
-// Second kernel of a split-K product: one workgroup per output tile, thread for thread the layout
-// of the pipelined kernel, so each thread adds up the accumulators its twins left in the workspace
-// (integer sums: any order gives the same result) and runs the same epilogue.
+// Second kernel of a split-K product: one single-wave workgroup per 32 x 32 accumulator fragment,
+// lane for lane the layout of the pipelined kernel, so each lane adds up the accumulators its twins
+// left in the workspace (integer sums: any order gives the same result) and runs the same epilogue.
 template <int WM, int WN, int BITS, typename OutT>
-__global__ void __launch_bounds__(G_THREADS) gemm_i8_reduce_kernel(const GemmArgs g) {
-  constexpr int BM = 64 * WM, BN = 64 * WN, QUADS = WM * WN * 4;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+__global__ void __launch_bounds__(64) gemm_i8_reduce_kernel(const GemmArgs g) {
+  constexpr int BM = 64 * WM, BN = 64 * WN, QUADS = WM * WN * 4, FRAGS = WM * WN;
+  const int lane = threadIdx.x;
+  const int frag = blockIdx.x % FRAGS, wave = (blockIdx.x / FRAGS) & 3, tile_id = blockIdx.x / (FRAGS * 4);
+  const int fi = frag / WN, fj = frag % WN;
   const int wm = wave >> 1, wn = wave & 1;
-  const int tile_id = blockIdx.x;
   int tm, tn;
   tile_of(g, tile_id, tm, tn);
-  const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
-  float sa_row[WM];
-  load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
+  const int64_t row0 = (int64_t)tm * BM + (wm * WM + fi) * 32, col0 = (int64_t)tn * BN + (wn * WN + fj) * 32;
+  float sa_row[1];
+  load_row_scales<1>(g, row0, lane, sa_row);
   const float sb = g.scale_b[0];
-  v16i acc[WM][WN];
+  v16i acc[1][1];
 #pragma unroll
-  for (int i = 0; i < WM; ++i)
-#pragma unroll
-    for (int j = 0; j < WN; ++j)
-#pragma unroll
-      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+  for (int e = 0; e < 16; ++e) acc[0][0][e] = 0;
   for (int s2 = 0; s2 < g.splits; ++s2) {
-    const v4i* part = g.partials + (((int64_t)tile_id * g.splits + s2) * 4 + wave) * (QUADS * 64) + lane;
+    const v4i* part = g.partials + (((int64_t)tile_id * g.splits + s2) * 4 + wave) * (QUADS * 64) + frag * 4 * 64 + lane;
 #pragma unroll
-    for (int i = 0; i < WM; ++i)
+    for (int q = 0; q < 4; ++q) {
+      const v4i c = part[q * 64];
 #pragma unroll
-      for (int j = 0; j < WN; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const v4i c = part[((i * WN + j) * 4 + q) * 64];
-#pragma unroll
-          for (int t = 0; t < 4; ++t) acc[i][j][4 * q + t] += c[t];
-        }
+      for (int t = 0; t < 4; ++t) acc[0][0][4 * q + t] += c[t];
+    }
   }
-  gemm_epilogue<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb);
+  gemm_epilogue<1, 1, BITS, OutT>(acc, g, row0, col0, lane, sa_row, sb);
 }
 
 template <int WM, int WN, int BITS, int S, typename OutT>
@@ -565,7 +558,7 @@ static int launch_gemm_pipe(GemmArgs& g, hipStream_t st) {
   hipLaunchKernelGGL((gemm_i8_pipe_kernel<WM, WN, BITS, S, OutT>), dim3((unsigned)(total * g.splits)), dim3(G_THREADS), 0, st, g);
   if (g.splits > 1) {
     if (int rc = check_launch("gemm_i8_pipe_kernel")) return rc;
-    hipLaunchKernelGGL((gemm_i8_reduce_kernel<WM, WN, BITS, OutT>), dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
+    hipLaunchKernelGGL((gemm_i8_reduce_kernel<WM, WN, BITS, OutT>), dim3((unsigned)(total * 4 * WM * WN)), dim3(64), 0, st, g);
     return check_launch("gemm_i8_reduce_kernel");
   }
   return check_launch("gemm_i8_pipe_kernel");
