@@ -23,6 +23,7 @@ EXPORTS = (
     "hot_last_error", "hot_abi_version", "hot_kpad", "hot_hq_rowwise", "hot_hla_tokenwise",
     "hot_wq_colwise", "hot_colwise_workspace_bytes", "hot_gemm_i8", "hot_abc_workspace_bytes",
     "hot_abc_forward", "hot_backward_workspace_bytes", "hot_linear_backward", "hot_linear_backward_kernels",
+    "hot_gemm_splits",
 )
 
 
@@ -74,6 +75,8 @@ def _declare(lib):
     lib.hot_linear_backward.restype = i32
     lib.hot_linear_backward.argtypes = [vp, vp, i32, vp, vp, i64, i64, i64, cfgp, vp, vp, i32, vp, sz,
                                         C.POINTER(C.c_float), vp]
+    lib.hot_gemm_splits.restype = i32
+    lib.hot_gemm_splits.argtypes = [i64, i64, i64, i32]
     lib.hot_linear_backward_kernels.restype = i32
     lib.hot_linear_backward_kernels.argtypes = lib.hot_linear_backward.argtypes
 

@@ -100,6 +100,11 @@ const char* hot_last_error(void) { return g_err; }
 int hot_abi_version(void) { return HOT_ABI_VERSION; }
 int64_t hot_kpad(int64_t k) { return round_up(k, GEMM_KTILE); }
 
+int hot_gemm_splits(int64_t M, int64_t N, int64_t K, int bits) {
+  if (bits != 4 && bits != 8) return 1;
+  return gemm_split_plan(M, N, K, bits).splits;
+}
+
 int hot_hq_rowwise(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, int rounding,
                    uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, float* scales_out,
                    void* workspace, size_t workspace_bytes, void* hip_stream) {

@@ -155,6 +155,10 @@ HOT_API int hot_abc_forward(const void* x, int dtype, int64_t L, int64_t I, cons
  *               {transform+quantise of g_y (both operands), transform+quantise
  *               of W, g_x GEMM+dequant, g_W GEMM+dequant}; non-NULL makes the
  *               call synchronise the stream
+ * Without timing, the two W kernels run on a side stream of the library (one per
+ * device, created on first use, default priority) between an event recorded on
+ * `hip_stream` and a wait on it, so they overlap the g_y kernels; everything is
+ * ordered after earlier work on `hip_stream` and before later work on it.
  */
 HOT_API size_t hot_backward_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_config* cfg);
 HOT_API int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq,
@@ -164,12 +168,22 @@ HOT_API int hot_linear_backward(const void* gy, const void* w, int dtype, const 
                         void* hip_stream);
 
 /*
+ * Number of K ranges into which the GEMMs inside hot_linear_backward cut a product of
+ * M x N outputs over K codes of `bits` bits (1 = one kernel; more = a kernel per range
+ * writing int32 partial tiles to the workspace, then a reduce kernel).  Products with
+ * few 128 x 128 output tiles and a long K are cut so that the whole chip takes part.
+ * hot_gemm_i8 itself has no workspace and never splits.  No counterpart in the
+ * reference (its CUTLASS GEMMs run without split-K, HLQ_backward_kernel.cu:236-250).
+ */
+HOT_API int hot_gemm_splits(int64_t M, int64_t N, int64_t K, int bits);
+
+/*
  * hot_linear_backward with a HIP event after every kernel group; synchronises
  * the stream.  times8 (host) receives the seconds of
  *   [0] clearing the statistics          [1] token-wise statistics pass over g_y
  *   [2] token-wise quantise pass (g_y)   [3] row-wise quantise pass(es) (g_y)
  *   [4] statistics pass over W           [5] quantise pass over W
- *   [6] g_x GEMM                         [7] g_W GEMM
+ *   [6] g_x GEMM                         [7] g_W GEMM (both launches when split)
  * The reference has no counterpart beyond the four clock() stage timers its op
  * returns (cuda_measure/HLQ_backward_kernel.cu:717-733); this is the
  * measurement hook of bench.py.
