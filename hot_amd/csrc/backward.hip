@@ -179,7 +179,7 @@ enum {
 // priority) and kept for the life of the process; a mutex keeps the fork / join of one call together.
 struct SideLane {
   hipStream_t stream = nullptr;
-  hipEvent_t fork = nullptr, join = nullptr;
+  hipEvent_t fork = nullptr, fork2 = nullptr, join = nullptr;
   bool tried = false, ok = false;
 };
 static std::mutex g_side_mutex;
@@ -193,6 +193,7 @@ static SideLane* side_lane_locked() {
     s.tried = true;
     s.ok = hipStreamCreateWithFlags(&s.stream, hipStreamNonBlocking) == hipSuccess &&
            hipEventCreateWithFlags(&s.fork, hipEventDisableTiming) == hipSuccess &&
+           hipEventCreateWithFlags(&s.fork2, hipEventDisableTiming) == hipSuccess &&
            hipEventCreateWithFlags(&s.join, hipEventDisableTiming) == hipSuccess;
     if (!s.ok) (void)hipGetLastError();
   }
@@ -250,7 +251,8 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
                               ws + b.off_colw, colwise_workspace_bytes_impl(I), s2, who, nullptr, /*stats_cleared=*/true,
                               mid(K_W_STATS));
   };
-  // Without per-kernel timing the W kernels overlap the g_y kernels on the side stream.
+  // Without per-kernel timing, independent kernels overlap on the side stream: first the W kernels
+  // beside the g_y statistics.
   std::unique_lock<std::mutex> side_guard(g_side_mutex, std::defer_lock);
   SideLane* side = nullptr;
   if (!ev) {
@@ -263,30 +265,56 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
     rc = check_hip(hipEventRecord(side->fork, st), "hipEventRecord");
     if (!rc) rc = check_hip(hipStreamWaitEvent(side->stream, side->fork, 0), "hipStreamWaitEvent");
     if (!rc) rc = quantise_w(side->stream);
-    if (!rc) rc = check_hip(hipEventRecord(side->join, side->stream), "hipEventRecord");
     if (rc) return rc;
   }
   // g_y: HLA along tokens + quantise, transposed (g_W operand); Hadamard along O + quantise (g_x
   // operand).  With one step per tensor both quantisers need the absmax of their transform first:
   // the statistics pass of the token-wise kernel delivers both from a single read of g_y.
   const bool fuse = cfg->gx_scale == HOT_SCALE_TENSOR && cfg->n_o == 16 && O % 16 == 0 && cfg->gw_scale != HOT_SCALE_SAWB;
+  // Side stream, beside the g_W GEMM on the main stream: always the row-wise quantise pass of g_y (a
+  // streaming kernel next to a matrix kernel); the g_x GEMM too when the g_W GEMM has fewer tiles
+  // than the chip has CUs and cannot fill it alone (two large GEMMs only get in each other's way).
+  const bool hq_aside = side != nullptr;
+  const bool gx_aside = side != nullptr && ((O + 127) / 128) * ((I + 127) / 128) < 256;
   rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->gw_bits, cfg->gw_round,
                           cfg->seed, HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp,
                           ws + b.off_colg, colwise_workspace_bytes_impl(O), st, who,
-                          fuse ? (float*)(ws + b.off_hq) : nullptr, /*stats_cleared=*/true, mid(K_GY_STATS));
+                          fuse ? (float*)(ws + b.off_hq) : nullptr, /*stats_cleared=*/true,
+                          hq_aside ? side->fork2 : mid(K_GY_STATS));
   if (rc) return rc;
   mark(K_GY_HLA);
-  // Each GEMM follows the kernel that wrote its large operand, while that operand is still in the
-  // last-level cache.  g_W = (qGp . xq^T) sGp sx / hla_n
+  // g_x operand of g_y on the side stream: a streaming kernel beside the g_W GEMM
+  auto quantise_gy_rows = [&](hipStream_t s2) {
+    return hq_rowwise_impl(gy, dtype, L, O, cfg->n_o, cfg->gx_bits, cfg->gx_round, cfg->seed, HOT_STREAM_GX,
+                           cfg->gx_scale, ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, 256, s2, fuse);
+  };
+  auto gemm_gx = [&](hipStream_t s2) {
+    // g_x = (qG . qW^T) sG sW / n_o   (never split here: the split workspace belongs to the g_W GEMM)
+    return gemm_i8_impl(ws + b.off_qg, b.ld_g, ws + b.off_qw, b.ld_w, cfg->gx_bits, L, I, O, sg,
+                        cfg->gx_scale == HOT_SCALE_ROW, sw, 1.0f / (float)cfg->n_o, gx, out_dtype, I, nullptr, s2,
+                        s2 == st && b.split_bytes ? ws + b.off_split : nullptr, s2 == st ? b.split_bytes : 0);
+  };
+  if (hq_aside) {
+    rc = check_hip(hipStreamWaitEvent(side->stream, side->fork2, 0), "hipStreamWaitEvent");   // statistics are in
+    if (!rc) rc = quantise_gy_rows(side->stream);
+    if (!rc && gx_aside) rc = gemm_gx(side->stream);
+    if (rc) return rc;
+  }
+  if (side) {
+    rc = check_hip(hipEventRecord(side->join, side->stream), "hipEventRecord");
+    if (rc) return rc;
+  }
+  // g_W = (qGp . xq^T) sGp sx / hla_n, right after the kernel that wrote its large operand
   rc = gemm_i8_impl(ws + b.off_qgp, b.ld_gp, xq, b.ld_gp, 8, O, I, lp, sgp, cfg->gw_scale == HOT_SCALE_ROW, sx,
                     1.0f / (float)cfg->hla_n, gw, out_dtype, I, nullptr, st,
                     b.split_bytes ? ws + b.off_split : nullptr, b.split_bytes);
   if (rc) return rc;
   mark(K_GEMM_GW);
-  rc = hq_rowwise_impl(gy, dtype, L, O, cfg->n_o, cfg->gx_bits, cfg->gx_round, cfg->seed, HOT_STREAM_GX,
-                       cfg->gx_scale, ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, 256, st, fuse);
-  if (rc) return rc;
-  mark(K_GY_HQ);
+  if (!hq_aside) {
+    rc = quantise_gy_rows(st);
+    if (rc) return rc;
+    mark(K_GY_HQ);
+  }
   if (side) {
     rc = check_hip(hipStreamWaitEvent(st, side->join, 0), "hipStreamWaitEvent");
     if (rc) return rc;
@@ -295,12 +323,11 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
     if (rc) return rc;
     mark(K_W_QUANT);
   }
-  // g_x = (qG . qW^T) sG sW / n_o
-  rc = gemm_i8_impl(ws + b.off_qg, b.ld_g, ws + b.off_qw, b.ld_w, cfg->gx_bits, L, I, O, sg,
-                    cfg->gx_scale == HOT_SCALE_ROW, sw, 1.0f / (float)cfg->n_o, gx, out_dtype, I, nullptr, st,
-                    b.split_bytes ? ws + b.off_split : nullptr, b.split_bytes);
-  if (rc) return rc;
-  mark(K_GEMM_GX);
+  if (!gx_aside) {
+    rc = gemm_gx(st);
+    if (rc) return rc;
+    mark(K_GEMM_GX);
+  }
   return HOT_OK;
 }
 

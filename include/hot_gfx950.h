@@ -155,10 +155,12 @@ HOT_API int hot_abc_forward(const void* x, int dtype, int64_t L, int64_t I, cons
  *               {transform+quantise of g_y (both operands), transform+quantise
  *               of W, g_x GEMM+dequant, g_W GEMM+dequant}; non-NULL makes the
  *               call synchronise the stream
- * Without timing, the two W kernels run on a side stream of the library (one per
- * device, created on first use, default priority) between an event recorded on
- * `hip_stream` and a wait on it, so they overlap the g_y kernels; everything is
- * ordered after earlier work on `hip_stream` and before later work on it.
+ * Without timing, independent kernels of the call (the two W kernels, the row-wise
+ * quantise pass of g_y and, for products too small to fill the chip, the g_x GEMM) run
+ * on a side stream of the library (one per device, created on first use, default
+ * priority) between events recorded on `hip_stream` and a wait on it, so they overlap
+ * the token-wise g_y kernels and the g_W GEMM; everything is ordered after earlier
+ * work on `hip_stream` and before later work on it.
  */
 HOT_API size_t hot_backward_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_config* cfg);
 HOT_API int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq,

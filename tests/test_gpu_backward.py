@@ -343,3 +343,32 @@ def test_backward_errors(gpu):
         ops.linear_backward(gy.to(gpu), w.to(gpu), xq, sx, bad)
     with pytest.raises(HotError):
         ops.abc_forward(x.to(gpu)[:100].contiguous(), opt)                               # L % n
+
+
+def test_backward_in_hip_graph(gpu):
+    """The whole call (main stream + the library's side stream, joined by events) is capturable;
+    every replay, with eager work in between, equals the eager result."""
+    from hot_amd import ops
+    L, O, I = 1344, 384, 192
+    x, w, gy = make_case(L, O, I, seed=11, dtype=torch.bfloat16)
+    _, opt = both_configs(L)
+    x, w, gy = x.to(gpu), w.to(gpu), gy.to(gpu)
+    xq, sx = ops.abc_forward(x, opt)
+    ws = torch.empty(1 << 26, dtype=torch.uint8, device=gpu)
+    eager = ops.linear_backward(gy, w, xq, sx, opt, workspace=ws)
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):                       # warm-up on a side stream, as capture requires
+        ops.linear_backward(gy, w, xq, sx, opt, workspace=ws)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = ops.linear_backward(gy, w, xq, sx, opt, workspace=ws)
+    for _ in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out[0], eager[0]) and torch.equal(out[1], eager[1])
+        again = ops.linear_backward(gy, w, xq, sx, opt, workspace=ws)      # eager work between replays
+        torch.cuda.synchronize()
+        assert torch.equal(again[0], eager[0]) and torch.equal(again[1], eager[1])
