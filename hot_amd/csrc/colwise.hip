@@ -103,7 +103,9 @@ __device__ __forceinline__ void fwht_regs(float (&v)[LEN]) {
 // sizeof(T)) rows; wave w issues KiB chunks w, w + 4, ...  Rows past the end
 // of the input and channels past C are redirected to valid addresses: what
 // they deliver is never consumed.
-constexpr int CW_DEPTH = 4;    // LDS buffers in the ring: three steps in flight behind the one in use
+// LDS buffers in the ring (steps in flight behind the one in use = depth - 1): four for 16-bit
+// inputs; 32-bit rows are twice as large, and three buffers keep a second workgroup on the CU.
+template <typename T> constexpr int ring_depth() { return sizeof(T) == 4 ? 3 : 4; }
 
 template <typename T>
 struct RowStream {
@@ -169,6 +171,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   extern __shared__ __align__(16) uint8_t lds[];
   __shared__ float s_max[CW / 64];
   __shared__ double s_sum[2][CW / 64];
+  constexpr int CW_DEPTH = ring_depth<T>();
   uint8_t* const stage = lds + CW_DEPTH * BUF;               // PASS 1: codes [channel][k]
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -461,7 +464,7 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   while ((tb * a.r) % (a.store4 ? 8 : 4) != 0 || tb * out_bytes_per_block < 32) tb <<= 1;
   while (tb * out_bytes_per_block < 128 && gx0 * ((a.NB + 2 * tb - 1) / (2 * tb)) >= 1024) tb <<= 1;
   a.tb = tb;
-  const size_t in_bytes = (size_t)CW_DEPTH * CW_ROWS * CW * sizeof(T);
+  const size_t in_bytes = (size_t)ring_depth<T>() * CW_ROWS * CW * sizeof(T);
   const size_t lds_stats = in_bytes, lds_quant = in_bytes + (size_t)CW * (tb * a.r + 4);
   if (lds_quant > 150 * 1024) return fail(HOT_ERR_UNSUPPORTED, "colwise: staging does not fit LDS");
   const int64_t gx = (a.C + CW - 1) / CW, gy = (a.NB + tb - 1) / tb;
