@@ -49,6 +49,7 @@ struct GemmArgs {
   int32_t tiles_m, tiles_n;
   int32_t group_m;   // tile rows per group of the launch order (tile_of)
   int32_t vec_out;   // out and ldo allow aligned four-element stores
+  int32_t vec16;     // out and its row pitch are 16-byte aligned (staged epilogue)
   int32_t splits;    // K is cut into this many ranges, one workgroup each (1 = no split)
   v4i* partials;     // [tile][range][wave][fragment quad][lane]: raw accumulators of the ranges
 };
@@ -261,6 +262,50 @@ gemm_i8_kernel(const GemmArgs g) {
   gemm_epilogue<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb);
 }
 
+// Epilogue through LDS for tiles that lie fully inside the output: a wave turns one row of its
+// fragments (32 output rows x WN * 32 columns) into output values, parks them row-major in a
+// wave-private LDS area and writes them back out 16 bytes per lane along the rows, so every store
+// instruction covers whole 128-byte lines (the direct epilogue hands the memory system 16-byte
+// pieces of 32 different rows per instruction).  Wave-private: the only synchronisation is the
+// wave's own LDS counter.  `area` must hold 32 * (WN * 32 * sizeof(OutT) + 16) bytes.
+template <int WM, int WN, int BITS, typename OutT>
+__device__ __forceinline__ void gemm_epilogue_staged(const v16i (&acc)[WM][WN], const GemmArgs& g, int64_t row_base,
+                                                     int64_t col_base, int lane, const float (&sa_row)[WM], float sb,
+                                                     uint8_t* area) {
+  constexpr int ROWB = WN * 32 * (int)sizeof(OutT);     // bytes of one staged row
+  constexpr int PITCH = ROWB + 16;
+  constexpr int CPR = ROWB / 16;                        // 16-byte chunks per row
+  constexpr int RPI = 64 / CPR;                         // rows one wave-wide store covers
+  typedef typename Quad<OutT>::type quad_t;
+  OutT* out = reinterpret_cast<OutT*>(g.out);
+  const int m = lane & 31, half = lane >> 5;
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const float sa = sa_row[i];
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        quad_t v;
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          int a = acc[i][j][4 * q + t];
+          if constexpr (BITS == 4) a >>= 8;
+          quad_set<OutT>(v, t, (((float)a * sa) * sb) * g.post_scale);
+        }
+        *reinterpret_cast<quad_t*>(area + m * PITCH + (j * 32 + 8 * q + 4 * half) * (int)sizeof(OutT)) = v;
+      }
+    __builtin_amdgcn_s_waitcnt(0xC07F);                 // lgkmcnt(0): the wave's LDS writes are done
+#pragma unroll
+    for (int r0 = 0; r0 < 32; r0 += RPI) {
+      const int r = r0 + lane / CPR, c = lane % CPR;
+      const v4i chunk = *reinterpret_cast<const v4i*>(area + r * PITCH + c * 16);
+      *reinterpret_cast<v4i*>(reinterpret_cast<uint8_t*>(out + (row_base + i * 32 + r) * g.ldo + col_base) + c * 16) = chunk;
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F);                 // reads done before the next fragment row overwrites
+  }
+}
+
 // ---------------------------------------------------------------------------
 // Pipelined variant: operand tiles travel HBM -> LDS without passing through
 // registers (global_load_lds_dwordx4), four LDS stages deep, so that two
@@ -341,9 +386,15 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
   int tm, tn;
   tile_of(g, tile_id, tm, tn);
   const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
+  // The steps of this lane's rows: loaded here, behind the K loop's latency, when registers allow;
+  // the 256 x 256 tile has none to spare and loads them in the epilogue.
+  constexpr bool EARLY_SCALES = WM * WN <= 4;
   float sa_row[WM];
-  load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
-  const float sb = g.scale_b[0];
+  float sb = 0.f;
+  if constexpr (EARLY_SCALES) {
+    load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
+    sb = g.scale_b[0];
+  }
 
   // DMA instruction i of this wave fills KiB chunk 4 i + wave of the stage (A rows first, then B
   // rows; BM / 16 is a multiple of 4, so instruction i serves A for i < BM / 64 and B otherwise).
@@ -495,7 +546,7 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
   for (; kt0 + 2 * S - 2 < KT; kt0 += S) rotation(std::true_type{}, kt0);   // every issue inside is in range
   for (; kt0 < KT; kt0 += S) rotation(std::false_type{}, kt0);
 
-  if (g.splits > 1) {
+  if (WM * WN <= 4 && g.splits > 1) {     // only the 128 x 128 kernel is ever launched split
     // Split K: every range leaves its raw accumulators in the workspace (lane-major, so each store
     // is one contiguous KiB per wave); gemm_i8_reduce_kernel adds them up and runs the epilogue.
     constexpr int QUADS = WM * WN * 4;
@@ -512,6 +563,17 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
     return;
   }
 
+  if constexpr (!EARLY_SCALES) {
+    load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
+    sb = g.scale_b[0];
+  }
+  constexpr int AREA = 32 * (WN * 32 * (int)sizeof(OutT) + 16);
+  if (4 * AREA <= S * STAGE_BYTES && g.vec16 && !g.acc_out && row0 + BM <= g.M && col0 + BN <= g.N) {
+    __syncthreads();                                     // every wave is done with the ring
+    gemm_epilogue_staged<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb,
+                                             ring + wave * AREA);
+    return;
+  }
   gemm_epilogue<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb);
 }
 
@@ -678,6 +740,7 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
   g.scale_a = scale_a; g.scale_b = scale_b; g.post_scale = post_scale; g.a_per_row = a_per_row;
   g.out = out; g.ldo = ldo; g.acc_out = acc_out;
   g.vec_out = ((ldo & 3) == 0 && ((uintptr_t)out & 15) == 0) ? 1 : 0;
+  g.vec16 = (((uintptr_t)out & 15) == 0 && ((ldo * (out_dtype == HOT_F32 ? 4 : 2)) & 15) == 0) ? 1 : 0;
   g.splits = 1; g.partials = nullptr;
   const GemmSplit plan = gemm_split_plan(M, N, K, bits);
   if (plan.splits > 1 && split_ws && split_ws_bytes >= plan.ws_bytes && M * lda < (1ll << 32) && N * ldb < (1ll << 32) &&

@@ -98,12 +98,8 @@ template <> __device__ __forceinline__ float load_scalar<float>(const float* p) 
 template <> __device__ __forceinline__ float load_scalar<bf16_t>(const bf16_t* p) { return as_f((uint32_t)p->v << 16); }
 template <> __device__ __forceinline__ float load_scalar<f16_t>(const f16_t* p) { return (float)p->v; }
 
-__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) {
-  uint32_t u = as_u(f);
-  if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x40);  // NaN
-  u += 0x7FFFu + ((u >> 16) & 1u);
-  return (uint16_t)(u >> 16);
-}
+// round-to-nearest-even; gfx950 converts in hardware (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint16_t f32_to_bf16_rne(float f) { return __builtin_bit_cast(uint16_t, (__bf16)f); }
 
 template <typename T> __device__ __forceinline__ void store_scalar(T* p, float v);
 template <> __device__ __forceinline__ void store_scalar<float>(float* p, float v) { *p = v; }
