@@ -109,15 +109,17 @@ template <typename T> constexpr int ring_depth() { return sizeof(T) == 4 ? 3 : 4
 
 template <typename T>
 struct RowStream {
-  static constexpr int RB = CW * (int)sizeof(T);                 // bytes per staged row
-  static constexpr int BUF_BYTES = CW_ROWS * RB;
-  static constexpr int LPW = BUF_BYTES / 1024 / (CW / 64);       // DMA instructions per wave per step
+  static constexpr int RB = 64 * (int)sizeof(T);                 // bytes per staged row of ONE wave (64 channels)
+  static constexpr int WAVE_BYTES = CW_ROWS * RB;                // one wave's share of a step
+  static constexpr int BUF_BYTES = (CW / 64) * WAVE_BYTES;       // all waves' shares of a step
+  static constexpr int LPW = WAVE_BYTES / 1024;                  // DMA instructions per wave per step
   static constexpr int VPR = RB / 16;                            // 16-byte vectors per staged row
-  const uint8_t* base;   // &in[0][cg0]
+  static constexpr int RPC = 1024 / RB;                          // rows per KiB chunk (one DMA instruction)
+  const uint8_t* base;   // &in[0][first channel of this wave] (or of the workgroup when the wave has none)
   uint32_t pitch;        // bytes per input row
   int64_t rows_total;
   int64_t row0;
-  int nvec_row;          // valid 16-byte vectors per row for this channel group
+  int nvec_row;          // valid 16-byte vectors per row for this wave (at least 1)
 };
 
 // s_waitcnt vmcnt(VM) lgkmcnt(0); vmcnt is split over bits 3:0 and 15:14
@@ -133,27 +135,28 @@ __device__ __forceinline__ void dma16_to_lds(uint32_t lds_addr, uint32_t voff, c
                : "memory", "m0");
 }
 
+// Every wave streams the rows of its own 64 channels into its own slice of each ring buffer
+// ([16 rows][64 channels]), so a wave waits for nothing but its own loads: no workgroup barrier
+// in the streaming loop, and the four waves of a workgroup drift apart freely.
 template <typename T>
-__device__ __forceinline__ void rs_issue(const RowStream<T>& rs, uint32_t buf_lds, int step, int wave, int lane) {
-  constexpr int VPR = RowStream<T>::VPR;
-  constexpr int RPC = 1024 / RowStream<T>::RB > 0 ? 1024 / RowStream<T>::RB : 1;   // rows per KiB chunk
+__device__ __forceinline__ void rs_issue(const RowStream<T>& rs, uint32_t wave_lds, int step, int lane) {
+  constexpr int VPR = RowStream<T>::VPR, RPC = RowStream<T>::RPC;
 #pragma unroll
   for (int i = 0; i < RowStream<T>::LPW; ++i) {
-    const int chunk = wave + (CW / 64) * i;
-    int64_t row = rs.row0 + (int64_t)step * CW_ROWS + chunk * RPC + lane / VPR;
+    int64_t row = rs.row0 + (int64_t)step * CW_ROWS + i * RPC + lane / VPR;
     if (row >= rs.rows_total) row = rs.rows_total - 1;
     int vec = lane % VPR;
     if (vec >= rs.nvec_row) vec = rs.nvec_row - 1;
-    dma16_to_lds(buf_lds + chunk * 1024, (uint32_t)row * rs.pitch + (uint32_t)vec * 16, rs.base);
+    dma16_to_lds(wave_lds + i * 1024, (uint32_t)row * rs.pitch + (uint32_t)vec * 16, rs.base);
   }
 }
 
 template <typename T>
-__device__ __forceinline__ void rs_column(const uint8_t* buf, int tid, float* v) {
+__device__ __forceinline__ void rs_column(const uint8_t* wave_buf, int lane, float* v) {
   typedef typename raw_of<T>::type raw_t;
-  const raw_t* p = reinterpret_cast<const raw_t*>(buf) + tid;
+  const raw_t* p = reinterpret_cast<const raw_t*>(wave_buf) + lane;
 #pragma unroll
-  for (int i = 0; i < CW_ROWS; ++i) v[i] = cvt_raw<T>(p[i * CW]);
+  for (int i = 0; i < CW_ROWS; ++i) v[i] = cvt_raw<T>(p[i * 64]);
 }
 
 // ---- the kernel: PASS 0 = statistics, PASS 1 = quantise + transposed store ----
@@ -187,12 +190,17 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   const int pitch = sb + 4;
 
   RowStream<T> rs;
-  rs.base = reinterpret_cast<const uint8_t*>(a.in) + cg0 * (int64_t)sizeof(T);
   rs.pitch = (uint32_t)(a.C * (int64_t)sizeof(T));
   rs.rows_total = a.R;
   rs.row0 = blk0 * N;
   {
-    const int64_t chans = (a.C - cg0) < CW ? (a.C - cg0) : CW;
+    // channels of this wave that exist; a wave past the end streams the workgroup's first
+    // channels instead (valid addresses, never consumed)
+    int64_t cw0 = cg0 + 64 * wave;
+    int64_t chans = a.C - cw0;
+    if (chans <= 0) { cw0 = cg0; chans = a.C - cg0; }
+    if (chans > 64) chans = 64;
+    rs.base = reinterpret_cast<const uint8_t*>(a.in) + cw0 * (int64_t)sizeof(T);
     rs.nvec_row = (int)(chans * (int64_t)sizeof(T) / 16);
   }
 
@@ -267,21 +275,21 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   };
 
   // ring of CW_DEPTH LDS buffers: steps s+1 .. s+CW_DEPTH-1 are in flight while step s is consumed
-  constexpr int LPW = RowStream<T>::LPW;
-  const uint32_t lds0 = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t*)lds;
+  constexpr int LPW = RowStream<T>::LPW, WB = RowStream<T>::WAVE_BYTES;
+  const uint32_t lds0 = (uint32_t)(uintptr_t)(const __attribute__((address_space(3))) uint8_t*)lds + wave * WB;
+  const uint8_t* const my = lds + wave * WB;               // this wave's slice of ring buffer 0
 #pragma unroll
   for (int s = 0; s < CW_DEPTH - 1; ++s)
-    if (s < nsteps) rs_issue<T>(rs, lds0 + s * BUF, s, wave, lane);
+    if (s < nsteps) rs_issue<T>(rs, lds0 + s * BUF, s, lane);
   // one step: wait for its rows, let the ring advance, pull this thread's 16 values into x[xo..]
   auto step = [&](int s, float* dst) {
-    // this wave's share of step s has landed, and its own LDS reads of step s-1 are complete ...
-    // steps s+1 .. s+CW_DEPTH-2 may still be in flight
+    // this wave's rows of step s have landed, and its LDS reads of step s-1 are complete: the
+    // slice that held step s-1 may be refilled.  Steps s+1 .. s+CW_DEPTH-2 may still be in flight.
     if (CW_DEPTH >= 4 && s + 2 < nsteps) wait_stream<2 * LPW>();
     else if (CW_DEPTH >= 3 && s + 1 < nsteps) wait_stream<LPW>();
     else wait_stream<0>();
-    __builtin_amdgcn_s_barrier();   // ... and so for every wave: the buffer of step s-1 may be refilled
-    if (s + CW_DEPTH - 1 < nsteps) rs_issue<T>(rs, lds0 + ((s + CW_DEPTH - 1) % CW_DEPTH) * BUF, s + CW_DEPTH - 1, wave, lane);
-    rs_column<T>(lds + (s % CW_DEPTH) * BUF, tid, dst);
+    if (s + CW_DEPTH - 1 < nsteps) rs_issue<T>(rs, lds0 + ((s + CW_DEPTH - 1) % CW_DEPTH) * BUF, s + CW_DEPTH - 1, lane);
+    rs_column<T>(my + (s % CW_DEPTH) * BUF, lane, dst);
     if constexpr (PASS == 0 && RS != 0) {
 #pragma unroll
       for (int i = 0; i < CW_ROWS; ++i) {
