@@ -98,10 +98,10 @@ __device__ __forceinline__ void fwht_regs(float (&v)[LEN]) {
 
 // Streams the rows of the workgroup's tile through a ring of LDS buffers with
 // direct global -> LDS loads (16 bytes per lane, no registers in between).
-// Step s covers rows [row0 + 16 s, +16); a buffer holds them as [16][256] raw
-// elements.  A wave-wide load fills one contiguous KiB, i.e. 1024 / (256
-// sizeof(T)) rows; wave w issues KiB chunks w, w + 4, ...  Rows past the end
-// of the input and channels past C are redirected to valid addresses: what
+// Step s covers rows [row0 + 16 s, +16); a buffer holds them as one
+// [16 rows][64 channels] slice per wave.  A wave-wide load fills one contiguous
+// KiB of the wave's own slice, i.e. 1024 / (64 sizeof(T)) rows.  Rows past the
+// end of the input and channels past C are redirected to valid addresses: what
 // they deliver is never consumed.
 // LDS buffers in the ring (steps in flight behind the one in use = depth - 1): four for 16-bit
 // inputs; 32-bit rows are twice as large, and three buffers keep a second workgroup on the CU.
