@@ -274,3 +274,51 @@ def test_gemm_i8_bf16_out(gpu):
                       out_dtype=torch.bfloat16)
     ref = torch.from_numpy(orc.int_gemm_nt(a, b).astype(np.float32)).to(torch.bfloat16)
     assert torch.equal(out.cpu(), ref)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("bits,M,N,K,per_row", [
+    (8, 256, 384, 512, False),      # whole tiles: the LDS-staged epilogue
+    (4, 384, 256, 1024, True),
+    (8, 515, 260, 300, True),       # ragged tiles; 260 columns: four-wide stores, rows not 16-byte aligned in bf16
+    (4, 200, 130, 256, False),      # 130 columns: scalar stores
+])
+def test_gemm_i8_epilogues(gpu, out_dtype, bits, M, N, K, per_row):
+    """Every store path of the epilogue, without the int32 side output (which forces the direct one)."""
+    from hot_amd import ops
+    a, b = rand_codes(M, K, bits, 11), rand_codes(N, K, bits, 12)
+    kp = ops.kpad(K)
+    rng = np.random.default_rng(13)
+    sa = rng.uniform(1e-4, 2e-4, size=(M if per_row else 1)).astype(np.float32)
+    sb = rng.uniform(1e-3, 2e-3, size=1).astype(np.float32)
+    out = ops.gemm_i8(to_operand(a, bits, kp).to(gpu), to_operand(b, bits, kp).to(gpu), K, bits,
+                      torch.from_numpy(sa).to(gpu), torch.from_numpy(sb).to(gpu), post_scale=1 / 64, out_dtype=out_dtype)
+    acc = orc.int_gemm_nt(a, b)
+    ref = ((acc.astype(np.float32) * sa.reshape(-1, 1)).astype(np.float32) * sb[0]).astype(np.float32) / np.float32(64)
+    assert torch.equal(out.cpu(), torch.from_numpy(ref.astype(np.float32)).to(out_dtype))
+
+
+@pytest.mark.parametrize("bits", [4, 8])
+def test_gemm_i8_large_tiles(gpu, bits):
+    """Enough 256 x 256 tiles for the large-tile kernel (20 x 26 of them, ragged on both edges)."""
+    from hot_amd import ops
+    M, N, K = 5000, 6600, 192
+    a, b = rand_codes(M, K, bits, 21), rand_codes(N, K, bits, 22)
+    kp = ops.kpad(K)
+    one = torch.ones(1, device=gpu)
+    out = ops.gemm_i8(to_operand(a, bits, kp).to(gpu), to_operand(b, bits, kp).to(gpu), K, bits, one, one,
+                      out_dtype=torch.float32)
+    ref = (a.astype(np.float64) @ b.astype(np.float64).T).astype(np.float32)      # exact: |acc| < 2^24
+    assert np.array_equal(out.cpu().numpy(), ref)
+
+
+def test_gemm_splits_rule():
+    """hot_gemm_splits: products with few output tiles and a long K are cut, others are not."""
+    from hot_amd import _lib
+    f = _lib.lib().hot_gemm_splits
+    assert f(3072, 768, 7092, 8) == 3          # ViT-B fc1 g_W: 144 tiles
+    assert f(12608, 768, 3072, 4) == 1         # ViT-B fc1 g_x: 594 tiles
+    assert f(11008, 4096, 4096, 8) == 1
+    assert f(256, 256, 128, 8) == 1            # short K
+    assert f(256, 256, 2304, 8) == 2
+
