@@ -21,9 +21,10 @@ template <> struct dtype_of<f16_t> { static constexpr int value = 2; };
 __device__ __forceinline__ float as_f(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t as_u(float f) { return __builtin_bit_cast(uint32_t, f); }
 
-// Value held by lane (lane ^ MASK).  1 and 2 are DPP quad permutes (folded by
-// the compiler into the consuming VALU op), 4..16 go through the LDS crossbar
-// without touching memory, 32 uses the wave-wide permute.
+// Value held by lane (lane ^ MASK).  1, 2, 3 and 8 are single DPP controls (folded by the compiler
+// into the consuming VALU op: quad permutes, and a rotation by 8 inside the row of 16 lanes); 4 is
+// two of them (xor 3, then the mirror of each half row, which is xor 7); 16 goes through the LDS
+// crossbar without touching memory, 32 uses the wave-wide permute.
 template <int MASK>
 __device__ __forceinline__ float lane_xor(float v) {
   int i = __builtin_bit_cast(int, v);
@@ -33,6 +34,11 @@ __device__ __forceinline__ float lane_xor(float v) {
     i = __builtin_amdgcn_update_dpp(0, i, 0x4E, 0xF, 0xF, true);  // quad_perm [2,3,0,1]
   } else if constexpr (MASK == 3) {
     i = __builtin_amdgcn_update_dpp(0, i, 0x1B, 0xF, 0xF, true);  // quad_perm [3,2,1,0]
+  } else if constexpr (MASK == 4) {
+    i = __builtin_amdgcn_update_dpp(0, i, 0x1B, 0xF, 0xF, true);  // quad_perm [3,2,1,0]: xor 3
+    i = __builtin_amdgcn_update_dpp(0, i, 0x141, 0xF, 0xF, true); // row_half_mirror: xor 7
+  } else if constexpr (MASK == 8) {
+    i = __builtin_amdgcn_update_dpp(0, i, 0x128, 0xF, 0xF, true); // row_ror:8
   } else if constexpr (MASK < 32) {
     i = __builtin_amdgcn_ds_swizzle(i, (MASK << 10) | 0x1F);      // bitmask mode: xor MASK
   } else {
