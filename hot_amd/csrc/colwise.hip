@@ -262,7 +262,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
                   sr_uniform4(quad, a.seed, a.stream, u);
                 }
                 const int w = visited & 3;
-                q = q_stoch(v / d, w == 0 ? u[0] : w == 1 ? u[1] : w == 2 ? u[2] : u[3]);
+                q = q_stoch_div(v, d, rcp, w == 0 ? u[0] : w == 1 ? u[1] : w == 2 ? u[2] : u[3]);
                 ++visited;
                 q = clampi(q, -qmax, qmax);   // floor + 1 may step past qmax at the very top
               }

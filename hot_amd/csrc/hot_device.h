@@ -120,8 +120,10 @@ __device__ __forceinline__ philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint3
                                                  uint32_t k0, uint32_t k1) {
 #pragma unroll
   for (int r = 0; r < 10; ++r) {
-    const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
-    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    // one 32 x 32 -> 64 multiply per product (v_mad_u64_u32) instead of a high and a low multiply
+    const uint64_t p0 = (uint64_t)0xD2511F53u * (uint64_t)c0, p1 = (uint64_t)0xCD9E8D57u * (uint64_t)c2;
+    const uint32_t hi0 = (uint32_t)(p0 >> 32), lo0 = (uint32_t)p0;
+    const uint32_t hi1 = (uint32_t)(p1 >> 32), lo1 = (uint32_t)p1;
     const uint32_t n0 = hi1 ^ c1 ^ k0, n2 = hi0 ^ c3 ^ k1;
     c0 = n0; c1 = lo1; c2 = n2; c3 = lo0;
     k0 += 0x9E3779B9u; k1 += 0xBB67AE85u;
@@ -157,6 +159,18 @@ __device__ __forceinline__ int q_stoch(float y, float u) {
   const float frac = ay - fl;
   const int m = (int)fl + (u < frac ? 1 : 0);
   return y < 0.f ? -m : m;
+}
+
+// q_stoch(x / d, u) with rcp = 1 / d precomputed.  p = x * rcp is within 2^-15 of the IEEE quotient
+// (|x / d| <= 128), so floor and the comparison with u come out the same unless the fractional part
+// lies within 2^-14 of 0, of 1 or of u; only then is the division carried out.
+__device__ __forceinline__ int q_stoch_div(float x, float d, float rcp, float u) {
+  const float eps = 6.103515625e-05f;
+  const float p = x * rcp;
+  const float ap = fabsf(p), fl = floorf(ap), frac = ap - fl;
+  if (__builtin_expect(fabsf(frac - u) < eps || frac < eps || frac > 1.0f - eps, 0)) return q_stoch(x / d, u);
+  const int m = (int)fl + (u < frac ? 1 : 0);
+  return p < 0.f ? -m : m;
 }
 
 __device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }

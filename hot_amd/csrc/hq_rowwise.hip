@@ -81,7 +81,7 @@ __device__ __forceinline__ void quant_store_chunk(const float* x, float d, float
     sr_uniform4(e0 >> 2, seed, stream, u);
     sr_uniform4((e0 >> 2) + 1, seed, stream, u + 4);
 #pragma unroll
-    for (int j = 0; j < EPL; ++j) q[j] = clampi(q_stoch(x[j] / d, u[j]), -QMAX, QMAX);
+    for (int j = 0; j < EPL; ++j) q[j] = clampi(q_stoch_div(x[j], d, rcp, u[j]), -QMAX, QMAX);
   }
   if constexpr (BITS == 4) {
     uint32_t w = 0;
