@@ -34,7 +34,7 @@ int check_launch(const char* what) { return check_hip(hipGetLastError(), what); 
 
 static int check_cfg(const hot_config* c, const char* who) {
   if (!c) return fail(HOT_ERR_INVALID, "%s: null config", who);
-  if (c->n_o != 16 && c->n_o != 32 && c->n_o != 64) return fail(HOT_ERR_UNSUPPORTED, "%s: n_o=%d (16, 32 or 64)", who, c->n_o);
+  if (c->n_o < 1 || c->n_o > 64 || (c->n_o & (c->n_o - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: n_o=%d (a power of two up to 64)", who, c->n_o);
   if (c->hla_n < 1 || c->hla_n > HOT_MAX_HLA_N || (c->hla_n & (c->hla_n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: hla_n=%d (power of two up to %d)", who, c->hla_n, HOT_MAX_HLA_N);
   if (c->hla_r < 1 || c->hla_r > c->hla_n) return fail(HOT_ERR_INVALID, "%s: hla_r=%d outside [1, %d]", who, c->hla_r, c->hla_n);
   const int bits[4] = {c->gx_bits, c->w_bits, c->gw_bits, c->act_bits};

@@ -467,10 +467,10 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   // of output dwords and cover the blocks that share a 16-row step; beyond that, longer runs (up
   // to 128 bytes) are taken only while they leave at least four workgroups per CU.
   const int64_t gx0 = (a.C + CW - 1) / CW;
-  const int out_bytes_per_block = a.store4 ? a.r / 2 : a.r;   // r is even when store4
+  auto run_bytes = [&](int t) { return a.store4 ? t * a.r / 2 : t * a.r; };   // t * r is a multiple of 8 when store4
   int tb = BPS;
-  while ((tb * a.r) % (a.store4 ? 8 : 4) != 0 || tb * out_bytes_per_block < 32) tb <<= 1;
-  while (tb * out_bytes_per_block < 128 && gx0 * ((a.NB + 2 * tb - 1) / (2 * tb)) >= 1024) tb <<= 1;
+  while ((tb * a.r) % (a.store4 ? 8 : 4) != 0 || run_bytes(tb) < 32) tb <<= 1;
+  while (run_bytes(tb) < 128 && gx0 * ((a.NB + 2 * tb - 1) / (2 * tb)) >= 1024) tb <<= 1;
   a.tb = tb;
   const size_t in_bytes = (size_t)ring_depth<T>() * CW_ROWS * CW * sizeof(T);
   const size_t lds_stats = in_bytes, lds_quant = in_bytes + (size_t)CW * (tb * a.r + 4);

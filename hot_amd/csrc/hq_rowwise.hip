@@ -35,11 +35,13 @@ __device__ __forceinline__ void load_chunk(const T* p, float* x) {
   }
 }
 
-// FWHT of the N-element blocks formed by N/EPL adjacent lanes.
+// FWHT of the N-element blocks formed by N/EPL adjacent lanes.  N = 8 stands for every block that
+// fits one lane's chunk: its actual size `nrt` (1, 2, 4 or 8) arrives at run time.
 template <int N>
-__device__ __forceinline__ void fwht_lanes(float* x, int lane) {
+__device__ __forceinline__ void fwht_lanes(float* x, int lane, int nrt) {
 #pragma unroll
   for (int h = 1; h < EPL; h <<= 1) {
+    if (N <= EPL && h >= nrt) break;
 #pragma unroll
     for (int j = 0; j < EPL; ++j) {
       if ((j & h) == 0) {
@@ -103,7 +105,7 @@ __device__ __forceinline__ void quant_store_chunk(const float* x, float d, float
 
 template <typename T, int N, int BITS, int ROUND, int C>
 __global__ void hq_row_kernel(const T* __restrict__ in, int64_t K, int8_t* __restrict__ codes, int64_t ld,
-                              float* __restrict__ scales, uint64_t seed, uint32_t stream) {
+                              float* __restrict__ scales, uint64_t seed, uint32_t stream, int nrt) {
   __shared__ float s_red[16];
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -126,7 +128,7 @@ __global__ void hq_row_kernel(const T* __restrict__ in, int64_t K, int8_t* __res
   float mx = 0.f;
 #pragma unroll
   for (int c = 0; c < C; ++c) {
-    fwht_lanes<N>(x[c], lane);
+    fwht_lanes<N>(x[c], lane, nrt);
 #pragma unroll
     for (int j = 0; j < EPL; ++j) mx = fmaxf(mx, fabsf(x[c][j]));
   }
@@ -159,7 +161,7 @@ __global__ void hq_row_kernel(const T* __restrict__ in, int64_t K, int8_t* __res
 // ---- per-tensor scale, pass 1: absmax of the transformed tensor -----------
 
 template <typename T, int N>
-__global__ void hq_absmax_kernel(const T* __restrict__ in, int64_t nchunks, float* __restrict__ absmax) {
+__global__ void hq_absmax_kernel(const T* __restrict__ in, int64_t nchunks, float* __restrict__ absmax, int nrt) {
   __shared__ float s_red[16];
   const int lane = threadIdx.x & 63;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
@@ -167,7 +169,7 @@ __global__ void hq_absmax_kernel(const T* __restrict__ in, int64_t nchunks, floa
   for (int64_t ch = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ch < nchunks; ch += stride) {
     float x[EPL];
     load_chunk<T>(in + ch * EPL, x);
-    fwht_lanes<N>(x, lane);
+    fwht_lanes<N>(x, lane, nrt);
 #pragma unroll
     for (int j = 0; j < EPL; ++j) mx = fmaxf(mx, fabsf(x[j]));
   }
@@ -186,7 +188,7 @@ __global__ void hq_absmax_kernel(const T* __restrict__ in, int64_t nchunks, floa
 template <typename T, int N, int BITS, int ROUND>
 __global__ void hq_tensor_kernel(const T* __restrict__ in, int64_t nchunks, int64_t nch_row, int64_t ld,
                                  const float* __restrict__ absmax, int8_t* __restrict__ codes,
-                                 float* __restrict__ scale_out, uint64_t seed, uint32_t stream) {
+                                 float* __restrict__ scale_out, uint64_t seed, uint32_t stream, int nrt) {
   const int lane = threadIdx.x & 63;
   constexpr float QMAXF = (float)((1 << (BITS - 1)) - 1);
   const float s = *absmax / QMAXF;
@@ -197,7 +199,7 @@ __global__ void hq_tensor_kernel(const T* __restrict__ in, int64_t nchunks, int6
   for (int64_t ch = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ch < nchunks; ch += stride) {
     float x[EPL];
     load_chunk<T>(in + ch * EPL, x);
-    fwht_lanes<N>(x, lane);
+    fwht_lanes<N>(x, lane, nrt);
     int64_t off = ch * (EPL * BITS / 8);
     if (ld != nch_row * (EPL * BITS / 8)) {  // padded rows
       const int64_t row = ch / nch_row;
@@ -225,7 +227,7 @@ __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
 
 template <typename T, int N, int BITS, int ROUND>
 static int launch_row(const void* in, int64_t M, int64_t K, void* codes, int64_t ld, float* scales, uint64_t seed,
-                      uint32_t stream_id, hipStream_t st) {
+                      uint32_t stream_id, hipStream_t st, int nrt) {
   const int64_t nch = K / EPL;
   int team = 64;
   while (team < 1024 && nch > 4 * (int64_t)team) team <<= 1;
@@ -234,7 +236,7 @@ static int launch_row(const void* in, int64_t M, int64_t K, void* codes, int64_t
   const dim3 grid((unsigned)M), block(team);
 #define HOT_ROW_CASE(CC)                                                                              \
   hipLaunchKernelGGL((hq_row_kernel<T, N, BITS, ROUND, CC>), grid, block, 0, st, (const T*)in, K, \
-                     (int8_t*)codes, ld, scales, seed, stream_id)
+                     (int8_t*)codes, ld, scales, seed, stream_id, nrt)
   switch (c) {
     case 1: HOT_ROW_CASE(1); break;
     case 2: HOT_ROW_CASE(2); break;
@@ -249,7 +251,7 @@ static int launch_row(const void* in, int64_t M, int64_t K, void* codes, int64_t
 
 template <typename T, int N, int BITS, int ROUND>
 static int launch_tensor(const void* in, int64_t M, int64_t K, void* codes, int64_t ld, float* scales, float* absmax,
-                         uint64_t seed, uint32_t stream_id, hipStream_t st, bool absmax_ready) {
+                         uint64_t seed, uint32_t stream_id, hipStream_t st, bool absmax_ready, int nrt) {
   const int64_t nch = M * K / EPL;
   const int block = 256;
   int64_t blocks = (nch + block - 1) / block;
@@ -258,37 +260,37 @@ static int launch_tensor(const void* in, int64_t M, int64_t K, void* codes, int6
   if (blocks < 1) blocks = 1;
   if (!absmax_ready) {
     hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, (uint32_t*)absmax, 0u, 1);
-    hipLaunchKernelGGL((hq_absmax_kernel<T, N>), dim3((unsigned)blocks), dim3(block), 0, st, (const T*)in, nch, absmax);
+    hipLaunchKernelGGL((hq_absmax_kernel<T, N>), dim3((unsigned)blocks), dim3(block), 0, st, (const T*)in, nch, absmax, nrt);
   }
   hipLaunchKernelGGL((hq_tensor_kernel<T, N, BITS, ROUND>), dim3((unsigned)blocks), dim3(block), 0, st,
-                     (const T*)in, nch, K / EPL, ld, absmax, (int8_t*)codes, scales, seed, stream_id);
+                     (const T*)in, nch, K / EPL, ld, absmax, (int8_t*)codes, scales, seed, stream_id, nrt);
   return check_launch("hq_tensor_kernel");
 }
 
 template <typename T, int N, int BITS, int ROUND>
 static int dispatch_mode(int scale_mode, const void* in, int64_t M, int64_t K, void* codes, int64_t ld, float* scales,
-                         float* absmax, uint64_t seed, uint32_t stream_id, hipStream_t st, bool absmax_ready) {
+                         float* absmax, uint64_t seed, uint32_t stream_id, hipStream_t st, bool absmax_ready, int nrt) {
   const int64_t row_bytes = K * BITS / 8;
   if (ld > row_bytes) {
     const int64_t n = M * ((ld - row_bytes) / 4);
     hipLaunchKernelGGL(zero_pad_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (int8_t*)codes, M, row_bytes, ld);
   }
-  if (scale_mode == HOT_SCALE_ROW) return launch_row<T, N, BITS, ROUND>(in, M, K, codes, ld, scales, seed, stream_id, st);
-  return launch_tensor<T, N, BITS, ROUND>(in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready);
+  if (scale_mode == HOT_SCALE_ROW) return launch_row<T, N, BITS, ROUND>(in, M, K, codes, ld, scales, seed, stream_id, st, nrt);
+  return launch_tensor<T, N, BITS, ROUND>(in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt);
 }
 
 template <typename T, int N>
 static int dispatch_bits(int bits, int rounding, int scale_mode, const void* in, int64_t M, int64_t K,
                          void* codes, int64_t ld, float* scales, float* absmax, uint64_t seed, uint32_t stream_id,
-                         hipStream_t st, bool absmax_ready) {
+                         hipStream_t st, bool absmax_ready, int nrt) {
   if (bits == 4) {
     return rounding == HOT_ROUND_NEAREST
-               ? dispatch_mode<T, N, 4, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready)
-               : dispatch_mode<T, N, 4, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready);
+               ? dispatch_mode<T, N, 4, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt)
+               : dispatch_mode<T, N, 4, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt);
   }
   return rounding == HOT_ROUND_NEAREST
-             ? dispatch_mode<T, N, 8, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready)
-             : dispatch_mode<T, N, 8, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready);
+             ? dispatch_mode<T, N, 8, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt)
+             : dispatch_mode<T, N, 8, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt);
 }
 
 template <typename T>
@@ -296,9 +298,11 @@ static int dispatch_n(int n, int bits, int rounding, int scale_mode, const void*
                       void* codes, int64_t ld, float* scales, float* absmax, uint64_t seed, uint32_t stream_id,
                       hipStream_t st, bool absmax_ready) {
   switch (n) {
-    case 16: return dispatch_bits<T, 16>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready);
-    case 32: return dispatch_bits<T, 32>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready);
-    default: return dispatch_bits<T, 64>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready);
+    case 1: case 2: case 4: case 8:
+      return dispatch_bits<T, 8>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n);
+    case 16: return dispatch_bits<T, 16>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n);
+    case 32: return dispatch_bits<T, 32>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n);
+    default: return dispatch_bits<T, 64>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n);
   }
 }
 
@@ -307,8 +311,8 @@ int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int 
                     float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st, bool absmax_ready) {
   if (M != 0 && (!in || !codes_out || !scales_out)) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: null pointer");
   if (M < 0 || K <= 0) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: bad shape M=%lld K=%lld", (long long)M, (long long)K);
-  if (n != 16 && n != 32 && n != 64) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: Hadamard block %d (16, 32 or 64)", n);
-  if (K % n) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: K=%lld is not a multiple of the block %d", (long long)K, n);
+  if (n < 1 || n > 64 || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: Hadamard block %d (a power of two up to 64)", n);
+  if (K % n || K % 8) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: K=%lld is not a multiple of the block %d and of 8", (long long)K, n);
   if (bits != 4 && bits != 8) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: bits=%d (4 or 8)", bits);
   if (rounding != HOT_ROUND_NEAREST && rounding != HOT_ROUND_STOCH) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: bad rounding %d", rounding);
   if (scale_mode != HOT_SCALE_TENSOR && scale_mode != HOT_SCALE_ROW) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: scale mode %d (tensor or row)", scale_mode);

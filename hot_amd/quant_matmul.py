@@ -27,7 +27,8 @@ from torch.autograd.function import Function
 
 from . import args
 from . import ops
-from .hadamard_matmul import (Transform_Dict, biggest_power2_factor, hla_rows, paper_rows)
+from .hadamard_matmul import (Transform_Dict, biggest_power2_factor, biggest_power2_factor_max16, hla_rows,
+                              paper_rows)
 
 TD = Transform_Dict()
 
@@ -69,8 +70,10 @@ def hot_switched_off() -> bool:
             and all(getattr(args, k) in off for k in ("quantBWDGogi", "quantBWDWgt", "quantBWDGogw", "quantBWDAct")))
 
 
-def options_for(tokens: int, layer_name: str = " ") -> ops.HotOptions:
-    """args.* -> HotOptions, following the branch structure of FLinearQ."""
+def options_for(tokens: int, layer_name: str = " ", out_features: int = 16) -> ops.HotOptions:
+    """args.* -> HotOptions, following the branch structure of FLinearQ.  The Hadamard block along the
+    out-features is the reference's make_hadamard rule: the largest power of two dividing them, at
+    most 16 (utils/hadamard_matmul.py:57-59): 16 for the usual widths, 4 for a 100-class head."""
     if args.transform_scheme != "gih_gwlr":
         raise NotImplementedError("transform scheme %r: only gih_gwlr runs natively" % args.transform_scheme)
     if not (args.TransformGogi and args.TransformWgt and args.TransformGogw and args.TransformInput):
@@ -88,11 +91,23 @@ def options_for(tokens: int, layer_name: str = " ") -> ops.HotOptions:
     w_round, w_scale = _scheme(args.quantBWDWgt, "Weight", ("int", "stoch", "sawb"))
     act_round, act_scale = _scheme(args.quantBWDAct, "Activation", ("int", "stoch", "sawb"))
     return ops.HotOptions(
-        n_o=16, hla_n=int(n), hla_rows=tuple(int(v) for v in rows),
+        n_o=int(biggest_power2_factor_max16(int(out_features))), hla_n=int(n), hla_rows=tuple(int(v) for v in rows),
         gx_bits=gx_bits, w_bits=args.weightQuantBit, gw_bits=gw_bits, act_bits=args.actQuantBit,
         gx_round=gx_round, w_round=w_round, gw_round=gw_round, act_round=act_round,
         gx_scale=gx_scale, w_scale=w_scale, gw_scale=gw_scale, act_scale=act_scale,
         seed=(int(args.sr_seed) << 20) + int(args.sr_step))
+
+
+def _check_padding(w: Tensor, opt: ops.HotOptions) -> None:
+    if (w.shape[0] % 8 or w.shape[1] % 8) and ops.SCALE_SAWB in (opt.w_scale, opt.act_scale):
+        raise NotImplementedError("SAWB statistics over zero-padded channels would differ from the reference: "
+                                  "feature counts must be multiples of 8 with the sawb quantisers")
+
+
+def _pad8(t: Tensor) -> Tensor:
+    """`t` (2-D) contiguous, its last dimension padded with zeros to a multiple of 8."""
+    extra = (-t.shape[-1]) % 8
+    return F.pad(t, (0, extra)).contiguous() if extra else t.contiguous()
 
 
 class FLinearQ(Function):
@@ -112,16 +127,20 @@ class FLinearQ(Function):
         if ctx.full_precision:
             ctx.save_for_backward(x, w)
             return
+        # the kernels move 16-byte vectors: feature counts that are not multiples of 8 are padded with
+        # zero channels, which change neither a Hadamard block of the real channels nor any absmax
         if x.dim() == 3 and args.batched_mode == "per_sample":
             tokens = x.shape[1]
-            opt = options_for(tokens, name)
-            bufs = [ops.abc_forward(x[b].contiguous(), opt) for b in range(x.shape[0])]
+            opt = options_for(tokens, name, w.shape[0])
+            _check_padding(w, opt)
+            bufs = [ops.abc_forward(_pad8(x[b]), opt) for b in range(x.shape[0])]
             xq = torch.stack([b[0] for b in bufs])
             sx = torch.cat([b[1] for b in bufs])
         else:
-            x2 = x.reshape(-1, x.shape[-1]).contiguous()
-            opt = options_for(x2.shape[0], name)
-            xq, sx = ops.abc_forward(x2, opt)
+            x2 = x.reshape(-1, x.shape[-1])
+            opt = options_for(x2.shape[0], name, w.shape[0])
+            _check_padding(w, opt)
+            xq, sx = ops.abc_forward(_pad8(x2), opt)
         ctx.opt = opt
         args.sr_step += 1
         ctx.save_for_backward(xq, w, sx)
@@ -138,21 +157,24 @@ class FLinearQ(Function):
         xq, w, sx = ctx.saved_tensors
         opt = ctx.opt
         go = grad_output
-        wc = w.contiguous()
+        O, I = w.shape
+        wc = _pad8(_pad8(w).t()).t().contiguous() if (O % 8 or I % 8) else w.contiguous()   # [O8, I8]
         if go.dtype != wc.dtype:
             go = go.to(wc.dtype)
         if go.dim() == 3 and args.batched_mode == "per_sample":
             gxs, gw = [], None
             for b in range(go.shape[0]):
-                gx_b, gw_b = ops.linear_backward(go[b].contiguous(), wc, xq[b], sx[b:b + 1], opt)
-                gxs.append(gx_b)
+                gx_b, gw_b = ops.linear_backward(_pad8(go[b]), wc, xq[b], sx[b:b + 1], opt)
+                gxs.append(gx_b[:, :I])
                 gw = gw_b.float() if gw is None else gw + gw_b.float()
             grad_input = torch.stack(gxs)
             grad_w = gw.to(wc.dtype)
         else:
-            go2 = go.reshape(-1, go.shape[-1]).contiguous()
-            gx, grad_w = ops.linear_backward(go2, wc, xq, sx, opt)
-            grad_input = gx.reshape(ctx.x_shape)
+            go2 = go.reshape(-1, go.shape[-1])
+            gx, grad_w = ops.linear_backward(_pad8(go2), wc, xq, sx, opt)
+            grad_input = gx[:, :I].reshape(ctx.x_shape)
+        if O % 8 or I % 8:
+            grad_w = grad_w[:O, :I]
         return grad_input, grad_w, None, None, None
 
 

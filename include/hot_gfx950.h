@@ -68,7 +68,7 @@ enum hot_rng_stream { HOT_STREAM_GX = 0, HOT_STREAM_GW = 1, HOT_STREAM_W = 2, HO
 /* Options of the fused path; mirrors the fields FLinearQ reads from the
  * reference's module-global `args` (args.py:29-49), scheme gih_gwlr. */
 typedef struct hot_config {
-  int32_t n_o;      /* Hadamard block along O: 16, 32 or 64                       */
+  int32_t n_o;      /* Hadamard block along O: a power of two, 1 .. 64            */
   int32_t hla_n;    /* HLA block along tokens: 1, 2, 4, ..., HOT_MAX_HLA_N        */
   int32_t hla_r;    /* kept coefficients per block, 1..hla_n                      */
   int32_t hla_rows[HOT_MAX_HLA_N]; /* natural-order row of output coefficient k  */

@@ -372,3 +372,63 @@ def test_backward_in_hip_graph(gpu):
         again = ops.linear_backward(gy, w, xq, sx, opt, workspace=ws)      # eager work between replays
         torch.cuda.synchronize()
         assert torch.equal(again[0], eager[0]) and torch.equal(again[1], eager[1])
+
+
+def test_small_vit_with_hot_layers(gpu, fresh_args):
+    """A whole (small) ViT with every Linear / Conv2d swapped: LQS calibration, then one HOT step whose
+    parameter gradients point the same way as the full-precision ones."""
+    from hot_amd import lqs, utils as hutils
+    from hot_amd.quant_matmul import HQ_Conv2d, HQ_Linear
+    from hot_amd.vit import ViT
+    torch.manual_seed(5)
+    model = ViT(image=32, patch=8, dim=64, depth=2, heads=4, mlp=128, classes=10, channels=8).to(gpu)
+    hutils.replace_layers(model, torch.nn.Conv2d, HQ_Conv2d)
+    hutils.replace_layers(model, torch.nn.Linear, HQ_Linear)
+    hutils.name_layers(model)
+    n_hot = sum(isinstance(m, (HQ_Linear, HQ_Conv2d)) for m in model.modules())
+    assert n_hot == 1 + 2 * 4 + 1
+    fresh_args.batched_mode = "flatten"
+    fresh_args.layer_quant_dict.clear()
+    x = torch.randn(16, 8, 32, 32, device=gpu)
+    t = torch.randint(0, 10, (16,), device=gpu)
+    lqs.calibrate(model, [(x, t)], torch.nn.CrossEntropyLoss())
+    assert len(fresh_args.layer_quant_dict) == 2 * n_hot
+    fresh_args.quantAuto = True
+    fresh_args.GogiQuantBit = fresh_args.weightQuantBit = 8          # a small model: keep the noise low
+    model.zero_grad()
+    torch.nn.functional.cross_entropy(model(x), t).backward()
+    hot = {n: p.grad.clone() for n, p in model.named_parameters()}
+    assert all(torch.isfinite(g).all() for g in hot.values())
+    for k_ in ("TransformGogi", "TransformWgt", "TransformGogw", "TransformInput"):
+        setattr(fresh_args, k_, False)
+    for k_ in ("quantBWDGogi", "quantBWDWgt", "quantBWDGogw", "quantBWDAct"):
+        setattr(fresh_args, k_, "no")
+    model.zero_grad()
+    torch.nn.functional.cross_entropy(model(x), t).backward()
+    for n, p in model.named_parameters():
+        if p.grad.numel() < 64:
+            continue
+        cos = torch.nn.functional.cosine_similarity(hot[n].flatten(), p.grad.flatten(), dim=0)
+        assert float(cos) > 0.5, (n, float(cos))
+
+
+@pytest.mark.parametrize("O,I", [(100, 96), (104, 100), (10, 36)])
+def test_hq_linear_odd_feature_counts(gpu, fresh_args, O, I):
+    """Heads and other layers whose widths are not multiples of 16: the Hadamard block along the
+    out-features follows the reference's rule (largest power of two dividing them, at most 16:
+    4 for 100 classes, 2 for 10) and widths that are not multiples of 8 are zero-padded on the way in."""
+    from hot_amd.quant_matmul import HQ_Linear
+    from hot_amd.hadamard_matmul import biggest_power2_factor_max16
+    L = 128
+    torch.manual_seed(7)
+    lin = HQ_Linear(I, O, bias=False).to(gpu)
+    x = torch.randn(L, I, device=gpu, requires_grad=True)
+    gy = torch.randn(L, O, device=gpu) * 1e-3
+    lin(x).backward(gy)
+    ocfg, _ = both_configs(L)
+    ocfg.n_o = biggest_power2_factor_max16(O)
+    assert ocfg.n_o == {100: 4, 104: 8, 10: 2}[O]
+    xq_ref, sx_ref = orc.abc_forward(x.detach().cpu().numpy(), ocfg)
+    tr = orc.linear_backward(gy.cpu().numpy(), lin.weight.detach().cpu().numpy(), xq_ref, sx_ref, ocfg)
+    assert np.array_equal(x.grad.cpu().numpy(), tr.g_x)
+    assert np.array_equal(lin.weight.grad.cpu().numpy(), tr.g_w)

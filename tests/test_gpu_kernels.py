@@ -111,13 +111,33 @@ def test_hq_rowwise_zero_and_empty(gpu):
     assert codes.shape == (0, 64)
 
 
+@pytest.mark.parametrize("n", [1, 2, 4, 8])
+@pytest.mark.parametrize("bits,scale,rounding", [(4, "tensor", "nearest"), (8, "row", "nearest"), (4, "row", "stoch")])
+def test_hq_rowwise_small_blocks(gpu, n, bits, scale, rounding):
+    """Blocks that fit one lane's chunk of 8 elements (heads whose width has few factors of two)."""
+    from hot_amd import ops
+    M, K = 37, 112
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(n)) * 1e-2
+    mode = orc.SCALE_TENSOR if scale == "tensor" else orc.SCALE_ROW
+    rnd = orc.ROUND_NEAREST if rounding == "nearest" else orc.ROUND_STOCH
+    t = orc.fwht_blocks_last(x.numpy(), n)
+    q_ref, s_ref = orc.quant(t, bits, mode, rnd, seed=5, stream=orc.STREAM_GX)
+    codes, s = ops.hq_rowwise(x.to(gpu), n=n, bits=bits, scale=scale, rounding=rounding, seed=5)
+    got = codes.cpu().numpy()
+    full = orc.unpack_int4(got) if bits == 4 else got
+    assert np.array_equal(s.cpu().numpy(), np.atleast_1d(s_ref).astype(np.float32).reshape(-1))
+    assert np.array_equal(full[:, :K], q_ref)
+
+
 def test_hq_rowwise_errors(gpu):
     from hot_amd import ops
     from hot_amd._lib import HotError
     with pytest.raises(HotError):
         ops.hq_rowwise(torch.zeros(4, 40, device=gpu), n=16)        # K % n
     with pytest.raises(HotError):
-        ops.hq_rowwise(torch.zeros(4, 64, device=gpu), n=8)         # block size
+        ops.hq_rowwise(torch.zeros(4, 64, device=gpu), n=12)        # block size: powers of two only
+    with pytest.raises(HotError):
+        ops.hq_rowwise(torch.zeros(4, 128, device=gpu), n=128)      # ... up to 64
     with pytest.raises(HotError):
         ops.hq_rowwise(torch.zeros(4, 64, device=gpu), bits=5)
     with pytest.raises(RuntimeError):
