@@ -215,6 +215,59 @@ def cpu_baseline(reps=5):
                 host_cpus=os.cpu_count())
 
 
+def vit_b16_backward(dev, batch=128, steps=3):
+    """Whole-model extra: ViT-B/16 (hot_amd/vit.py, random weights, bf16) on synthetic images, every
+    Linear / Conv2d swapped for the HOT layers, quantisers chosen per layer by the calibration pass;
+    backward time of one step against the same model with plain layers (hipBLASLt bf16)."""
+    import torch
+    import torch.nn as nn
+    from hot_amd import args, lqs
+    from hot_amd import utils as hutils
+    from hot_amd.quant_matmul import HQ_Conv2d, HQ_Linear
+    from hot_amd.vit import ViT
+
+    torch.manual_seed(0)
+    model = ViT().to(dev).to(torch.bfloat16)
+    img = torch.randn(batch, 3, 224, 224, device=dev, dtype=torch.bfloat16)
+    tgt = torch.randint(0, 100, (batch,), device=dev)
+
+    def backward_ms(m):
+        best = None
+        for it in range(steps + 1):
+            m.zero_grad(set_to_none=True)
+            loss = nn.functional.cross_entropy(m(img).float(), tgt)
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            loss.backward()
+            e1.record()
+            torch.cuda.synchronize()
+            if it > 0:
+                ms = e0.elapsed_time(e1)
+                best = ms if best is None else min(best, ms)
+        return best
+
+    plain = backward_ms(model)
+    saved = {k: getattr(args, k) for k in ("batched_mode", "quantAuto")}
+    try:
+        hutils.replace_layers(model, nn.Conv2d, HQ_Conv2d)
+        hutils.replace_layers(model, nn.Linear, HQ_Linear)
+        hutils.name_layers(model)
+        args.batched_mode = "flatten"
+        args.layer_quant_dict.clear()
+        lqs.calibrate(model, [(img[:32], tgt[:32])], nn.CrossEntropyLoss())
+        args.quantAuto = True
+        hot = backward_ms(model)
+        picks = list(args.layer_quant_dict.values())
+    finally:
+        for k, v in saved.items():
+            setattr(args, k, v)
+        args.layer_quant_dict.clear()
+    return {"model": "ViT-B/16, batch %d, bf16, flattened tokens" % batch, "backward_ms_plain_bf16": round(plain, 2),
+            "backward_ms_hot": round(hot, 2), "hot_layers": len(picks) // 2,
+            "per_token_quantiser_layers": sum(1 for i, v in enumerate(picks) if i % 2 == 0 and v == "norm_quantizer")}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -296,6 +349,11 @@ def main():
         out["llama_gate_up"] = {"us_per_layer": round(lsec * 1e6, 1), "L": Ll, "O": Ol, "I": Il,
                                 "hla": "n=16 r=8", "int8_tops": round((2.0 * Ll * Ol * Il + 2.0 * Ol * Il * (Ll // 2)) / lsec / 1e12, 1)}
         del lw, lsets
+    if not a.no_extras and not a.table_only:
+        try:
+            out["vit_b16"] = vit_b16_backward(dev)
+        except Exception as e:          # an extra: never costs the headline line
+            out["vit_b16"] = {"error": repr(e)[:200]}
     if not a.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
