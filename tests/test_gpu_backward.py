@@ -432,3 +432,23 @@ def test_hq_linear_odd_feature_counts(gpu, fresh_args, O, I):
     tr = orc.linear_backward(gy.cpu().numpy(), lin.weight.detach().cpu().numpy(), xq_ref, sx_ref, ocfg)
     assert np.array_equal(x.grad.cpu().numpy(), tr.g_x)
     assert np.array_equal(lin.weight.grad.cpu().numpy(), tr.g_w)
+
+
+@pytest.mark.parametrize("name", ["nearest_int4_L320_O64_I48", "stoch_row_int8_L192_O32_I40"])
+def test_backward_matches_golden_fixture(gpu, name):
+    """The committed fixtures (inputs, saved buffer, outputs) against the native path."""
+    import os
+    from hot_amd import ops
+    f = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", name + ".npz"))
+    stoch = name.startswith("stoch")
+    opt = ops.HotOptions(hla_n=int(f["hla_n"]), hla_rows=tuple(int(v) for v in f["hla_rows"]),
+                         gx_bits=8 if stoch else 4, w_bits=8 if stoch else 4,
+                         gx_round="stoch" if stoch else "nearest", gw_round="stoch" if stoch else "nearest",
+                         gx_scale="row" if stoch else "tensor", gw_scale="row" if stoch else "tensor",
+                         seed=1234 if stoch else 0)
+    x, w, gy = (torch.from_numpy(f[k]).to(gpu) for k in ("x", "w", "gy"))
+    xq, sx = ops.abc_forward(x, opt)
+    lp = f["xq"].shape[0]
+    assert np.array_equal(xq.cpu().numpy()[:, :lp], f["xq"].T) and np.array_equal(sx.cpu().numpy(), f["sx"])
+    gx, gw = ops.linear_backward(gy, w, xq, sx, opt)
+    assert np.array_equal(gx.cpu().numpy(), f["g_x"]) and np.array_equal(gw.cpu().numpy(), f["g_w"])

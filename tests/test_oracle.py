@@ -5,6 +5,7 @@ block_diag), brute force on small sizes, hand-derived tables, published
 known-answer vectors (Philox, Random123) and statistical properties.  None of
 the checks re-types the oracle's own formula."""
 import itertools
+import os
 
 import numpy as np
 import pytest
@@ -341,3 +342,24 @@ def test_reference_cuda_rounding_is_biased():
     only): values with an all-zero mantissa (0 and the powers of two) are
     rounded UP, so it cannot be unbiased."""
     assert orc.stoch_round_mantissa(np.array([2.0, -3.0, 0.0, 4.0], F32)).tolist() == [3, -3, 1, 5]
+
+
+# ------------------------------------------------------------------ frozen snapshots of the oracle
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+
+
+@pytest.mark.parametrize("name", ["nearest_int4_L320_O64_I48", "stoch_row_int8_L192_O32_I40"])
+def test_oracle_matches_its_frozen_snapshots(name):
+    """tests/golden/*.npz were written by tests/golden/make_fixtures.py from this oracle: any change of
+    its arithmetic (butterfly order, rounding, RNG numbering, nibble order) shows up here."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("make_fixtures", os.path.join(GOLDEN, "make_fixtures.py"))
+    mk = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mk)
+    data_seed, L, O, I, kw = mk.CASES[name]
+    fresh = mk.case(data_seed, L, O, I, **kw)
+    frozen = np.load(os.path.join(GOLDEN, name + ".npz"))
+    assert set(frozen.files) == set(fresh)
+    for k in frozen.files:
+        assert np.array_equal(frozen[k], np.asarray(fresh[k])), k
