@@ -237,7 +237,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       const int blk = bl + g;
       if (blk < nblk) {
         int visited = 0;      // kept coefficients of this block quantised so far (stochastic rounding)
-        float u[4] = {0.f, 0.f, 0.f, 0.f};
+        float u[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int i = 0; i < N; ++i) {
           int sl;
@@ -255,14 +255,13 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
                 // the rounded code cannot leave [-qmax, qmax]
                 q = (int)rint_div_fast(v, d, rcp);
               } else {
-                // counter = ((channel * NB + block) * rpad + visit index) / 4, word = visit index % 4
-                if ((visited & 3) == 0) {
-                  const uint64_t quad = ((uint64_t)c * (uint64_t)a.NB + (uint64_t)(blk0 + blk)) * (uint64_t)(a.rpad >> 2) +
-                                        (uint64_t)(visited >> 2);
-                  sr_uniform4(quad, a.seed, a.stream, u);
+                // counter = ((channel * NB + block) * rpad + visit index) / 8, slot = visit index % 8
+                if ((visited & 7) == 0) {
+                  const uint64_t oct = ((uint64_t)c * (uint64_t)a.NB + (uint64_t)(blk0 + blk)) * (uint64_t)(a.rpad >> 3) +
+                                       (uint64_t)(visited >> 3);
+                  sr_uniform8(oct, a.seed, a.stream, u);
                 }
-                const int w = visited & 3;
-                q = q_stoch_div(v, d, rcp, w == 0 ? u[0] : w == 1 ? u[1] : w == 2 ? u[2] : u[3]);
+                q = q_stoch_div(v, d, rcp, u[visited & 7]);
                 ++visited;
                 q = clampi(q, -qmax, qmax);   // floor + 1 may step past qmax at the very top
               }
@@ -551,7 +550,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   a.in = in; a.R = R; a.C = C; a.NB = R / n; a.Kout = a.NB * r;
   a.out = (int8_t*)codes_out; a.ld_out = ld_out;
   a.seed = seed; a.stream = rng_stream;
-  a.r = r; a.rpad = (r + 3) & ~3; a.bits = bits; a.rounding = rounding; a.mode = scale_mode; a.tb = 4;
+  a.r = r; a.rpad = (r + 7) & ~7; a.bits = bits; a.rounding = rounding; a.mode = scale_mode; a.tb = 4;
   for (int i = 0; i < HOT_MAX_HLA_N; ++i) a.slot[i] = -1;
   for (int k = 0; k < r; ++k) {
     if (rows[k] < 0 || rows[k] >= n) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d outside [0, %d)", who, k, rows[k], n);

@@ -132,20 +132,16 @@ __device__ __forceinline__ philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint3
   return o;
 }
 
-// Uniforms for the four elements whose linear indices are 4*quad .. 4*quad+3.
-__device__ __forceinline__ void sr_uniform4(uint64_t quad, uint64_t seed, uint32_t stream, float* u) {
-  const philox4 p = philox4x32_10((uint32_t)quad, (uint32_t)(quad >> 32), stream, 0u,
+// Uniforms (2^-16 grid) for the eight elements whose linear indices are 8*oct .. 8*oct+7: element
+// 2 i + h takes the low (h = 0) or high (h = 1) half of output word i of one Philox call.
+__device__ __forceinline__ void sr_uniform8(uint64_t oct, uint64_t seed, uint32_t stream, float* u) {
+  const philox4 p = philox4x32_10((uint32_t)oct, (uint32_t)(oct >> 32), stream, 0u,
                                   (uint32_t)seed, (uint32_t)(seed >> 32));
 #pragma unroll
-  for (int i = 0; i < 4; ++i) u[i] = (float)(p.w[i] >> 8) * 5.9604644775390625e-08f;  // 2^-24
-}
-
-// Uniform of the single element with linear index e.
-__device__ __forceinline__ float sr_uniform1(uint64_t e, uint64_t seed, uint32_t stream) {
-  float u[4];
-  sr_uniform4(e >> 2, seed, stream, u);
-  const uint32_t l = (uint32_t)e & 3u;
-  return l == 0 ? u[0] : l == 1 ? u[1] : l == 2 ? u[2] : u[3];
+  for (int i = 0; i < 4; ++i) {
+    u[2 * i] = (float)(p.w[i] & 0xFFFFu) * 1.52587890625e-05f;      // 2^-16
+    u[2 * i + 1] = (float)(p.w[i] >> 16) * 1.52587890625e-05f;
+  }
 }
 
 // ---- quantisation of one value --------------------------------------------

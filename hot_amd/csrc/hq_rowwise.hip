@@ -80,8 +80,7 @@ __device__ __forceinline__ void quant_store_chunk(const float* x, float d, float
     for (int j = 0; j < EPL; ++j) q[j] = (int)rint_div_fast(x[j], d, rcp);
   } else {
     float u[EPL];
-    sr_uniform4(e0 >> 2, seed, stream, u);
-    sr_uniform4((e0 >> 2) + 1, seed, stream, u + 4);
+    sr_uniform8(e0 >> 3, seed, stream, u);       // e0 is a multiple of EPL = 8
 #pragma unroll
     for (int j = 0; j < EPL; ++j) q[j] = clampi(q_stoch_div(x[j], d, rcp, u[j]), -QMAX, QMAX);
   }

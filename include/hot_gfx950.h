@@ -110,7 +110,7 @@ HOT_API int hot_hq_rowwise(const void* in, int dtype, int64_t M, int64_t K, int 
  *   workspace   device, >= hot_colwise_workspace_bytes(C)
  * Stochastic rounding numbers the kept coefficients of block b of channel c
  * in increasing natural-row order v = 0..r-1 and gives coefficient v the RNG
- * element index ((c * (R/n) + b) * rpad + v), rpad = r rounded up to 4.
+ * element index ((c * (R/n) + b) * rpad + v), rpad = r rounded up to 8.
  */
 HOT_API int hot_hla_tokenwise(const void* in, int dtype, int64_t R, int64_t C, int n,
                       const int32_t* rows, int r, int bits, int rounding, uint64_t seed,

@@ -229,16 +229,20 @@ def philox4x32(c0, c1, c2, c3, k0: int, k1: int, rounds: int = 10):
 
 
 def sr_uniform(index: np.ndarray, seed: int, stream: int) -> np.ndarray:
-    """u in [0, 1) on a 2^-24 grid for the element with linear index ``index``
-    (int64 array): counter = (index>>2 lo, index>>2 hi, stream, 0),
-    key = (seed lo, seed hi), word = index & 3, u = (word >> 8) * 2^-24."""
+    """u in [0, 1) on a 2^-16 grid for the element with linear index ``index``
+    (int64 array).  One Philox call serves eight consecutive elements:
+    counter = (index>>3 lo, index>>3 hi, stream, 0), key = (seed lo, seed hi);
+    element index & 7 = 2 i + h takes the low (h = 0) or high (h = 1) 16 bits of
+    output word i, u = halfword * 2^-16.  (Sixteen bits bound the bias of a
+    rounding probability by 2^-16 of a quantisation step.)"""
     index = np.asarray(index, dtype=np.uint64)
-    q = index >> np.uint64(2)
+    q = index >> np.uint64(3)
     w = philox4x32(q & _MASK, q >> np.uint64(32), np.full(q.shape, stream, np.uint64),
                    np.zeros(q.shape, np.uint64), seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF)
-    lane = (index & np.uint64(3)).astype(np.int64)
-    word = np.choose(lane, w)
-    return ((word >> np.uint32(8)).astype(F32) * F32(2.0 ** -24)).astype(F32)
+    slot = (index & np.uint64(7)).astype(np.int64)
+    word = np.choose(slot >> 1, w).astype(np.uint32)
+    half = np.where((slot & 1) == 0, word & np.uint32(0xFFFF), word >> np.uint32(16))
+    return (half.astype(F32) * F32(2.0 ** -16)).astype(F32)
 
 
 # --------------------------------------------------------------------------
@@ -402,11 +406,11 @@ def colwise_rng_index(C: int, NB: int, rows) -> np.ndarray:
     """RNG element index of every coefficient of a column-wise transformed
     matrix, laid out [C, NB * r] (K-major).  The kernels walk the kept
     coefficients of a block in increasing natural-row order and number them
-    ((c * NB + block) * rpad + visit) with rpad = r rounded up to 4, so that one
-    Philox call serves four consecutive visits of a channel."""
+    ((c * NB + block) * rpad + visit) with rpad = r rounded up to 8, so that one
+    Philox call serves eight consecutive visits of a channel."""
     rows = np.asarray(rows)
     r = len(rows)
-    rpad = (r + 3) // 4 * 4
+    rpad = (r + 7) // 8 * 8
     visit = np.argsort(np.argsort(rows))                      # rank of rows[k] among the kept rows
     c = np.arange(C, dtype=np.int64)[:, None, None]
     b = np.arange(NB, dtype=np.int64)[None, :, None]

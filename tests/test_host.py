@@ -170,7 +170,7 @@ def test_library_argument_checks_need_no_gpu():
     from hot_amd import _lib, ops
     lib = _lib.lib()
     one = C.c_void_p(4096)  # never dereferenced: every call below fails validation first
-    assert lib.hot_hq_rowwise(one, 0, 4, 64, 8, 4, 0, 0, 0, 0, one, one, None, 0, None) == -2
+    assert lib.hot_hq_rowwise(one, 0, 4, 64, 12, 4, 0, 0, 0, 0, one, one, None, 0, None) == -2
     assert b"Hadamard block" in lib.hot_last_error()
     assert lib.hot_hq_rowwise(one, 0, 4, 40, 16, 4, 0, 0, 0, 0, one, one, None, 0, None) == -1
     assert lib.hot_hq_rowwise(one, 0, 4, 64, 16, 4, 0, 0, 0, 0, one, one, None, 0, None) == -3   # no workspace
@@ -183,7 +183,7 @@ def test_library_argument_checks_need_no_gpu():
     need = lib.hot_backward_workspace_bytes(12608, 3072, 768, C.byref(cfg))
     # packed g_y codes + packed W codes + int8 low-rank g_y codes dominate
     assert need >= 12608 * 1536 + 768 * 1536 + 3072 * 7168
-    cfg.n_o = 8
+    cfg.n_o = 12            # not a power of two
     assert lib.hot_backward_workspace_bytes(12608, 3072, 768, C.byref(cfg)) == 0
     with pytest.raises(_lib.HotError):
         _lib.check(-2)

@@ -169,6 +169,13 @@ def test_sr_uniform_range_and_moments():
     assert not np.array_equal(u, orc.sr_uniform(np.arange(1 << 16), seed=12346, stream=1))
     assert not np.array_equal(u, orc.sr_uniform(np.arange(1 << 16), seed=12345, stream=2))
     assert np.array_equal(u[4:8], orc.sr_uniform(np.arange(4, 8), seed=12345, stream=1))
+    # elements 8 q .. 8 q + 7 share Philox call q: low half of word 0, high half of word 0, low half of word 1, ...
+    w = orc.philox4x32(np.array([5], np.uint64), np.array([0], np.uint64), np.array([1], np.uint64),
+                       np.array([0], np.uint64), 12345, 0)
+    halves = []
+    for i in range(4):
+        halves += [int(w[i][0]) & 0xFFFF, int(w[i][0]) >> 16]
+    assert np.array_equal(u[40:48], (np.array(halves, dtype=np.float32) / np.float32(65536.0)))
 
 
 # --------------------------------------------------------------- quantisers
