@@ -215,6 +215,39 @@ def cpu_baseline(reps=5):
                 host_cpus=os.cpu_count())
 
 
+def hq_rowwise_sweep(dev):
+    """Kernel-level extra: the fused block-Hadamard + per-token absmax step + quantise kernel alone
+    (hot_hq_rowwise, bf16 input with per-channel scales drawn log-uniform in [0.1, 10]), GB/s of
+    algorithmic bytes (input read once + codes + steps written) against the 8 TB/s HBM peak."""
+    import torch
+    from hot_amd import ops
+    rows = []
+    g = torch.Generator(device=dev).manual_seed(0)
+    for M in (4096, 16384, 65536):
+        for K in (768, 3072, 4096, 11008):
+            x = (torch.randn(M, K, generator=g, device=dev) *
+                 (10.0 ** (torch.rand(K, generator=g, device=dev) * 2 - 1))).to(torch.bfloat16)
+            for n in (16, 32, 64):
+                if K % n:
+                    continue
+                for bits in (4, 8):
+                    for _ in range(3):
+                        ops.hq_rowwise(x, n=n, bits=bits, scale="row")
+                    torch.cuda.synchronize()
+                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                    e0.record()
+                    for _ in range(10):
+                        ops.hq_rowwise(x, n=n, bits=bits, scale="row")
+                    e1.record()
+                    torch.cuda.synchronize()
+                    us = e0.elapsed_time(e1) * 100.0
+                    byt = M * K * 2 + M * K * bits // 8 + 4 * M
+                    rows.append([M, K, n, bits, round(us, 1), round(byt / us / 1e3), round(byt / us / 1e3 / HBM_PEAK_GBS, 3)])
+            del x
+    return {"columns": ["M", "K", "hadamard_block", "bits", "us", "GB/s", "frac_of_8TB/s"], "rows": rows,
+            "note": "per-token steps, round-to-nearest; includes the Python wrapper (about 14 us floor)"}
+
+
 def vit_b16_backward(dev, batch=128, steps=3):
     """Whole-model extra: ViT-B/16 (hot_amd/vit.py, random weights, bf16) on synthetic images, every
     Linear / Conv2d swapped for the HOT layers, quantisers chosen per layer by the calibration pass;
@@ -358,6 +391,10 @@ def main():
                                 "hla": "n=16 r=8", "int8_tops": round((2.0 * Ll * Ol * Il + 2.0 * Ol * Il * (Ll // 2)) / lsec / 1e12, 1)}
         del lw, lsets
     if not a.no_extras and not a.table_only:
+        try:
+            out["hq_rowwise_sweep"] = hq_rowwise_sweep(dev)
+        except Exception as e:
+            out["hq_rowwise_sweep"] = {"error": repr(e)[:200]}
         try:
             out["vit_b16"] = vit_b16_backward(dev)
         except Exception as e:          # an extra: never costs the headline line
