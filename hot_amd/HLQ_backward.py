@@ -25,7 +25,7 @@ gx_bits = 4
 gw_bits = 8
 gx_rounding = "stoch"
 other_rounding = "nearest"
-hla_max_block = 64
+hla_max_block = 8192     # see hot_amd.args.hla_max_block
 seed = 0
 
 

@@ -11,7 +11,8 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libhot_gfx950.so")
 
-HOT_MAX_HLA_N = 64
+HOT_MAX_HLA_N = 64        # rows inline in the config
+HOT_MAX_HLA_BIG = 8192    # rows through hla_rows_big
 
 # enums of include/hot_gfx950.h
 F32, BF16, F16 = 0, 1, 2
@@ -23,7 +24,7 @@ EXPORTS = (
     "hot_last_error", "hot_abi_version", "hot_kpad", "hot_hq_rowwise", "hot_hla_tokenwise",
     "hot_wq_colwise", "hot_colwise_workspace_bytes", "hot_gemm_i8", "hot_abc_workspace_bytes",
     "hot_abc_forward", "hot_backward_workspace_bytes", "hot_linear_backward", "hot_linear_backward_kernels",
-    "hot_gemm_splits",
+    "hot_gemm_splits", "hot_hla_workspace_bytes",
 )
 
 
@@ -36,6 +37,7 @@ class HotConfig(C.Structure):
         ("gx_round", C.c_int32), ("w_round", C.c_int32), ("gw_round", C.c_int32), ("act_round", C.c_int32),
         ("gx_scale", C.c_int32), ("w_scale", C.c_int32), ("gw_scale", C.c_int32), ("act_scale", C.c_int32),
         ("seed", C.c_uint64),
+        ("hla_rows_big", C.POINTER(C.c_int32)),
     ]
 
 
@@ -62,6 +64,8 @@ def _declare(lib):
                                       vp, i64, vp, vp, sz, vp]
     lib.hot_wq_colwise.restype = i32
     lib.hot_wq_colwise.argtypes = [vp, i32, i64, i64, i32, i32, i32, u64, u32, i32, vp, i64, vp, vp, sz, vp]
+    lib.hot_hla_workspace_bytes.restype = sz
+    lib.hot_hla_workspace_bytes.argtypes = [i64, i64, i32, i32]
     lib.hot_colwise_workspace_bytes.restype = sz
     lib.hot_colwise_workspace_bytes.argtypes = [i64]
     lib.hot_gemm_i8.restype = i32

@@ -43,9 +43,11 @@ layer_quant_dict = defaultdict()
 # Token-dimension rule for the low-rank projection: "python" = the reference's
 # make_WHT rule on the token count, "paper" = n 16 / 8 lowest sequencies.
 hla_rule = "python"
-# The kernels hold one token block in registers; when the python rule asks for a
-# larger block (for example 8192 tokens -> n = 8192) the block is limited to this.
-hla_max_block = 64
+# Largest token block of the python rule.  The reference takes the largest power of two dividing the
+# token count, whatever it is (8192 tokens -> n = 8192, r = 2080); blocks up to 64 tokens run in the
+# fast one-pass kernels, larger ones in an exact two-level path through an fp32 workspace.  Lower this
+# (for example to 64: then n = 64, r = 36) to trade the reference's compression ratio for speed.
+hla_max_block = 8192
 # 3-D activations [B, L, C]: "per_sample" follows the reference (one call and one
 # set of steps per sample), "flatten" treats them as [B*L, C].
 batched_mode = "per_sample"

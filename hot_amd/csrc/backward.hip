@@ -32,10 +32,13 @@ int check_hip(hipError_t e, const char* what) {
 
 int check_launch(const char* what) { return check_hip(hipGetLastError(), what); }
 
+static const int32_t* cfg_rows(const hot_config* c) { return c->hla_n > HOT_MAX_HLA_N ? c->hla_rows_big : c->hla_rows; }
+
 static int check_cfg(const hot_config* c, const char* who) {
   if (!c) return fail(HOT_ERR_INVALID, "%s: null config", who);
   if (c->n_o < 1 || c->n_o > 64 || (c->n_o & (c->n_o - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: n_o=%d (a power of two up to 64)", who, c->n_o);
-  if (c->hla_n < 1 || c->hla_n > HOT_MAX_HLA_N || (c->hla_n & (c->hla_n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: hla_n=%d (power of two up to %d)", who, c->hla_n, HOT_MAX_HLA_N);
+  if (c->hla_n < 1 || c->hla_n > HOT_MAX_HLA_BIG || (c->hla_n & (c->hla_n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: hla_n=%d (power of two up to %d)", who, c->hla_n, HOT_MAX_HLA_BIG);
+  if (c->hla_n > HOT_MAX_HLA_N && !c->hla_rows_big) return fail(HOT_ERR_INVALID, "%s: hla_n=%d needs hla_rows_big", who, c->hla_n);
   if (c->hla_r < 1 || c->hla_r > c->hla_n) return fail(HOT_ERR_INVALID, "%s: hla_r=%d outside [1, %d]", who, c->hla_r, c->hla_n);
   const int bits[4] = {c->gx_bits, c->w_bits, c->gw_bits, c->act_bits};
   for (int i = 0; i < 4; ++i)
@@ -60,7 +63,7 @@ static BwdLayout bwd_layout(int64_t L, int64_t O, int64_t I, const hot_config* c
   size_t o = 0;
   b.off_hq = o;   o += 256;
   b.off_colw = o; o += align256(colwise_workspace_bytes_impl(I));
-  b.off_colg = o; o += align256(colwise_workspace_bytes_impl(O));
+  b.off_colg = o; o += align256(hla_workspace_bytes_impl(L, O, c->hla_n, c->hla_r));
   b.off_sg = o;   o += align256((size_t)L * 4);
   b.off_sw = o;   o += 256;
   b.off_sgp = o;  o += align256((size_t)O * 4);
@@ -115,6 +118,11 @@ int hot_hq_rowwise(const void* in, int dtype, int64_t M, int64_t K, int n, int b
 
 size_t hot_colwise_workspace_bytes(int64_t C) { return colwise_workspace_bytes_impl(C > 0 ? C : 0); }
 
+size_t hot_hla_workspace_bytes(int64_t R, int64_t C, int n, int r) {
+  if (R <= 0 || C <= 0 || n < 1 || r < 1) return 0;
+  return hla_workspace_bytes_impl(R, C, n, r);
+}
+
 int hot_hla_tokenwise(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r,
                       int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
                       void* codes_out, int64_t ld_out, float* scales_out, void* workspace,
@@ -141,8 +149,8 @@ int hot_gemm_i8(const void* A, int64_t lda, const void* B, int64_t ldb, int bits
 }
 
 size_t hot_abc_workspace_bytes(int64_t L, int64_t I, const hot_config* cfg) {
-  (void)L; (void)cfg;
-  return colwise_workspace_bytes_impl(I > 0 ? I : 0);
+  if (!cfg || L <= 0 || I <= 0) return colwise_workspace_bytes_impl(I > 0 ? I : 0);
+  return hla_workspace_bytes_impl(L, I, cfg->hla_n, cfg->hla_r);
 }
 
 int hot_abc_forward(const void* x, int dtype, int64_t L, int64_t I, const hot_config* cfg, void* xq_out,
@@ -151,7 +159,7 @@ int hot_abc_forward(const void* x, int dtype, int64_t L, int64_t I, const hot_co
   if (L <= 0 || I <= 0 || L % cfg->hla_n) return fail(HOT_ERR_INVALID, "hot_abc_forward: L=%lld must be a positive multiple of hla_n=%d", (long long)L, cfg->hla_n);
   if (cfg->act_scale == HOT_SCALE_ROW) return fail(HOT_ERR_UNSUPPORTED, "hot_abc_forward: the activation buffer uses one step per tensor");
   const int64_t lp = (L / cfg->hla_n) * cfg->hla_r;
-  return colwise_quant_impl(x, dtype, L, I, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->act_bits, cfg->act_round,
+  return colwise_quant_impl(x, dtype, L, I, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, cfg->act_bits, cfg->act_round,
                             cfg->seed, HOT_STREAM_ACT, cfg->act_scale, xq_out, round_up(lp, GEMM_KTILE), 0,
                             sx_out, workspace, workspace_bytes, (hipStream_t)hip_stream, "hot_abc_forward");
 }
@@ -270,15 +278,16 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   // g_y: HLA along tokens + quantise, transposed (g_W operand); Hadamard along O + quantise (g_x
   // operand).  With one step per tensor both quantisers need the absmax of their transform first:
   // the statistics pass of the token-wise kernel delivers both from a single read of g_y.
-  const bool fuse = cfg->gx_scale == HOT_SCALE_TENSOR && cfg->n_o == 16 && O % 16 == 0 && cfg->gw_scale != HOT_SCALE_SAWB;
+  const bool fuse = cfg->gx_scale == HOT_SCALE_TENSOR && cfg->n_o == 16 && O % 16 == 0 && cfg->gw_scale != HOT_SCALE_SAWB &&
+                    cfg->hla_n <= HOT_MAX_HLA_N;
   // Side stream, beside the g_W GEMM on the main stream: always the row-wise quantise pass of g_y (a
   // streaming kernel next to a matrix kernel); the g_x GEMM too when the g_W GEMM has fewer tiles
   // than the chip has CUs and cannot fill it alone (two large GEMMs only get in each other's way).
   const bool hq_aside = side != nullptr;
   const bool gx_aside = side != nullptr && ((O + 127) / 128) * ((I + 127) / 128) < 256;
-  rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg->hla_rows, cfg->hla_r, cfg->gw_bits, cfg->gw_round,
+  rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, cfg->gw_bits, cfg->gw_round,
                           cfg->seed, HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp,
-                          ws + b.off_colg, colwise_workspace_bytes_impl(O), st, who,
+                          ws + b.off_colg, hla_workspace_bytes_impl(L, O, cfg->hla_n, cfg->hla_r), st, who,
                           fuse ? (float*)(ws + b.off_hq) : nullptr, /*stats_cleared=*/true,
                           hq_aside ? side->fork2 : mid(K_GY_STATS));
   if (rc) return rc;

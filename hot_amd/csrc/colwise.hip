@@ -441,6 +441,10 @@ static constexpr size_t COL_STAT_BYTES = 256;
 
 size_t colwise_stats_bytes_impl(int64_t C) { return COL_STAT_BYTES + (size_t)round_up(C * 4, 256); }
 
+size_t hla_workspace_bytes_impl(int64_t R, int64_t C, int n, int r) {
+  return n > HOT_MAX_HLA_N ? hla_big_workspace_bytes_impl(R, C, n, r) : colwise_workspace_bytes_impl(C);
+}
+
 size_t colwise_workspace_bytes_impl(int64_t C) {
   // stat | per-channel max | per-workgroup partial sums (at most 65536 workgroups)
   return COL_STAT_BYTES + (size_t)round_up(C * 4, 256) + (size_t)(2 * sizeof(double)) * 65536;
@@ -536,6 +540,17 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
                        bool stats_cleared, hipEvent_t after_stats) {
   if (!in || !codes_out || !scales_out || !rows) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
   if (R <= 0 || C <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape R=%lld C=%lld", who, (long long)R, (long long)C);
+  if (n > HOT_MAX_HLA_N) {
+    // blocks one thread cannot hold: the two-level path
+    if (store4 || row16_absmax_out) return fail(HOT_ERR_UNSUPPORTED, "%s: blocks above %d tokens have no packed-INT4 store and no fused row statistic", who, HOT_MAX_HLA_N);
+    if (R % n) return fail(HOT_ERR_INVALID, "%s: R=%lld is not a multiple of the block %d", who, (long long)R, n);
+    if (r < 1 || r > n) return fail(HOT_ERR_INVALID, "%s: r=%d outside [1, %d]", who, r, n);
+    if (bits != 4 && bits != 8) return fail(HOT_ERR_UNSUPPORTED, "%s: bits=%d (4 or 8)", who, bits);
+    if (rounding != HOT_ROUND_NEAREST && rounding != HOT_ROUND_STOCH) return fail(HOT_ERR_INVALID, "%s: bad rounding %d", who, rounding);
+    if (scale_mode < HOT_SCALE_TENSOR || scale_mode > HOT_SCALE_SAWB) return fail(HOT_ERR_INVALID, "%s: bad scale mode %d", who, scale_mode);
+    return hla_big_impl(in, dtype, R, C, n, rows, r, bits, rounding, seed, rng_stream, scale_mode, codes_out, ld_out,
+                        scales_out, workspace, workspace_bytes, st, who, after_stats);
+  }
   if (n < 1 || n > HOT_MAX_HLA_N || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (power of two up to %d)", who, n, HOT_MAX_HLA_N);
   if (R % n) return fail(HOT_ERR_INVALID, "%s: R=%lld is not a multiple of the block %d", who, (long long)R, n);
   if (r < 1 || r > n) return fail(HOT_ERR_INVALID, "%s: r=%d outside [1, %d]", who, r, n);

@@ -1,0 +1,333 @@
+// Hadamard low-rank projection along tokens for blocks larger than one thread can hold:
+// n = 64 m tokens, m = 2 .. 128 (the reference's make_WHT rule asks for the largest power of two
+// dividing the token count: 128 for 25216 tokens, 8192 for 8192; utils/hadamard_matmul.py:209-226).
+//
+// A Sylvester transform of n = 64 m points is the 64-point transform inside each run of 64 rows
+// followed by the m-point transform across the runs, and the canonical butterfly order
+// (h = 1, 2, 4, ...) is exactly that sequence: stages h < 64 stay inside a run, stages h >= 64 pair
+// run j with run j ^ (h / 64).  Two kernels therefore reproduce the one-pass arithmetic bit for bit:
+//   stage 1   every run of 64 rows of a channel -> fp32 coefficients, written back in place of the
+//             rows into a workspace T [R, C]
+//   stage 2   for coefficient k of the runs of one block: the m values T[(64 j + k), c] -> m-point
+//             transform -> natural-order coefficient 64 j + k of the block; kept ones are measured
+//             (statistics pass) or quantised (quantise pass) into codes [L', C]
+//   transpose codes [L', C] -> [C, ld] (K-major for the GEMM), padding zeroed
+// This is the exactness path for large blocks, not a tuned one: the input is read with scalar loads
+// and the coefficients make a round trip through HBM in fp32.
+#include <algorithm>
+#include <vector>
+
+#include "hot_device.h"
+#include "hot_host.h"
+
+namespace hot {
+
+namespace {
+
+constexpr int BT = 256;  // threads per workgroup = channels per workgroup
+
+struct BigArgs {
+  const void* in;
+  float* T;            // [R, C] fp32 coefficients of the 64-point stage
+  int8_t* tmp;         // [Kout, C] codes before the transpose
+  const int32_t* tab;  // per natural row of a block: slot | visit << 16, or -1 when dropped
+  int64_t R, C, NB;    // NB = R / n blocks
+  int32_t n, r, rpad, bits, rounding, mode;
+  float* stat;         // [0] absmax, [1] step, [2] clip
+  float* colmax;       // per-channel absmax (ROW)
+  double* partial;     // SAWB: 2 doubles per workgroup
+  float* scales_out;
+  uint64_t seed;
+  uint32_t stream;
+};
+
+template <typename T> __device__ __forceinline__ float load_f32(const T* p);
+template <> __device__ __forceinline__ float load_f32<float>(const float* p) { return *p; }
+template <> __device__ __forceinline__ float load_f32<bf16_t>(const bf16_t* p) { return as_f((uint32_t)p->v << 16); }
+template <> __device__ __forceinline__ float load_f32<f16_t>(const f16_t* p) { return (float)p->v; }
+
+template <int N>
+__device__ __forceinline__ void fwht(float (&v)[N]) {
+#pragma unroll
+  for (int h = 1; h < N; h <<= 1) {
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      if ((i & h) == 0) {
+        const float a = v[i], b = v[i + h];
+        v[i] = a + b;
+        v[i + h] = a - b;
+      }
+    }
+  }
+}
+
+template <typename T>
+__global__ void __launch_bounds__(BT) big_stage1_kernel(const BigArgs a) {
+  const int64_t c = (int64_t)blockIdx.x * BT + threadIdx.x;
+  if (c >= a.C) return;
+  const int64_t row0 = (int64_t)blockIdx.y * 64;
+  const T* in = reinterpret_cast<const T*>(a.in) + row0 * a.C + c;
+  float v[64];
+#pragma unroll
+  for (int i = 0; i < 64; ++i) v[i] = load_f32<T>(in + (int64_t)i * a.C);
+  fwht<64>(v);
+  float* out = a.T + row0 * a.C + c;
+#pragma unroll
+  for (int i = 0; i < 64; ++i) out[(int64_t)i * a.C] = v[i];
+}
+
+__device__ __forceinline__ float uniform_of(uint64_t e, uint64_t seed, uint32_t stream) {
+  float u[8];
+  sr_uniform8(e >> 3, seed, stream, u);
+  float r = u[0];
+#pragma unroll
+  for (int i = 1; i < 8; ++i) r = ((uint32_t)e & 7u) == (uint32_t)i ? u[i] : r;
+  return r;
+}
+
+// blockIdx.y = block * 64 + k
+template <int M, int PASS, int ROUND, bool SAWB>
+__global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
+  __shared__ float s_max[BT / 64];
+  __shared__ double s_sum[2][BT / 64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t c = (int64_t)blockIdx.x * BT + tid;
+  const bool active = c < a.C;
+  const int64_t blk = blockIdx.y >> 6;
+  const int k = blockIdx.y & 63;
+  const int qmax = (1 << (a.bits - 1)) - 1;
+  float v[M];
+  if (active) {
+    const float* t = a.T + (blk * a.n + k) * a.C + c;
+#pragma unroll
+    for (int j = 0; j < M; ++j) v[j] = t[(int64_t)j * 64 * a.C];
+  } else {
+#pragma unroll
+    for (int j = 0; j < M; ++j) v[j] = 0.f;
+  }
+  fwht<M>(v);
+
+  if constexpr (PASS == 0) {
+    float cmax = 0.f;
+    double ssq = 0.0, sab = 0.0;
+#pragma unroll
+    for (int j = 0; j < M; ++j) {
+      if (a.tab[j * 64 + k] >= 0) {
+        cmax = fmaxf(cmax, fabsf(v[j]));
+        if constexpr (SAWB) { ssq += (double)v[j] * (double)v[j]; sab += (double)fabsf(v[j]); }
+      }
+    }
+    if (a.mode == HOT_SCALE_ROW) {
+      if (active) atomic_max_nonneg(a.colmax + c, cmax);
+      return;
+    }
+    if (a.mode == HOT_SCALE_TENSOR) {
+      const float m = wave_max(active ? cmax : 0.f);
+      if (lane == 0) s_max[wave] = m;
+      __syncthreads();
+      if (tid == 0) {
+        float mm = s_max[0];
+        for (int i = 1; i < BT / 64; ++i) mm = fmaxf(mm, s_max[i]);
+        atomic_max_nonneg(a.stat, mm);
+      }
+      return;
+    }
+    ssq = wave_sum(active ? ssq : 0.0);
+    sab = wave_sum(active ? sab : 0.0);
+    if (lane == 0) { s_sum[0][wave] = ssq; s_sum[1][wave] = sab; }
+    __syncthreads();
+    if (tid == 0) {
+      double q = 0.0, b = 0.0;
+      for (int i = 0; i < BT / 64; ++i) { q += s_sum[0][i]; b += s_sum[1][i]; }
+      const int64_t wg = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
+      a.partial[2 * wg] = q;
+      a.partial[2 * wg + 1] = b;
+    }
+  } else {
+    if (!active) return;
+    float d, clip = 0.f;
+    if (a.mode == HOT_SCALE_ROW) d = a.colmax[c] / (float)qmax + 1e-11f;
+    else if (a.mode == HOT_SCALE_TENSOR) d = a.stat[0] / (float)qmax + 1e-11f;
+    else { d = a.stat[1] + 1e-11f; clip = a.stat[2]; }
+#pragma unroll
+    for (int j = 0; j < M; ++j) {
+      const int32_t e = a.tab[j * 64 + k];
+      if (e < 0) continue;
+      const int slot = e & 0xFFFF, visit = e >> 16;
+      float x = v[j];
+      if constexpr (SAWB) x = fminf(fmaxf(x, -clip), clip);
+      int q;
+      if constexpr (ROUND == HOT_ROUND_NEAREST) {
+        q = (int)rintf(x / d);
+      } else {
+        const uint64_t idx = ((uint64_t)c * (uint64_t)a.NB + (uint64_t)blk) * (uint64_t)a.rpad + (uint64_t)visit;
+        q = clampi(q_stoch(x / d, uniform_of(idx, a.seed, a.stream)), -qmax, qmax);
+      }
+      a.tmp[(blk * a.r + slot) * a.C + c] = (int8_t)q;
+    }
+  }
+}
+
+__global__ void big_clear_kernel(float* stat, float* colmax, int64_t C) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < 4) stat[i] = 0.f;
+  if (i < C) colmax[i] = 0.f;
+}
+
+// statistics -> steps (absmax modes are also read directly by the quantise pass)
+__global__ void __launch_bounds__(256) big_finalize_kernel(const BigArgs a, int64_t nwg, int64_t kout) {
+  __shared__ double s_q[256], s_b[256];
+  const float qmax = (float)((1 << (a.bits - 1)) - 1);
+  const int tid = threadIdx.x;
+  if (a.mode == HOT_SCALE_ROW) {
+    for (int64_t c = tid; c < a.C; c += 256) a.scales_out[c] = a.colmax[c] / qmax;
+    return;
+  }
+  if (a.mode == HOT_SCALE_TENSOR) {
+    if (tid == 0) a.scales_out[0] = a.stat[0] / qmax;
+    return;
+  }
+  double q = 0.0, b = 0.0;
+  for (int64_t i = tid; i < nwg; i += 256) { q += a.partial[2 * i]; b += a.partial[2 * i + 1]; }
+  s_q[tid] = q; s_b[tid] = b;
+  __syncthreads();
+  for (int s = 128; s > 0; s >>= 1) {
+    if (tid < s) { s_q[tid] += s_q[tid + s]; s_b[tid] += s_b[tid + s]; }
+    __syncthreads();
+  }
+  if (tid == 0) {
+    const double cnt = (double)kout * (double)a.C;
+    const float clip = (float)(12.1 * sqrt(s_q[0] / cnt) - 12.2 * (s_b[0] / cnt));
+    const float s = clip / qmax;
+    a.stat[1] = s;
+    a.stat[2] = clip;
+    a.scales_out[0] = s;
+  }
+}
+
+// tmp [K, C] -> out [C, ld] with the bytes [K, ld) of every row zeroed; 64 x 64 tiles through LDS
+__global__ void __launch_bounds__(256) transpose_i8_kernel(const int8_t* __restrict__ tmp, int64_t K, int64_t C,
+                                                           int8_t* __restrict__ out, int64_t ld) {
+  __shared__ int8_t tile[64][65];
+  const int64_t k0 = (int64_t)blockIdx.x * 64, c0 = (int64_t)blockIdx.y * 64;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int i = ty; i < 64; i += 4) {
+    const int64_t k = k0 + i, c = c0 + tx;
+    tile[i][tx] = (k < K && c < C) ? tmp[k * C + c] : (int8_t)0;
+  }
+  __syncthreads();
+  for (int i = ty; i < 64; i += 4) {
+    const int64_t c = c0 + i, k = k0 + tx;
+    if (c < C && k < ld) out[c * ld + k] = tile[tx][i];
+  }
+}
+
+template <int M>
+int launch_stage2(const BigArgs& a, dim3 grid, int pass, hipStream_t st) {
+  const bool sawb = a.mode == HOT_SCALE_SAWB, stoch = a.rounding == HOT_ROUND_STOCH;
+  if (pass == 0) {
+    if (sawb) hipLaunchKernelGGL((big_stage2_kernel<M, 0, 0, true>), grid, dim3(BT), 0, st, a);
+    else hipLaunchKernelGGL((big_stage2_kernel<M, 0, 0, false>), grid, dim3(BT), 0, st, a);
+  } else if (stoch) {
+    if (sawb) hipLaunchKernelGGL((big_stage2_kernel<M, 1, 1, true>), grid, dim3(BT), 0, st, a);
+    else hipLaunchKernelGGL((big_stage2_kernel<M, 1, 1, false>), grid, dim3(BT), 0, st, a);
+  } else {
+    if (sawb) hipLaunchKernelGGL((big_stage2_kernel<M, 1, 0, true>), grid, dim3(BT), 0, st, a);
+    else hipLaunchKernelGGL((big_stage2_kernel<M, 1, 0, false>), grid, dim3(BT), 0, st, a);
+  }
+  return check_launch("big_stage2_kernel");
+}
+
+int dispatch_stage2(int m, const BigArgs& a, dim3 grid, int pass, hipStream_t st) {
+  switch (m) {
+    case 2: return launch_stage2<2>(a, grid, pass, st);
+    case 4: return launch_stage2<4>(a, grid, pass, st);
+    case 8: return launch_stage2<8>(a, grid, pass, st);
+    case 16: return launch_stage2<16>(a, grid, pass, st);
+    case 32: return launch_stage2<32>(a, grid, pass, st);
+    case 64: return launch_stage2<64>(a, grid, pass, st);
+    case 128: return launch_stage2<128>(a, grid, pass, st);
+    default: return fail(HOT_ERR_UNSUPPORTED, "hla: block size %d (64 m with m a power of two up to 128)", 64 * m);
+  }
+}
+
+constexpr size_t STAT_BYTES = 256;
+
+struct BigLayout { size_t off_colmax, off_partial, off_tab, off_T, off_tmp, total; };
+
+BigLayout big_layout(int64_t R, int64_t C, int n, int r) {
+  BigLayout b;
+  size_t o = STAT_BYTES;
+  b.off_colmax = o;  o += (size_t)round_up(C * 4, 256);
+  b.off_partial = o; o += (size_t)(2 * sizeof(double)) * 65536;
+  b.off_tab = o;     o += (size_t)round_up((int64_t)n * 4, 256);
+  b.off_T = o;       o += (size_t)round_up(R * C * 4, 256);
+  b.off_tmp = o;     o += (size_t)round_up((R / n) * r * C, 256);
+  b.total = o;
+  return b;
+}
+
+}  // namespace
+
+size_t hla_big_workspace_bytes_impl(int64_t R, int64_t C, int n, int r) {
+  if (R <= 0 || C <= 0 || n <= 0 || r <= 0) return 0;
+  return big_layout(R, C, n, r).total;
+}
+
+int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r, int bits,
+                 int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_out,
+                 float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st, const char* who,
+                 hipEvent_t after_stats) {
+  const int m = n / 64;
+  if (n < 128 || n > 8192 || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (a power of two, 128 .. 8192)", who, n);
+  const int64_t NB = R / n, kout = NB * r;
+  if (ld_out < kout || (ld_out & 15)) return fail(HOT_ERR_INVALID, "%s: ld_out=%lld must be a multiple of 16 and >= %lld", who, (long long)ld_out, (long long)kout);
+  const BigLayout b = big_layout(R, C, n, r);
+  if (!workspace || workspace_bytes < b.total) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, b.total, workspace_bytes);
+  if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
+  const int64_t gx = (C + BT - 1) / BT;
+  if (NB * 64 > 65535 || R / 64 > 65535 || (scale_mode == HOT_SCALE_SAWB && gx * NB * 64 > 65536))
+    return fail(HOT_ERR_UNSUPPORTED, "%s: %lld blocks of %d tokens x %lld channels exceed the grid of the large-block path", who, (long long)NB, n, (long long)C);
+
+  // slot and visit number of every natural row of a block (visit = rank among the kept rows)
+  thread_local std::vector<int32_t> tab;
+  tab.assign((size_t)n, -1);
+  std::vector<int32_t> sorted(rows, rows + r);
+  for (int k = 0; k < r; ++k) {
+    if (rows[k] < 0 || rows[k] >= n) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d outside [0, %d)", who, k, rows[k], n);
+    if (tab[(size_t)rows[k]] != -1) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d listed twice", who, k, rows[k]);
+    tab[(size_t)rows[k]] = k;
+  }
+  std::sort(sorted.begin(), sorted.end());
+  for (int v = 0; v < r; ++v) tab[(size_t)sorted[(size_t)v]] |= v << 16;
+
+  uint8_t* ws = (uint8_t*)workspace;
+  BigArgs a;
+  a.in = in; a.T = (float*)(ws + b.off_T); a.tmp = (int8_t*)(ws + b.off_tmp); a.tab = (const int32_t*)(ws + b.off_tab);
+  a.R = R; a.C = C; a.NB = NB; a.n = n; a.r = r; a.rpad = (r + 7) & ~7; a.bits = bits; a.rounding = rounding;
+  a.mode = scale_mode; a.stat = (float*)ws; a.colmax = (float*)(ws + b.off_colmax);
+  a.partial = (double*)(ws + b.off_partial); a.scales_out = scales_out; a.seed = seed; a.stream = rng_stream;
+
+  // the table travels through a staged copy: the call returns once the host buffer has been read
+  if (int rc = check_hip(hipMemcpyAsync(ws + b.off_tab, tab.data(), (size_t)n * 4, hipMemcpyHostToDevice, st), "hipMemcpyAsync(row table)")) return rc;
+  const int64_t nclr = C > 4 ? C : 4;
+  hipLaunchKernelGGL(big_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat, a.colmax, C);
+  const dim3 g1((unsigned)gx, (unsigned)(R / 64));
+  switch (dtype) {
+    case HOT_F32: hipLaunchKernelGGL(big_stage1_kernel<float>, g1, dim3(BT), 0, st, a); break;
+    case HOT_BF16: hipLaunchKernelGGL(big_stage1_kernel<bf16_t>, g1, dim3(BT), 0, st, a); break;
+    case HOT_F16: hipLaunchKernelGGL(big_stage1_kernel<f16_t>, g1, dim3(BT), 0, st, a); break;
+    default: return fail(HOT_ERR_INVALID, "%s: bad dtype %d", who, dtype);
+  }
+  if (int rc = check_launch("big_stage1_kernel")) return rc;
+  const dim3 g2((unsigned)gx, (unsigned)(NB * 64));
+  if (int rc = dispatch_stage2(m, a, g2, 0, st)) return rc;
+  hipLaunchKernelGGL(big_finalize_kernel, dim3(1), dim3(256), 0, st, a, (int64_t)gx * NB * 64, kout);
+  if (after_stats) (void)hipEventRecord(after_stats, st);
+  if (int rc = dispatch_stage2(m, a, g2, 1, st)) return rc;
+  const dim3 gt((unsigned)((ld_out + 63) / 64), (unsigned)((C + 63) / 64));
+  hipLaunchKernelGGL(transpose_i8_kernel, gt, dim3(256), 0, st, a.tmp, kout, C, (int8_t*)codes_out, ld_out);
+  return check_launch("transpose_i8_kernel");
+}
+
+}  // namespace hot

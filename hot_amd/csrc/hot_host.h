@@ -35,6 +35,16 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
 size_t colwise_workspace_bytes_impl(int64_t C);
 size_t colwise_stats_bytes_impl(int64_t C);  // leading part of the workspace that must be zero before the statistics pass
 
+// Blocks of 128 .. 8192 tokens (two-level transform through an fp32 workspace); same contract as
+// colwise_quant_impl without the packed-INT4 store and the fused row statistic.
+int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r, int bits,
+                 int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_out,
+                 float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st, const char* who,
+                 hipEvent_t after_stats = nullptr);
+size_t hla_big_workspace_bytes_impl(int64_t R, int64_t C, int n, int r);
+// Workspace of a token-wise transform of [R, C] with blocks of n tokens and r kept rows, either path.
+size_t hla_workspace_bytes_impl(int64_t R, int64_t C, int n, int r);
+
 int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bits, int64_t M, int64_t N,
                  int64_t K, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
                  void* out, int out_dtype, int64_t ldo, int32_t* acc_out, hipStream_t st, void* split_ws = nullptr,

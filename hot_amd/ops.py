@@ -81,12 +81,17 @@ class HotOptions:
         return (L // self.hla_n) * self.hla_r
 
     def to_c(self) -> _lib.HotConfig:
-        if self.hla_n > _lib.HOT_MAX_HLA_N:
-            raise HotError("HLA block %d exceeds the native maximum %d" % (self.hla_n, _lib.HOT_MAX_HLA_N))
+        if self.hla_n > _lib.HOT_MAX_HLA_BIG:
+            raise HotError("HLA block %d exceeds the native maximum %d" % (self.hla_n, _lib.HOT_MAX_HLA_BIG))
         c = _lib.HotConfig()
         c.n_o, c.hla_n, c.hla_r = self.n_o, self.hla_n, self.hla_r
-        for i, v in enumerate(self.hla_rows):
-            c.hla_rows[i] = int(v)
+        if self.hla_n > _lib.HOT_MAX_HLA_N:
+            big = (C.c_int32 * self.hla_r)(*[int(v) for v in self.hla_rows])
+            c.hla_rows_big = C.cast(big, C.POINTER(C.c_int32))
+            c._rows_keepalive = big          # the struct only holds a pointer
+        else:
+            for i, v in enumerate(self.hla_rows):
+                c.hla_rows[i] = int(v)
         c.gx_bits, c.w_bits, c.gw_bits, c.act_bits = self.gx_bits, self.w_bits, self.gw_bits, self.act_bits
         c.gx_round, c.w_round, c.gw_round, c.act_round = (_ROUND[self.gx_round], _ROUND[self.w_round],
                                                           _ROUND[self.gw_round], _ROUND[self.act_round])
@@ -124,7 +129,7 @@ def hla_tokenwise(x: torch.Tensor, n: int, rows: Sequence[int], bits: int = 8, r
     mode = _SCALE[scale]
     codes = torch.empty((Cc, ld), dtype=torch.int8, device=x.device)
     scales = torch.empty((Cc if mode == SCALE_ROW else 1,), dtype=torch.float32, device=x.device)
-    ws = _ws(_lib.lib().hot_colwise_workspace_bytes(Cc), x.device)
+    ws = _ws(_lib.lib().hot_hla_workspace_bytes(R, Cc, n, r), x.device)
     rows_c = (C.c_int32 * r)(*[int(v) for v in rows])
     _lib.check(_lib.lib().hot_hla_tokenwise(x.data_ptr(), _dt(x), R, Cc, n, rows_c, r, bits, _ROUND[rounding], seed,
                                             rng_stream, mode, codes.data_ptr(), ld, scales.data_ptr(),

@@ -196,10 +196,17 @@ class HQ_Linear(nn.Linear):
         self.layer_name = " "
 
     def _refresh_bs(self, tokens: int) -> None:
-        if self._bs_tokens == tokens:
+        key = (tokens, args.hla_rule, args.hla_max_block, args.vectorPercentile)
+        if self._bs_tokens == key:
             return
         n, rows = token_rule(tokens)
-        # P = rows of H_n; small (at most 64 x 64) because of args.hla_max_block
+        self._bs_tokens = key
+        if n > 64:
+            # the kernels take the row list, not the matrix: a block of 8192 tokens would make P
+            # 2080 x 8192 per layer, so beyond 64 tokens the attribute is only a placeholder
+            self.hadamard_bs = torch.ones((1, 1), dtype=self.weight.dtype, device=self.weight.device)
+            return
+        # P = rows of H_n
         idx = torch.as_tensor(np.asarray(rows), dtype=torch.long)
         i = idx[:, None] & torch.arange(n)[None, :]
         par = torch.zeros_like(i)
@@ -207,7 +214,6 @@ class HQ_Linear(nn.Linear):
             par ^= i & 1
             i >>= 1
         self.hadamard_bs = (1 - 2 * par).to(self.weight.dtype).to(self.weight.device)
-        self._bs_tokens = tokens
 
     def forward(self, input: Tensor) -> Tensor:
         if input.dim() == 3 and args.batched_mode == "per_sample":

@@ -41,7 +41,7 @@
 extern "C" {
 #endif
 
-#define HOT_ABI_VERSION 1
+#define HOT_ABI_VERSION 2
 #define HOT_API __attribute__((visibility("default")))
 
 enum hot_status {
@@ -63,19 +63,26 @@ enum hot_scale_mode {
 /* Counter-based RNG stream identifiers (Philox counter word 2). */
 enum hot_rng_stream { HOT_STREAM_GX = 0, HOT_STREAM_GW = 1, HOT_STREAM_W = 2, HOT_STREAM_ACT = 3 };
 
-#define HOT_MAX_HLA_N 64
+#define HOT_MAX_HLA_N 64        /* largest block with its rows inline in hot_config     */
+#define HOT_MAX_HLA_BIG 8192    /* largest block at all (rows through hla_rows_big)     */
 
 /* Options of the fused path; mirrors the fields FLinearQ reads from the
  * reference's module-global `args` (args.py:29-49), scheme gih_gwlr. */
 typedef struct hot_config {
   int32_t n_o;      /* Hadamard block along O: a power of two, 1 .. 64            */
-  int32_t hla_n;    /* HLA block along tokens: 1, 2, 4, ..., HOT_MAX_HLA_N        */
+  int32_t hla_n;    /* HLA block along tokens: a power of two, 1 .. HOT_MAX_HLA_BIG */
   int32_t hla_r;    /* kept coefficients per block, 1..hla_n                      */
-  int32_t hla_rows[HOT_MAX_HLA_N]; /* natural-order row of output coefficient k  */
+  int32_t hla_rows[HOT_MAX_HLA_N]; /* natural-order row of output coefficient k
+                                      (blocks up to HOT_MAX_HLA_N)                */
   int32_t gx_bits, w_bits, gw_bits, act_bits;         /* 4 or 8                   */
   int32_t gx_round, w_round, gw_round, act_round;     /* hot_rounding             */
   int32_t gx_scale, w_scale, gw_scale, act_scale;     /* hot_scale_mode           */
   uint64_t seed;    /* stochastic-rounding key                                    */
+  const int32_t* hla_rows_big; /* host, hla_r entries: the rows of blocks above
+                                  HOT_MAX_HLA_N tokens (NULL otherwise); such blocks
+                                  take a two-level transform through an fp32
+                                  workspace and a staged host-to-device copy of
+                                  the row table, which cannot be graph-captured  */
 } hot_config;
 
 HOT_API const char* hot_last_error(void);
@@ -107,7 +114,7 @@ HOT_API int hot_hq_rowwise(const void* in, int dtype, int64_t M, int64_t K, int 
  *   codes_out   device, logical [C, (R/n)*r] codes; row pitch ld_out bytes;
  *               bytes beyond the logical row up to ld_out are written as zero
  *   scales_out  [1] (TENSOR, SAWB) or [C] (ROW)
- *   workspace   device, >= hot_colwise_workspace_bytes(C)
+ *   workspace   device, >= hot_hla_workspace_bytes(R, C, n, r)
  * Stochastic rounding numbers the kept coefficients of block b of channel c
  * in increasing natural-row order v = 0..r-1 and gives coefficient v the RNG
  * element index ((c * (R/n) + b) * rpad + v), rpad = r rounded up to 8.
@@ -126,6 +133,9 @@ HOT_API int hot_wq_colwise(const void* in, int dtype, int64_t O, int64_t I, int 
                    size_t workspace_bytes, void* hip_stream);
 
 HOT_API size_t hot_colwise_workspace_bytes(int64_t C);
+/* Workspace of hot_hla_tokenwise for any block size: hot_colwise_workspace_bytes(C)
+ * up to HOT_MAX_HLA_N tokens, plus an fp32 copy of the input above. */
+HOT_API size_t hot_hla_workspace_bytes(int64_t R, int64_t C, int n, int r);
 
 /*
  * out[M, N] = ((acc * scale_a[row or 0]) * scale_b[0]) * post_scale,

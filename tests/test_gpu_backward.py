@@ -222,6 +222,7 @@ def test_hq_linear_training_step(gpu, fresh_args):
     """HQ_Linear forward (full precision) + backward (HOT) through autograd."""
     from hot_amd.quant_matmul import HQ_Linear
     L, I, O = 256, 96, 128
+    fresh_args.hla_max_block = 64          # 256 tokens: blocks of 64 (one-pass kernels); the default is below
     torch.manual_seed(0)
     lin = HQ_Linear(I, O).to(gpu)
     x = torch.randn(L, I, device=gpu, requires_grad=True)
@@ -235,7 +236,19 @@ def test_hq_linear_training_step(gpu, fresh_args):
     assert np.array_equal(x.grad.cpu().numpy(), tr.g_x)
     assert np.array_equal(lin.weight.grad.cpu().numpy(), tr.g_w)
     assert torch.allclose(lin.bias.grad, gy.sum(0), rtol=1e-5, atol=1e-8)
-    assert lin.hadamard_bs.shape == (36, 128 if L % 128 == 0 and fresh_args.hla_max_block >= 128 else 64)
+    assert lin.hadamard_bs.shape == (36, 64)
+    # default: the reference's rule without a cap, 256 tokens -> one block of 256, 136 rows kept
+    fresh_args.hla_max_block = 8192
+    lin.zero_grad()
+    x2 = x.detach().clone().requires_grad_(True)
+    lin(x2).backward(gy)
+    ocfg = orc.HotConfig.python_rule(L)
+    assert (ocfg.hla_n, len(ocfg.hla_rows)) == (256, 136)
+    xq_ref, sx_ref = orc.abc_forward(x2.detach().cpu().numpy(), ocfg)
+    tr = orc.linear_backward(gy.cpu().numpy(), lin.weight.detach().cpu().numpy(), xq_ref, sx_ref, ocfg)
+    assert np.array_equal(x2.grad.cpu().numpy(), tr.g_x)
+    assert np.array_equal(lin.weight.grad.cpu().numpy(), tr.g_w)
+    assert lin.hadamard_bs.shape == (1, 1)          # placeholder beyond 64 tokens per block
 
 
 @pytest.mark.parametrize("mode", ["per_sample", "flatten"])
@@ -327,7 +340,9 @@ def test_lqs_then_hot_training_step(gpu, fresh_args):
     torch.nn.functional.cross_entropy(model(x), t).backward()
     for h, p in zip(hot, model.parameters()):
         cos = torch.nn.functional.cosine_similarity(h.flatten(), p.grad.flatten(), dim=0)
-        assert float(cos) > 0.7, float(cos)
+        # random tokens have no low-sequency structure: keeping about half the rows keeps about half the
+        # energy of g_W, a cosine near 0.7
+        assert float(cos) > 0.55, float(cos)
 
 
 def test_backward_errors(gpu):
@@ -419,7 +434,7 @@ def test_hq_linear_odd_feature_counts(gpu, fresh_args, O, I):
     4 for 100 classes, 2 for 10) and widths that are not multiples of 8 are zero-padded on the way in."""
     from hot_amd.quant_matmul import HQ_Linear
     from hot_amd.hadamard_matmul import biggest_power2_factor_max16
-    L = 128
+    L = 192
     torch.manual_seed(7)
     lin = HQ_Linear(I, O, bias=False).to(gpu)
     x = torch.randn(L, I, device=gpu, requires_grad=True)
@@ -452,3 +467,25 @@ def test_backward_matches_golden_fixture(gpu, name):
     assert np.array_equal(xq.cpu().numpy()[:, :lp], f["xq"].T) and np.array_equal(sx.cpu().numpy(), f["sx"])
     gx, gw = ops.linear_backward(gy, w, xq, sx, opt)
     assert np.array_equal(gx.cpu().numpy(), f["g_x"]) and np.array_equal(gw.cpu().numpy(), f["g_w"])
+
+
+@pytest.mark.parametrize("L,O,I,variant", [
+    (256, 64, 48, dict()),                                                      # n = 256, r = 136
+    (384, 32, 40, dict(gx_scale=orc.SCALE_ROW, gw_scale=orc.SCALE_ROW)),        # 384 = 128 * 3 -> n = 128
+    (2048, 48, 32, dict(gw_round=orc.ROUND_STOCH, gx_round=orc.ROUND_STOCH, seed=9)),
+    (8192, 32, 16, dict(w_scale=orc.SCALE_SAWB, act_scale=orc.SCALE_SAWB)),     # the Llama token count: n = 8192, r = 2080
+])
+def test_backward_exact_python_rule_on_large_blocks(gpu, L, O, I, variant):
+    """The make_WHT rule without a cap on the block: token counts with many factors of two."""
+    from hot_amd import ops
+    ocfg = orc.HotConfig.python_rule(L, **variant)
+    assert ocfg.hla_n == (L & -L) and ocfg.hla_n > 64
+    opt = ops.HotOptions(n_o=ocfg.n_o, hla_n=ocfg.hla_n, hla_rows=ocfg.hla_rows, gx_bits=ocfg.gx_bits,
+                         w_bits=ocfg.w_bits, gw_bits=ocfg.gw_bits, act_bits=ocfg.act_bits,
+                         gx_round=ocfg.gx_round, w_round=ocfg.w_round, gw_round=ocfg.gw_round,
+                         act_round=ocfg.act_round, gx_scale=ocfg.gx_scale, w_scale=ocfg.w_scale,
+                         gw_scale=ocfg.gw_scale, act_scale=ocfg.act_scale, seed=ocfg.seed)
+    x, w, gy = make_case(L, O, I, seed=L)
+    gx, gw, tr = run_both(x, w, gy, ocfg, opt, gpu)
+    assert np.array_equal(gx.cpu().numpy(), tr.g_x)
+    assert np.array_equal(gw.cpu().numpy(), tr.g_w)

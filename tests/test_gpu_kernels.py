@@ -342,3 +342,29 @@ def test_gemm_splits_rule():
     assert f(256, 256, 128, 8) == 1            # short K
     assert f(256, 256, 2304, 8) == 2
 
+
+
+@pytest.mark.parametrize("n,L,C,scale,rounding,dtype", [
+    (128, 256, 72, "tensor", "nearest", torch.float32),
+    (128, 512, 264, "row", "stoch", torch.bfloat16),
+    (256, 512, 64, "sawb", "nearest", torch.float32),
+    (1024, 2048, 40, "tensor", "stoch", torch.float32),
+    (8192, 8192, 16, "tensor", "nearest", torch.bfloat16),
+])
+def test_hla_tokenwise_large_blocks(gpu, n, L, C, scale, rounding, dtype):
+    """Blocks above 64 tokens (the make_WHT rule on token counts with many factors of two) take the
+    two-level path; codes, steps and the transposed layout must equal the one-pass oracle."""
+    from hot_amd import ops
+    nn_, rows = orc.hla_rows(n)
+    assert nn_ == n
+    x = (torch.randn(L, C, generator=torch.Generator().manual_seed(n + C)) * 0.5).to(dtype)
+    mode = {"tensor": orc.SCALE_TENSOR, "row": orc.SCALE_ROW, "sawb": orc.SCALE_SAWB}[scale]
+    rnd = orc.ROUND_STOCH if rounding == "stoch" else orc.ROUND_NEAREST
+    tt = np.ascontiguousarray(orc.fwht_blocks_first(x.float().numpy(), n, rows).T)      # [C, L']
+    q_ref, s_ref = orc.quant(tt, 8, mode, rnd, seed=3, stream=orc.STREAM_GW,
+                             index=orc.colwise_rng_index(C, L // n, rows))
+    codes, s, kout = ops.hla_tokenwise(x.to(gpu), n, list(rows), bits=8, rounding=rounding, scale=scale, seed=3)
+    got = codes.cpu().numpy()
+    assert kout == tt.shape[1]
+    assert np.array_equal(s.cpu().numpy(), np.atleast_1d(s_ref).astype(np.float32).reshape(-1))
+    assert np.array_equal(got[:, :kout], q_ref) and not got[:, kout:].any()
