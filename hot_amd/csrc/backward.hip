@@ -279,7 +279,7 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   // operand).  With one step per tensor both quantisers need the absmax of their transform first:
   // the statistics pass of the token-wise kernel delivers both from a single read of g_y.
   const bool fuse = cfg->gx_scale == HOT_SCALE_TENSOR && cfg->n_o == 16 && O % 16 == 0 && cfg->gw_scale != HOT_SCALE_SAWB &&
-                    cfg->hla_n <= HOT_MAX_HLA_N;
+                    cfg->hla_n <= COL_MAX_N;
   // Side stream, beside the g_W GEMM on the main stream: always the row-wise quantise pass of g_y (a
   // streaming kernel next to a matrix kernel); the g_x GEMM too when the g_W GEMM has fewer tiles
   // than the chip has CUs and cannot fill it alone (two large GEMMs only get in each other's way).

@@ -47,7 +47,7 @@ struct ColArgs {
   uint32_t stream;
   int32_t r, rpad, bits, store4, rounding, mode, tb, stats_cleared;
   hipEvent_t after_stats;  // host only: recorded between the statistics and the quantise pass
-  int8_t slot[HOT_MAX_HLA_N];  // output position of natural row i, -1 = dropped
+  int8_t slot[COL_MAX_N];  // output position of natural row i, -1 = dropped
 };
 
 // Which coefficients of a block are kept and where they go.  The generic policy reads the table
@@ -65,6 +65,10 @@ struct SelPy64 {  // make_WHT rule for n = 64: 36 coefficients, sequency order
                                        18, -1, 4,  -1, 21, -1, 10, -1, 19, -1, 1,  -1, 24, 27, 13, 34, 16, 31, 6,  -1, -1, -1,
                                        8,  -1, -1, -1, 2,  -1, 23, 28, 12, -1, 17, 30, 5,  -1, -1, -1, 9,  -1, 20, -1};
   static constexpr int slot(int i) { return TABLE[i]; }
+};
+struct SelPy128 {  // make_WHT rule for n = 128: the n = 64 selection on the even rows, no odd row
+  static constexpr bool STATIC = true;
+  static constexpr int slot(int i) { return (i & 1) ? -1 : SelPy64::TABLE[i >> 1]; }
 };
 struct SelPaper16 {  // the 8 lowest sequencies of a 16-block
   static constexpr bool STATIC = true;
@@ -442,7 +446,7 @@ static constexpr size_t COL_STAT_BYTES = 256;
 size_t colwise_stats_bytes_impl(int64_t C) { return COL_STAT_BYTES + (size_t)round_up(C * 4, 256); }
 
 size_t hla_workspace_bytes_impl(int64_t R, int64_t C, int n, int r) {
-  return n > HOT_MAX_HLA_N ? hla_big_workspace_bytes_impl(R, C, n, r) : colwise_workspace_bytes_impl(C);
+  return n > COL_MAX_N ? hla_big_workspace_bytes_impl(R, C, n, r) : colwise_workspace_bytes_impl(C);
 }
 
 size_t colwise_workspace_bytes_impl(int64_t C) {
@@ -529,7 +533,10 @@ static int dispatch_colwise_n(int n, ColArgs& a, hipStream_t st) {
       if (a.r == 36 && matches<SelPy64, 64>(a)) return launch_colwise<T, 64, SelPy64>(a, st);
       if (a.r == 64 && matches<SelFull<64>, 64>(a)) return launch_colwise<T, 64, SelFull<64>>(a, st);
       return launch_colwise<T, 64, SelRuntime>(a, st);
-    default: return fail(HOT_ERR_UNSUPPORTED, "colwise: block size %d (power of two up to %d)", n, HOT_MAX_HLA_N);
+    case 128:
+      if (a.r == 36 && matches<SelPy128, 128>(a)) return launch_colwise<T, 128, SelPy128>(a, st);
+      return launch_colwise<T, 128, SelRuntime>(a, st);
+    default: return fail(HOT_ERR_UNSUPPORTED, "colwise: block size %d (power of two up to %d)", n, COL_MAX_N);
   }
 }
 
@@ -540,9 +547,9 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
                        bool stats_cleared, hipEvent_t after_stats) {
   if (!in || !codes_out || !scales_out || !rows) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
   if (R <= 0 || C <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape R=%lld C=%lld", who, (long long)R, (long long)C);
-  if (n > HOT_MAX_HLA_N) {
+  if (n > COL_MAX_N) {
     // blocks one thread cannot hold: the two-level path
-    if (store4 || row16_absmax_out) return fail(HOT_ERR_UNSUPPORTED, "%s: blocks above %d tokens have no packed-INT4 store and no fused row statistic", who, HOT_MAX_HLA_N);
+    if (store4 || row16_absmax_out) return fail(HOT_ERR_UNSUPPORTED, "%s: blocks above %d tokens have no packed-INT4 store and no fused row statistic", who, COL_MAX_N);
     if (R % n) return fail(HOT_ERR_INVALID, "%s: R=%lld is not a multiple of the block %d", who, (long long)R, n);
     if (r < 1 || r > n) return fail(HOT_ERR_INVALID, "%s: r=%d outside [1, %d]", who, r, n);
     if (bits != 4 && bits != 8) return fail(HOT_ERR_UNSUPPORTED, "%s: bits=%d (4 or 8)", who, bits);
@@ -551,7 +558,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
     return hla_big_impl(in, dtype, R, C, n, rows, r, bits, rounding, seed, rng_stream, scale_mode, codes_out, ld_out,
                         scales_out, workspace, workspace_bytes, st, who, after_stats);
   }
-  if (n < 1 || n > HOT_MAX_HLA_N || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (power of two up to %d)", who, n, HOT_MAX_HLA_N);
+  if (n < 1 || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (a power of two)", who, n);
   if (R % n) return fail(HOT_ERR_INVALID, "%s: R=%lld is not a multiple of the block %d", who, (long long)R, n);
   if (r < 1 || r > n) return fail(HOT_ERR_INVALID, "%s: r=%d outside [1, %d]", who, r, n);
   if (bits != 4 && bits != 8) return fail(HOT_ERR_UNSUPPORTED, "%s: bits=%d (4 or 8)", who, bits);
@@ -566,7 +573,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   a.out = (int8_t*)codes_out; a.ld_out = ld_out;
   a.seed = seed; a.stream = rng_stream;
   a.r = r; a.rpad = (r + 7) & ~7; a.bits = bits; a.rounding = rounding; a.mode = scale_mode; a.tb = 4;
-  for (int i = 0; i < HOT_MAX_HLA_N; ++i) a.slot[i] = -1;
+  for (int i = 0; i < COL_MAX_N; ++i) a.slot[i] = -1;
   for (int k = 0; k < r; ++k) {
     if (rows[k] < 0 || rows[k] >= n) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d outside [0, %d)", who, k, rows[k], n);
     if (a.slot[rows[k]] != -1) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d listed twice", who, k, rows[k]);

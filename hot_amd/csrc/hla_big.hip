@@ -1,6 +1,7 @@
 // Hadamard low-rank projection along tokens for blocks larger than one thread can hold:
-// n = 64 m tokens, m = 2 .. 128 (the reference's make_WHT rule asks for the largest power of two
-// dividing the token count: 128 for 25216 tokens, 8192 for 8192; utils/hadamard_matmul.py:209-226).
+// n = 64 m tokens, m = 4 .. 128 (the reference's make_WHT rule asks for the largest power of two
+// dividing the token count, e.g. 8192 for 8192 tokens; utils/hadamard_matmul.py:209-226).  Blocks of
+// up to 128 tokens are served by the register kernel (colwise.hip).
 //
 // A Sylvester transform of n = 64 m points is the 64-point transform inside each run of 64 rows
 // followed by the m-point transform across the runs, and the canonical butterfly order
@@ -240,14 +241,13 @@ int launch_stage2(const BigArgs& a, dim3 grid, int pass, hipStream_t st) {
 
 int dispatch_stage2(int m, const BigArgs& a, dim3 grid, int pass, hipStream_t st) {
   switch (m) {
-    case 2: return launch_stage2<2>(a, grid, pass, st);
     case 4: return launch_stage2<4>(a, grid, pass, st);
     case 8: return launch_stage2<8>(a, grid, pass, st);
     case 16: return launch_stage2<16>(a, grid, pass, st);
     case 32: return launch_stage2<32>(a, grid, pass, st);
     case 64: return launch_stage2<64>(a, grid, pass, st);
     case 128: return launch_stage2<128>(a, grid, pass, st);
-    default: return fail(HOT_ERR_UNSUPPORTED, "hla: block size %d (64 m with m a power of two up to 128)", 64 * m);
+    default: return fail(HOT_ERR_UNSUPPORTED, "hla: block size %d (64 m with m a power of two, 4 .. 128)", 64 * m);
   }
 }
 
@@ -279,7 +279,7 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
                  float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st, const char* who,
                  hipEvent_t after_stats) {
   const int m = n / 64;
-  if (n < 128 || n > 8192 || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (a power of two, 128 .. 8192)", who, n);
+  if (n < 256 || n > 8192 || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (a power of two, 256 .. 8192)", who, n);
   const int64_t NB = R / n, kout = NB * r;
   if (ld_out < kout || (ld_out & 15)) return fail(HOT_ERR_INVALID, "%s: ld_out=%lld must be a multiple of 16 and >= %lld", who, (long long)ld_out, (long long)kout);
   const BigLayout b = big_layout(R, C, n, r);

@@ -21,6 +21,7 @@ int check_hip(hipError_t e, const char* what);
 inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 
 constexpr int64_t GEMM_KTILE = 128;  // codes per K-tile of the int8 GEMM
+constexpr int COL_MAX_N = 128;       // largest token block one thread transforms in registers
 
 int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, int rounding,
                     uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_codes,
@@ -35,7 +36,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
 size_t colwise_workspace_bytes_impl(int64_t C);
 size_t colwise_stats_bytes_impl(int64_t C);  // leading part of the workspace that must be zero before the statistics pass
 
-// Blocks of 128 .. 8192 tokens (two-level transform through an fp32 workspace); same contract as
+// Blocks of 256 .. 8192 tokens (two-level transform through an fp32 workspace); same contract as
 // colwise_quant_impl without the packed-INT4 store and the fused row statistic.
 int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r, int bits,
                  int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_out,

@@ -79,10 +79,12 @@ typedef struct hot_config {
   int32_t gx_scale, w_scale, gw_scale, act_scale;     /* hot_scale_mode           */
   uint64_t seed;    /* stochastic-rounding key                                    */
   const int32_t* hla_rows_big; /* host, hla_r entries: the rows of blocks above
-                                  HOT_MAX_HLA_N tokens (NULL otherwise); such blocks
-                                  take a two-level transform through an fp32
-                                  workspace and a staged host-to-device copy of
-                                  the row table, which cannot be graph-captured  */
+                                  HOT_MAX_HLA_N tokens (NULL otherwise).  Blocks of
+                                  128 tokens run in the same kernels as smaller
+                                  ones; from 256 on they take a two-level
+                                  transform through an fp32 workspace and a staged
+                                  host-to-device copy of the row table, which
+                                  cannot be graph-captured                       */
 } hot_config;
 
 HOT_API const char* hot_last_error(void);
@@ -134,7 +136,7 @@ HOT_API int hot_wq_colwise(const void* in, int dtype, int64_t O, int64_t I, int 
 
 HOT_API size_t hot_colwise_workspace_bytes(int64_t C);
 /* Workspace of hot_hla_tokenwise for any block size: hot_colwise_workspace_bytes(C)
- * up to HOT_MAX_HLA_N tokens, plus an fp32 copy of the input above. */
+ * up to 128 tokens, plus an fp32 copy of the input above. */
 HOT_API size_t hot_hla_workspace_bytes(int64_t R, int64_t C, int n, int r);
 
 /*

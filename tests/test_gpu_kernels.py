@@ -352,8 +352,9 @@ def test_gemm_splits_rule():
     (8192, 8192, 16, "tensor", "nearest", torch.bfloat16),
 ])
 def test_hla_tokenwise_large_blocks(gpu, n, L, C, scale, rounding, dtype):
-    """Blocks above 64 tokens (the make_WHT rule on token counts with many factors of two) take the
-    two-level path; codes, steps and the transposed layout must equal the one-pass oracle."""
+    """Blocks above 64 tokens (the make_WHT rule on token counts with many factors of two): 128 in
+    registers, larger ones through the two-level path; codes, steps and the transposed layout must
+    equal the one-pass oracle."""
     from hot_amd import ops
     nn_, rows = orc.hla_rows(n)
     assert nn_ == n
@@ -367,4 +368,23 @@ def test_hla_tokenwise_large_blocks(gpu, n, L, C, scale, rounding, dtype):
     got = codes.cpu().numpy()
     assert kout == tt.shape[1]
     assert np.array_equal(s.cpu().numpy(), np.atleast_1d(s_ref).astype(np.float32).reshape(-1))
+    assert np.array_equal(got[:, :kout], q_ref) and not got[:, kout:].any()
+
+
+@pytest.mark.parametrize("bits,rounding,dtype", [(8, "stoch", torch.bfloat16), (4, "nearest", torch.float32)])
+def test_hla_tokenwise_block128_any_selection(gpu, bits, rounding, dtype):
+    """A 128-token block with a selection that is not the make_WHT one (table read at run time),
+    8-bit and 4-bit codes."""
+    from hot_amd import ops
+    n, L, C = 128, 384, 136
+    rows = np.random.default_rng(5).permutation(n)[:50]
+    x = (torch.randn(L, C, generator=torch.Generator().manual_seed(9)) * 0.5).to(dtype)
+    rnd = orc.ROUND_STOCH if rounding == "stoch" else orc.ROUND_NEAREST
+    tt = np.ascontiguousarray(orc.fwht_blocks_first(x.float().numpy(), n, rows).T)
+    q_ref, s_ref = orc.quant(tt, bits, orc.SCALE_TENSOR, rnd, seed=3, stream=orc.STREAM_GW,
+                             index=orc.colwise_rng_index(C, L // n, rows))
+    codes, s, kout = ops.hla_tokenwise(x.to(gpu), n, [int(v) for v in rows], bits=bits, rounding=rounding,
+                                       scale="tensor", seed=3)
+    got = codes.cpu().numpy()
+    assert s.cpu().numpy()[0] == np.float32(s_ref)
     assert np.array_equal(got[:, :kout], q_ref) and not got[:, kout:].any()
