@@ -372,10 +372,15 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     const int ndw = (int)((seg_end - seg0) / 4);            // output dwords per channel
     const int sdw = out_sb / 4;                             // of which staged
     const int nch = (int)((a.C - cg0) < CW ? (a.C - cg0) : CW);
-    // consecutive threads walk along K within a channel, then on to the next channel
+    // consecutive threads walk along K within a channel, then on to the next channel; (ch, jd) of
+    // position p = tid + k CW advance by a fixed step, so the loop carries them instead of dividing
     const int total = nch * ndw;
-    for (int p = tid; p < total; p += CW) {
-      const int ch = p / ndw, jd = p - ch * ndw;
+    const int step_ch = CW / ndw, step_jd = CW - step_ch * ndw;
+    int ch = tid / ndw, jd = tid - ch * ndw;
+    int8_t* dst = a.out + (cg0 + ch) * a.ld_out + seg0 + (int64_t)jd * 4;
+    const int64_t step_dst = step_ch * a.ld_out + (int64_t)step_jd * 4, wrap_dst = a.ld_out - (int64_t)ndw * 4;
+    for (int p = tid; p < total; p += CW, ch += step_ch, jd += step_jd, dst += step_dst) {
+      if (jd >= ndw) { jd -= ndw; ++ch; dst += wrap_dst; }
       const uint32_t* row = reinterpret_cast<const uint32_t*>(stage + ch * pitch);
       uint32_t w = 0u;
       if (jd < sdw) {
@@ -389,7 +394,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
           w = row[jd];
         }
       }
-      *reinterpret_cast<uint32_t*>(a.out + (cg0 + ch) * a.ld_out + seg0 + (int64_t)jd * 4) = w;
+      *reinterpret_cast<uint32_t*>(dst) = w;
     }
   }
 }
