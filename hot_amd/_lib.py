@@ -12,6 +12,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libhot_gfx950.so")
 
 HOT_MAX_HLA_N = 64        # rows inline in the config
+HOT_HQ_WORKSPACE_BYTES = 2048
 HOT_MAX_HLA_BIG = 8192    # rows through hla_rows_big
 
 # enums of include/hot_gfx950.h

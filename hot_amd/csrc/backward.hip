@@ -61,7 +61,7 @@ static BwdLayout bwd_layout(int64_t L, int64_t O, int64_t I, const hot_config* c
   b.ld_w = round_up(O, GEMM_KTILE) * c->w_bits / 8;
   b.ld_gp = round_up(lp, GEMM_KTILE);
   size_t o = 0;
-  b.off_hq = o;   o += 256;
+  b.off_hq = o;   o += STAT_SLOT_BYTES;
   b.off_colw = o; o += align256(colwise_workspace_bytes_impl(I));
   b.off_colg = o; o += align256(hla_workspace_bytes_impl(L, O, c->hla_n, c->hla_r));
   b.off_sg = o;   o += align256((size_t)L * 4);
@@ -246,7 +246,7 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   if (ev) (void)hipEventRecord(ev[0], st);
   // one launch zeroes every statistic of the call (absmax slots, per-channel maxima)
   {
-    const int n0 = 64, n1 = (int)(colwise_stats_bytes_impl(I) / 4), n2 = (int)(colwise_stats_bytes_impl(O) / 4);
+    const int n0 = (int)(STAT_SLOT_BYTES / 4), n1 = (int)(colwise_stats_bytes_impl(I) / 4), n2 = (int)(colwise_stats_bytes_impl(O) / 4);
     const int total = n0 + n1 + n2;
     hipLaunchKernelGGL(clear3_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
                        (uint32_t*)(ws + b.off_hq), n0, (uint32_t*)(ws + b.off_colw), n1, (uint32_t*)(ws + b.off_colg), n2);
@@ -295,7 +295,7 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   // g_x operand of g_y on the side stream: a streaming kernel beside the g_W GEMM
   auto quantise_gy_rows = [&](hipStream_t s2) {
     return hq_rowwise_impl(gy, dtype, L, O, cfg->n_o, cfg->gx_bits, cfg->gx_round, cfg->seed, HOT_STREAM_GX,
-                           cfg->gx_scale, ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, 256, s2, fuse);
+                           cfg->gx_scale, ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, STAT_SLOT_BYTES, s2, fuse);
   };
   auto gemm_gx = [&](hipStream_t s2) {
     // g_x = (qG . qW^T) sG sW / n_o   (never split here: the split workspace belongs to the g_W GEMM)

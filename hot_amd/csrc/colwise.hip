@@ -29,6 +29,7 @@
 namespace hot {
 
 constexpr int CW = 256;        // threads per workgroup = channels per workgroup
+constexpr size_t COL_STAT_BYTES = 256 + STAT_SLOT_BYTES;   // step / clip words, then the absmax slots
 constexpr int CW_ROWS = 16;    // rows staged per step
 
 struct ColArgs {
@@ -38,11 +39,12 @@ struct ColArgs {
   int64_t Kout;       // NB * r codes per output row
   int8_t* out;
   int64_t ld_out;     // bytes
-  float* stat;        // [0] absmax, [1] step s, [2] clip
+  float* stat;        // [1] step s, [2] clip (SAWB)
+  float* slots;       // TENSOR: absmax in STAT_SLOTS partial maxima
   double* partial;    // SAWB: 2 doubles per workgroup
   float* colmax;      // ROW: per-channel absmax
   float* scales_out;
-  float* row_absmax;  // statistics pass with RS != 0: absmax of the row-wise block Hadamard
+  float* row_absmax;  // statistics pass with RS != 0: absmax of the row-wise block Hadamard (STAT_SLOTS partial maxima)
   uint64_t seed;
   uint32_t stream;
   int32_t r, rpad, bits, store4, rounding, mode, tb, stats_cleared;
@@ -84,11 +86,12 @@ template <> __device__ __forceinline__ float cvt_raw<float>(uint32_t v) { return
 template <> __device__ __forceinline__ float cvt_raw<bf16_t>(uint16_t v) { return as_f((uint32_t)v << 16); }
 template <> __device__ __forceinline__ float cvt_raw<f16_t>(uint16_t v) { return (float)__builtin_bit_cast(_Float16, v); }
 
-// Unnormalised FWHT of the N-point groups of v[0..LEN), stages h = 1, 2, 4, ...
-template <int N, int LEN>
+// Unnormalised FWHT of the N-point groups of v[0..LEN), stages h = H0, 2 H0, 4 H0, ... (H0 = 2: the
+// caller has run the first stage already)
+template <int N, int LEN, int H0 = 1>
 __device__ __forceinline__ void fwht_regs(float (&v)[LEN]) {
 #pragma unroll
-  for (int h = 1; h < N; h <<= 1) {
+  for (int h = H0; h < N; h <<= 1) {
 #pragma unroll
     for (int i = 0; i < LEN; ++i) {
       if ((i & h) == 0) {
@@ -184,7 +187,12 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int64_t cg0 = (int64_t)blockIdx.x * CW;
-  const int64_t c = cg0 + tid;
+  // Fused row statistic: within each group of 16 lanes the channels are dealt out so that the four
+  // stages of the 16-point row transform pair lanes at the distances a single DPP operand reaches
+  // (channel bit 0 <-> lane xor 1, bit 1 <-> xor 2, bit 2 <-> xor 15, bit 3 <-> xor 8).
+  constexpr bool RSP = PASS == 0 && RS == 16;
+  const int chan = RSP ? (tid ^ ((tid & 4) ? 0xB : 0)) : tid;   // channel of this thread within the workgroup
+  const int64_t c = cg0 + chan;
   const bool active = c < a.C;
   const int64_t blk0 = (int64_t)blockIdx.y * a.tb;
   int nblk = (int)((a.NB - blk0) < a.tb ? (a.NB - blk0) : a.tb);
@@ -219,7 +227,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       d = active ? sc + 1e-11f : 1.f;
       if (active && blockIdx.y == 0) a.scales_out[c] = sc;
     } else if (a.mode == HOT_SCALE_TENSOR) {
-      const float sc = a.stat[0] / (float)qmax;
+      const float sc = stat_slots_max(a.slots, lane) / (float)qmax;
       d = sc + 1e-11f;
       if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) a.scales_out[0] = sc;
     } else {
@@ -235,7 +243,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
 
   // Transforms and consumes the token blocks held in x; `bl` is the group-local index of the first.
   auto consume = [&](int bl) {
-    fwht_regs<N, XL>(x);
+    fwht_regs<N, XL, (RSP && N >= 2) ? 2 : 1>(x);   // the fused statistics pass runs stage h = 1 while loading
 #pragma unroll
     for (int g = 0; g < BPS; ++g) {
       const int blk = bl + g;
@@ -285,6 +293,9 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   for (int s = 0; s < CW_DEPTH - 1; ++s)
     if (s < nsteps) rs_issue<T>(rs, lds0 + s * BUF, s, lane);
   // one step: wait for its rows, let the ring advance, pull this thread's 16 values into x[xo..]
+  // -1 on the lane that holds the upper channel of a pair, per channel bit
+  const float sg1 = (chan & 1) ? -1.f : 1.f, sg2 = (chan & 2) ? -1.f : 1.f;
+  const float sg4 = (chan & 4) ? -1.f : 1.f, sg8 = (chan & 8) ? -1.f : 1.f;
   auto step = [&](int s, float* dst) {
     // this wave's rows of step s have landed, and its LDS reads of step s-1 are complete: the
     // slice that held step s-1 may be refilled.  Steps s+1 .. s+CW_DEPTH-2 may still be in flight.
@@ -292,6 +303,42 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     else if (CW_DEPTH >= 3 && s + 1 < nsteps) wait_stream<LPW>();
     else wait_stream<0>();
     if (s + CW_DEPTH - 1 < nsteps) rs_issue<T>(rs, lds0 + ((s + CW_DEPTH - 1) % CW_DEPTH) * BUF, s + CW_DEPTH - 1, lane);
+    if constexpr (RSP) {
+      // Row-wise 16-point transform across lanes, magnitudes only.  A stage computes
+      // own + s * partner with s = +1 on the lane of the lower channel of a pair (own + partner) and
+      // -1 on the other (own - partner = -(partner - own)): a lane's value may come out negated,
+      // but paired lanes agree in all lower channel bits and so carry the same sign, every value
+      // stays +-(the true coefficient), and the product with +-1 is exact: the magnitudes are those
+      // of the add/sub butterflies.  One v_fmac with a DPP operand per stage; the stages run
+      // row-major over the 16 rows, so no DPP read follows the write of its register within two
+      // instructions.  The raw rows are consumed here, so the first token-wise stage (rows 2j and
+      // 2j+1, always within a step) is taken from them first.
+      float t[CW_ROWS];
+      rs_column<T>(my + (s % CW_DEPTH) * BUF, chan & 63, t);
+      if constexpr (N >= 2) {
+#pragma unroll
+        for (int j = 0; j < CW_ROWS; j += 2) { dst[j] = t[j] + t[j + 1]; dst[j + 1] = t[j] - t[j + 1]; }
+      } else {
+#pragma unroll
+        for (int j = 0; j < CW_ROWS; ++j) dst[j] = t[j];
+      }
+      asm volatile("s_nop 1");
+#pragma unroll
+      for (int i = 0; i < CW_ROWS; ++i)
+        asm volatile("v_fmac_f32_dpp %0, %0, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf" : "+v"(t[i]) : "v"(sg1));
+#pragma unroll
+      for (int i = 0; i < CW_ROWS; ++i)
+        asm volatile("v_fmac_f32_dpp %0, %0, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf" : "+v"(t[i]) : "v"(sg2));
+#pragma unroll
+      for (int i = 0; i < CW_ROWS; ++i)
+        asm volatile("v_fmac_f32_dpp %0, %0, %1 row_mirror row_mask:0xf bank_mask:0xf" : "+v"(t[i]) : "v"(sg4));
+#pragma unroll
+      for (int i = 0; i < CW_ROWS; ++i)
+        asm volatile("v_fmac_f32_dpp %0, %0, %1 row_ror:8 row_mask:0xf bank_mask:0xf" : "+v"(t[i]) : "v"(sg8));
+#pragma unroll
+      for (int i = 0; i < CW_ROWS; ++i) rmax = fmaxf(rmax, fabsf(t[i]));
+      return;
+    }
     rs_column<T>(my + (s % CW_DEPTH) * BUF, lane, dst);
     if constexpr (PASS == 0 && RS != 0) {
 #pragma unroll
@@ -331,7 +378,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       if (tid == 0) {
         float mm = s_max[0];
         for (int i = 1; i < CW / 64; ++i) mm = fmaxf(mm, s_max[i]);
-        atomic_max_nonneg(a.row_absmax, mm);
+        stat_slot_update(a.row_absmax, blockIdx.y * gridDim.x + blockIdx.x, mm);
       }
       __syncthreads();
     }
@@ -346,7 +393,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       if (tid == 0) {
         float mm = s_max[0];
         for (int i = 1; i < CW / 64; ++i) mm = fmaxf(mm, s_max[i]);
-        atomic_max_nonneg(a.stat, mm);
+        stat_slot_update(a.slots, blockIdx.y * gridDim.x + blockIdx.x, mm);
       }
       return;
     }
@@ -410,8 +457,8 @@ __global__ void __launch_bounds__(256) colwise_finalize_kernel(const ColArgs a, 
     return;
   }
   if (a.mode == HOT_SCALE_TENSOR) {
+    const float mx = stat_slots_max(a.slots, tid & 63);
     if (tid == 0) {
-      const float mx = a.stat[0];
       const float s = mx / qmax;
       a.stat[1] = s;
       a.stat[2] = mx;
@@ -437,16 +484,16 @@ __global__ void __launch_bounds__(256) colwise_finalize_kernel(const ColArgs a, 
   }
 }
 
+// stat | slots are adjacent (COL_STAT_BYTES); row_absmax is another slot array
 __global__ void colwise_clear_kernel(float* stat, float* colmax, int64_t C, float* row_absmax) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < 4) stat[i] = 0.f;
-  if (i == 0 && row_absmax) *row_absmax = 0.f;
+  if (i < (int64_t)(COL_STAT_BYTES / 4)) stat[i] = 0.f;
+  if (row_absmax && i < (int64_t)(STAT_SLOT_BYTES / 4)) row_absmax[i] = 0.f;
   if (colmax && i < C) colmax[i] = 0.f;
 }
 
 // ---- host ---------------------------------------------------------------------
 
-static constexpr size_t COL_STAT_BYTES = 256;
 
 size_t colwise_stats_bytes_impl(int64_t C) { return COL_STAT_BYTES + (size_t)round_up(C * 4, 256); }
 
@@ -491,7 +538,7 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   if (gy > 65535 || gx * gy > 65536) return fail(HOT_ERR_UNSUPPORTED, "colwise: grid %lld x %lld too large", (long long)gx, (long long)gy);
   const dim3 grid((unsigned)gx, (unsigned)gy);
   if (!a.stats_cleared) {
-    const int64_t nclr = a.C > 4 ? a.C : 4;
+    const int64_t nclr = a.C > (int64_t)(COL_STAT_BYTES / 4) ? a.C : (int64_t)(COL_STAT_BYTES / 4);
     hipLaunchKernelGGL(colwise_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat,
                        a.mode == HOT_SCALE_ROW ? a.colmax : (float*)nullptr, a.C, a.row_absmax);
   }
@@ -594,6 +641,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   a.after_stats = after_stats;
   uint8_t* ws = (uint8_t*)workspace;
   a.stat = (float*)ws;
+  a.slots = (float*)(ws + 256);
   a.colmax = (float*)(ws + COL_STAT_BYTES);
   a.partial = (double*)(ws + COL_STAT_BYTES + round_up(C * 4, 256));
   a.scales_out = scales_out;

@@ -26,6 +26,7 @@ namespace hot {
 namespace {
 
 constexpr int BT = 256;  // threads per workgroup = channels per workgroup
+constexpr size_t STAT_BYTES = 256 + STAT_SLOT_BYTES;   // [0] absmax, [1] step, [2] clip; then the absmax slots
 
 struct BigArgs {
   const void* in;
@@ -34,7 +35,7 @@ struct BigArgs {
   const int32_t* tab;  // per natural row of a block: slot | visit << 16, or -1 when dropped
   int64_t R, C, NB;    // NB = R / n blocks
   int32_t n, r, rpad, bits, rounding, mode;
-  float* stat;         // [0] absmax, [1] step, [2] clip
+  float* stat;         // [0] absmax, [1] step, [2] clip; the absmax slots from word 64
   float* colmax;       // per-channel absmax (ROW)
   double* partial;     // SAWB: 2 doubles per workgroup
   float* scales_out;
@@ -129,7 +130,7 @@ __global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
       if (tid == 0) {
         float mm = s_max[0];
         for (int i = 1; i < BT / 64; ++i) mm = fmaxf(mm, s_max[i]);
-        atomic_max_nonneg(a.stat, mm);
+        stat_slot_update(a.stat + 64, blockIdx.y * gridDim.x + blockIdx.x, mm);
       }
       return;
     }
@@ -171,7 +172,7 @@ __global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
 
 __global__ void big_clear_kernel(float* stat, float* colmax, int64_t C) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i < 4) stat[i] = 0.f;
+  if (i < (int64_t)(STAT_BYTES / 4)) stat[i] = 0.f;
   if (i < C) colmax[i] = 0.f;
 }
 
@@ -185,7 +186,8 @@ __global__ void __launch_bounds__(256) big_finalize_kernel(const BigArgs a, int6
     return;
   }
   if (a.mode == HOT_SCALE_TENSOR) {
-    if (tid == 0) a.scales_out[0] = a.stat[0] / qmax;
+    const float mx = stat_slots_max(a.stat + 64, tid & 63);
+    if (tid == 0) { a.stat[0] = mx; a.scales_out[0] = mx / qmax; }
     return;
   }
   double q = 0.0, b = 0.0;
@@ -251,7 +253,6 @@ int dispatch_stage2(int m, const BigArgs& a, dim3 grid, int pass, hipStream_t st
   }
 }
 
-constexpr size_t STAT_BYTES = 256;
 
 struct BigLayout { size_t off_colmax, off_partial, off_tab, off_T, off_tmp, total; };
 
@@ -310,7 +311,7 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
 
   // the table travels through a staged copy: the call returns once the host buffer has been read
   if (int rc = check_hip(hipMemcpyAsync(ws + b.off_tab, tab.data(), (size_t)n * 4, hipMemcpyHostToDevice, st), "hipMemcpyAsync(row table)")) return rc;
-  const int64_t nclr = C > 4 ? C : 4;
+  const int64_t nclr = C > (int64_t)(STAT_BYTES / 4) ? C : (int64_t)(STAT_BYTES / 4);
   hipLaunchKernelGGL(big_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat, a.colmax, C);
   const dim3 g1((unsigned)gx, (unsigned)(R / 64));
   switch (dtype) {

@@ -179,6 +179,16 @@ __device__ __forceinline__ void atomic_max_nonneg(float* addr, float v) {
   if (v > *reinterpret_cast<volatile float*>(addr)) atomicMax(reinterpret_cast<unsigned int*>(addr), as_u(v));
 }
 
+// Per-tensor absmax spread over 16 slots, 32 floats (one 128-byte line) apart: workgroup `wg` folds
+// its maximum into slot wg % 16; a reader takes the maximum of the slots (every lane of the calling
+// wave gets it).
+__device__ __forceinline__ void stat_slot_update(float* slots, unsigned wg, float v) {
+  atomic_max_nonneg(slots + (wg & 15u) * 32u, v);
+}
+__device__ __forceinline__ float stat_slots_max(const float* slots, int lane) {
+  return wave_max(lane < 16 ? slots[lane * 32] : 0.f);
+}
+
 // rint(x / d) with rcp = 1 / d precomputed: the product x * rcp is within 1.5 * 2^-23 |x/d| of
 // the correctly rounded quotient, so it rounds to the same integer unless it lies within 2^-14 of
 // a half-integer (|x/d| <= 128); only then is the IEEE division carried out.

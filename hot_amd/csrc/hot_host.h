@@ -23,6 +23,13 @@ inline int64_t round_up(int64_t v, int64_t m) { return (v + m - 1) / m * m; }
 constexpr int64_t GEMM_KTILE = 128;  // codes per K-tile of the int8 GEMM
 constexpr int COL_MAX_N = 128;       // largest token block one thread transforms in registers
 
+// A per-tensor absmax is collected in STAT_SLOTS partial maxima, one per 128-byte line, and the
+// consumers take the maximum of the slots: thousands of workgroups updating ONE address queue up
+// behind each other at the memory side (measured: 10 us of a 29 us statistics pass).
+constexpr int STAT_SLOTS = 16;
+constexpr int STAT_SLOT_STRIDE = 32;                                   // floats between slots
+constexpr size_t STAT_SLOT_BYTES = (size_t)STAT_SLOTS * STAT_SLOT_STRIDE * 4;   // 2048
+
 int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, int rounding,
                     uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_codes,
                     float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st,

@@ -22,6 +22,8 @@
 
 namespace hot {
 
+static_assert(STAT_SLOT_BYTES == HOT_HQ_WORKSPACE_BYTES, "the public workspace size of hot_hq_rowwise is the slot array");
+
 constexpr int EPL = 8;  // elements per lane-chunk
 
 template <typename T>
@@ -178,7 +180,7 @@ __global__ void hq_absmax_kernel(const T* __restrict__ in, int64_t nchunks, floa
   if (threadIdx.x == 0) {
     float m = s_red[0];
     for (int i = 1; i < (int)(blockDim.x >> 6); ++i) m = fmaxf(m, s_red[i]);
-    atomic_max_nonneg(absmax, m);
+    stat_slot_update(absmax, blockIdx.x, m);
   }
 }
 
@@ -190,7 +192,7 @@ __global__ void hq_tensor_kernel(const T* __restrict__ in, int64_t nchunks, int6
                                  float* __restrict__ scale_out, uint64_t seed, uint32_t stream, int nrt) {
   const int lane = threadIdx.x & 63;
   constexpr float QMAXF = (float)((1 << (BITS - 1)) - 1);
-  const float s = *absmax / QMAXF;
+  const float s = stat_slots_max(absmax, lane) / QMAXF;   // absmax: STAT_SLOTS partial maxima
   const float d = s + 1e-11f;
   const float rcp = 1.0f / d;
   if (blockIdx.x == 0 && threadIdx.x == 0) *scale_out = s;
@@ -258,7 +260,7 @@ static int launch_tensor(const void* in, int64_t M, int64_t K, void* codes, int6
   if (blocks > cap) blocks = cap;
   if (blocks < 1) blocks = 1;
   if (!absmax_ready) {
-    hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(64), 0, st, (uint32_t*)absmax, 0u, 1);
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(2), dim3(256), 0, st, (uint32_t*)absmax, 0u, (int)(STAT_SLOT_BYTES / 4));
     hipLaunchKernelGGL((hq_absmax_kernel<T, N>), dim3((unsigned)blocks), dim3(block), 0, st, (const T*)in, nch, absmax, nrt);
   }
   hipLaunchKernelGGL((hq_tensor_kernel<T, N, BITS, ROUND>), dim3((unsigned)blocks), dim3(block), 0, st,
@@ -320,7 +322,7 @@ int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int 
   if (ld_codes < K * bits / 8 || (ld_codes & 7)) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: code pitch %lld must be a multiple of 8 and >= %lld", (long long)ld_codes, (long long)(K * bits / 8));
   float* absmax = nullptr;
   if (scale_mode == HOT_SCALE_TENSOR) {
-    if (!workspace || workspace_bytes < 256) return fail(HOT_ERR_WORKSPACE, "hot_hq_rowwise: per-tensor scale needs a 256-byte workspace");
+    if (!workspace || workspace_bytes < STAT_SLOT_BYTES) return fail(HOT_ERR_WORKSPACE, "hot_hq_rowwise: per-tensor scale needs a %zu-byte workspace", STAT_SLOT_BYTES);
     absmax = (float*)workspace;
   }
   if (M == 0) return HOT_OK;

@@ -110,7 +110,7 @@ def hq_rowwise(x: torch.Tensor, n: int = 16, bits: int = 4, rounding="nearest", 
     mode = _SCALE[scale]
     codes = torch.empty((M, K * bits // 8), dtype=torch.int8, device=x.device)
     scales = torch.empty((M if mode == SCALE_ROW else 1,), dtype=torch.float32, device=x.device)
-    ws = _ws(256, x.device)
+    ws = _ws(_lib.HOT_HQ_WORKSPACE_BYTES, x.device)
     _lib.check(_lib.lib().hot_hq_rowwise(x.data_ptr(), _dt(x), M, K, n, bits, _ROUND[rounding], seed, rng_stream,
                                          mode, codes.data_ptr(), scales.data_ptr(), ws.data_ptr(), ws.numel(),
                                          _stream()))

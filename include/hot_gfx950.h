@@ -63,6 +63,7 @@ enum hot_scale_mode {
 /* Counter-based RNG stream identifiers (Philox counter word 2). */
 enum hot_rng_stream { HOT_STREAM_GX = 0, HOT_STREAM_GW = 1, HOT_STREAM_W = 2, HOT_STREAM_ACT = 3 };
 
+#define HOT_HQ_WORKSPACE_BYTES 2048 /* per-tensor absmax of hot_hq_rowwise: 16 partial maxima, one per 128-byte line */
 #define HOT_MAX_HLA_N 64        /* largest block with its rows inline in hot_config     */
 #define HOT_MAX_HLA_BIG 8192    /* largest block at all (rows through hla_rows_big)     */
 
@@ -101,7 +102,7 @@ HOT_API int64_t hot_kpad(int64_t k);
  *   bits        4: codes_out is [M, K/2] bytes, element 2j in bits 3:0 of byte j
  *               8: codes_out is [M, K] int8
  *   scale_mode  HOT_SCALE_TENSOR -> scales_out[1]; HOT_SCALE_ROW -> scales_out[M]
- *   workspace   device, >= 256 bytes, 256-byte aligned (TENSOR mode only)
+ *   workspace   device, >= HOT_HQ_WORKSPACE_BYTES, 256-byte aligned (TENSOR mode only)
  */
 HOT_API int hot_hq_rowwise(const void* in, int dtype, int64_t M, int64_t K, int n, int bits,
                    int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
