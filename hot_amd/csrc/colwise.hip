@@ -30,6 +30,7 @@ namespace hot {
 
 constexpr int CW = 256;        // threads per workgroup = channels per workgroup
 constexpr size_t COL_STAT_BYTES = 256 + STAT_SLOT_BYTES;   // step / clip words, then the absmax slots
+constexpr int COLMAX_COPIES = 8;  // per-channel maxima: workgroup row y folds into copy y % 8 (fewer atomics per line)
 constexpr int CW_ROWS = 16;    // rows staged per step
 
 struct ColArgs {
@@ -42,7 +43,7 @@ struct ColArgs {
   float* stat;        // [1] step s, [2] clip (SAWB)
   float* slots;       // TENSOR: absmax in STAT_SLOTS partial maxima
   double* partial;    // SAWB: 2 doubles per workgroup
-  float* colmax;      // ROW: per-channel absmax
+  float* colmax;      // ROW: per-channel absmax, COLMAX_COPIES arrays of C floats
   float* scales_out;
   float* row_absmax;  // statistics pass with RS != 0: absmax of the row-wise block Hadamard (STAT_SLOTS partial maxima)
   uint64_t seed;
@@ -223,7 +224,12 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     __syncthreads();
     // absmax modes read the statistic itself (no finalize kernel in between) and publish the step
     if (a.mode == HOT_SCALE_ROW) {
-      const float sc = active ? a.colmax[c] / (float)qmax : 0.f;
+      float cm = 0.f;
+      if (active) {
+#pragma unroll
+        for (int k = 0; k < COLMAX_COPIES; ++k) cm = fmaxf(cm, a.colmax[k * a.C + c]);
+      }
+      const float sc = cm / (float)qmax;
       d = active ? sc + 1e-11f : 1.f;
       if (active && blockIdx.y == 0) a.scales_out[c] = sc;
     } else if (a.mode == HOT_SCALE_TENSOR) {
@@ -383,7 +389,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       __syncthreads();
     }
     if (a.mode == HOT_SCALE_ROW) {
-      if (active) atomic_max_nonneg(a.colmax + c, cmax);
+      if (active) atomic_max_nonneg(a.colmax + (blockIdx.y % COLMAX_COPIES) * a.C + c, cmax);
       return;
     }
     if (a.mode == HOT_SCALE_TENSOR) {
@@ -419,29 +425,39 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     const int ndw = (int)((seg_end - seg0) / 4);            // output dwords per channel
     const int sdw = out_sb / 4;                             // of which staged
     const int nch = (int)((a.C - cg0) < CW ? (a.C - cg0) : CW);
-    // consecutive threads walk along K within a channel, then on to the next channel; (ch, jd) of
-    // position p = tid + k CW advance by a fixed step, so the loop carries them instead of dividing
-    const int total = nch * ndw;
-    const int step_ch = CW / ndw, step_jd = CW - step_ch * ndw;
-    int ch = tid / ndw, jd = tid - ch * ndw;
-    int8_t* dst = a.out + (cg0 + ch) * a.ld_out + seg0 + (int64_t)jd * 4;
-    const int64_t step_dst = step_ch * a.ld_out + (int64_t)step_jd * 4, wrap_dst = a.ld_out - (int64_t)ndw * 4;
-    for (int p = tid; p < total; p += CW, ch += step_ch, jd += step_jd, dst += step_dst) {
-      if (jd >= ndw) { jd -= ndw; ++ch; dst += wrap_dst; }
-      const uint32_t* row = reinterpret_cast<const uint32_t*>(stage + ch * pitch);
-      uint32_t w = 0u;
-      if (jd < sdw) {
-        if (a.store4) {
-          const uint32_t lo = row[2 * jd], hi = row[2 * jd + 1];
-          // bytes b0..b7 -> nibbles: byte j of the result = (b[2j+1] << 4) | (b[2j] & 15)
-          const uint32_t l = (lo & 0x0F) | ((lo >> 4) & 0xF0) | ((lo >> 8) & 0x0F00) | ((lo >> 12) & 0xF000);
-          const uint32_t h = (hi & 0x0F) | ((hi >> 4) & 0xF0) | ((hi >> 8) & 0x0F00) | ((hi >> 12) & 0xF000);
-          w = (l & 0xFFFF) | (h << 16);
-        } else {
-          w = row[jd];
-        }
+    // output dword jd of a staged channel row (packing two codes per byte when store4)
+    auto word = [&](const uint32_t* row, int jd) -> uint32_t {
+      if (jd >= sdw) return 0u;
+      if (a.store4) {
+        const uint32_t lo = row[2 * jd], hi = row[2 * jd + 1];
+        // bytes b0..b7 -> nibbles: byte j of the result = (b[2j+1] << 4) | (b[2j] & 15)
+        const uint32_t l = (lo & 0x0F) | ((lo >> 4) & 0xF0) | ((lo >> 8) & 0x0F00) | ((lo >> 12) & 0xF000);
+        const uint32_t h = (hi & 0x0F) | ((hi >> 4) & 0xF0) | ((hi >> 8) & 0x0F00) | ((hi >> 12) & 0xF000);
+        return (l & 0xFFFF) | (h << 16);
       }
-      *reinterpret_cast<uint32_t*>(dst) = w;
+      return row[jd];
+    };
+    // consecutive threads walk along K within a channel, then on to the next channel; (ch, jd) of
+    // position p = tid + k CW advance by a fixed step, so the loop carries them instead of dividing.
+    // Units of 8 bytes when the segments allow it (half the store instructions), else of 4.
+    const int unit = ((out_sb & 7) == 0 && (ndw & 1) == 0) ? 2 : 1;      // dwords per store
+    const int nun = ndw / unit;                                          // units per channel
+    const int total = nch * nun;
+    const int step_ch = CW / nun, step_jd = CW - step_ch * nun;
+    int ch = tid / nun, jd = tid - ch * nun;
+    int8_t* dst = a.out + (cg0 + ch) * a.ld_out + seg0 + (int64_t)jd * 4 * unit;
+    const int64_t step_dst = step_ch * a.ld_out + (int64_t)step_jd * 4 * unit, wrap_dst = a.ld_out - (int64_t)nun * 4 * unit;
+    for (int p = tid; p < total; p += CW, ch += step_ch, jd += step_jd, dst += step_dst) {
+      if (jd >= nun) { jd -= nun; ++ch; dst += wrap_dst; }
+      const uint32_t* row = reinterpret_cast<const uint32_t*>(stage + ch * pitch);
+      if (unit == 2) {
+        uint2 w2;
+        w2.x = word(row, 2 * jd);
+        w2.y = word(row, 2 * jd + 1);
+        *reinterpret_cast<uint2*>(dst) = w2;
+      } else {
+        *reinterpret_cast<uint32_t*>(dst) = word(row, jd);
+      }
     }
   }
 }
@@ -453,7 +469,11 @@ __global__ void __launch_bounds__(256) colwise_finalize_kernel(const ColArgs a, 
   const float qmax = (float)((1 << (a.bits - 1)) - 1);
   const int tid = threadIdx.x;
   if (a.mode == HOT_SCALE_ROW) {
-    for (int64_t c = tid; c < a.C; c += 256) a.scales_out[c] = a.colmax[c] / qmax;
+    for (int64_t c = tid; c < a.C; c += 256) {
+      float cm = 0.f;
+      for (int k = 0; k < COLMAX_COPIES; ++k) cm = fmaxf(cm, a.colmax[k * a.C + c]);
+      a.scales_out[c] = cm / qmax;
+    }
     return;
   }
   if (a.mode == HOT_SCALE_TENSOR) {
@@ -489,13 +509,13 @@ __global__ void colwise_clear_kernel(float* stat, float* colmax, int64_t C, floa
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < (int64_t)(COL_STAT_BYTES / 4)) stat[i] = 0.f;
   if (row_absmax && i < (int64_t)(STAT_SLOT_BYTES / 4)) row_absmax[i] = 0.f;
-  if (colmax && i < C) colmax[i] = 0.f;
+  if (colmax && i < C * COLMAX_COPIES) colmax[i] = 0.f;
 }
 
 // ---- host ---------------------------------------------------------------------
 
 
-size_t colwise_stats_bytes_impl(int64_t C) { return COL_STAT_BYTES + (size_t)round_up(C * 4, 256); }
+size_t colwise_stats_bytes_impl(int64_t C) { return COL_STAT_BYTES + (size_t)round_up(C * 4 * COLMAX_COPIES, 256); }
 
 size_t hla_workspace_bytes_impl(int64_t R, int64_t C, int n, int r) {
   return n > COL_MAX_N ? hla_big_workspace_bytes_impl(R, C, n, r) : colwise_workspace_bytes_impl(C);
@@ -503,7 +523,7 @@ size_t hla_workspace_bytes_impl(int64_t R, int64_t C, int n, int r) {
 
 size_t colwise_workspace_bytes_impl(int64_t C) {
   // stat | per-channel max | per-workgroup partial sums (at most 65536 workgroups)
-  return COL_STAT_BYTES + (size_t)round_up(C * 4, 256) + (size_t)(2 * sizeof(double)) * 65536;
+  return COL_STAT_BYTES + (size_t)round_up(C * 4 * COLMAX_COPIES, 256) + (size_t)(2 * sizeof(double)) * 65536;
 }
 
 template <typename T, int N, int PASS, int ROUND, bool SAWB, typename SEL, int RS = 0>
@@ -538,7 +558,7 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   if (gy > 65535 || gx * gy > 65536) return fail(HOT_ERR_UNSUPPORTED, "colwise: grid %lld x %lld too large", (long long)gx, (long long)gy);
   const dim3 grid((unsigned)gx, (unsigned)gy);
   if (!a.stats_cleared) {
-    const int64_t nclr = a.C > (int64_t)(COL_STAT_BYTES / 4) ? a.C : (int64_t)(COL_STAT_BYTES / 4);
+    const int64_t nclr = a.C * COLMAX_COPIES > (int64_t)(COL_STAT_BYTES / 4) ? a.C * COLMAX_COPIES : (int64_t)(COL_STAT_BYTES / 4);
     hipLaunchKernelGGL(colwise_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat,
                        a.mode == HOT_SCALE_ROW ? a.colmax : (float*)nullptr, a.C, a.row_absmax);
   }
@@ -643,7 +663,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   a.stat = (float*)ws;
   a.slots = (float*)(ws + 256);
   a.colmax = (float*)(ws + COL_STAT_BYTES);
-  a.partial = (double*)(ws + COL_STAT_BYTES + round_up(C * 4, 256));
+  a.partial = (double*)(ws + COL_STAT_BYTES + round_up(C * 4 * COLMAX_COPIES, 256));
   a.scales_out = scales_out;
   // the fused row-wise statistic exists for block 16 and absmax steps, and needs whole 16-blocks of channels
   a.row_absmax = (row16_absmax_out && scale_mode != HOT_SCALE_SAWB && C % 16 == 0) ? row16_absmax_out : nullptr;
