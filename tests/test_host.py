@@ -168,6 +168,9 @@ def test_library_exports_every_declared_symbol():
     for n in names:
         assert hasattr(lib, n), n
     assert _lib.lib().hot_abi_version() == 2
+    header = open(os.path.join(ROOT, "include", "hot_gfx950.h")).read()
+    for name in ("HOT_MAX_HLA_N", "HOT_MAX_HLA_BIG", "HOT_HQ_WORKSPACE_BYTES"):     # the binding repeats these constants
+        assert int(re.search(r"#define\s+%s\s+(\d+)" % name, header).group(1)) == getattr(_lib, name)
     assert [_lib.lib().hot_kpad(k) for k in (1, 128, 129, 7092)] == [128, 128, 256, 7168]
 
 
