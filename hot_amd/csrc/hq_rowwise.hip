@@ -43,13 +43,14 @@ template <int N>
 __device__ __forceinline__ void fwht_lanes(float* x, int lane, int nrt) {
 #pragma unroll
   for (int h = 1; h < EPL; h <<= 1) {
-    if (N <= EPL && h >= nrt) break;
+    if (N > EPL || h < nrt) {   // no early exit: the stage loop must unroll for x to stay in registers
 #pragma unroll
-    for (int j = 0; j < EPL; ++j) {
-      if ((j & h) == 0) {
-        const float a = x[j], b = x[j + h];
-        x[j] = a + b;
-        x[j + h] = a - b;
+      for (int j = 0; j < EPL; ++j) {
+        if ((j & h) == 0) {
+          const float a = x[j], b = x[j + h];
+          x[j] = a + b;
+          x[j + h] = a - b;
+        }
       }
     }
   }
