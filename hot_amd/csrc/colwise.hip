@@ -221,9 +221,13 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
 
   float d = 1.f, rcp = 1.f, clip = 0.f;
   if constexpr (PASS == 1) {
-    uint32_t* l32 = reinterpret_cast<uint32_t*>(stage);
-    for (int i = tid; i < CW * pitch / 4; i += CW) l32[i] = 0u;   // gaps of partial groups must read as 0
-    __syncthreads();
+    // gaps of partial groups must read as 0; a workgroup with all its channels and blocks writes
+    // every staged byte itself
+    if (nblk < a.tb || cg0 + CW > a.C) {
+      uint32_t* l32 = reinterpret_cast<uint32_t*>(stage);
+      for (int i = tid; i < CW * pitch / 4; i += CW) l32[i] = 0u;
+      __syncthreads();
+    }
     // absmax modes read the statistic itself (no finalize kernel in between) and publish the step
     if (a.mode == HOT_SCALE_ROW) {
       float cm = 0.f;
