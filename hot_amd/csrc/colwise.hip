@@ -323,8 +323,10 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       // stays +-(the true coefficient), and the product with +-1 is exact: the magnitudes are those
       // of the add/sub butterflies.  One v_fmac with a DPP operand per stage; the stages run
       // row-major over the 16 rows, so no DPP read follows the write of its register within two
-      // instructions.  The raw rows are consumed here, so the first token-wise stage (rows 2j and
-      // 2j+1, always within a step) is taken from them first.
+      // instructions (and two wait states separate the rows' last writes from the first stage).
+      // The raw rows are consumed here, so the first token-wise stage (rows 2j and 2j+1, always
+      // within a step) is taken from them first.
+      static_assert(CW_ROWS == 16, "the operand list below names sixteen rows");
       float t[CW_ROWS];
       rs_column<T>(my + (s % CW_DEPTH) * BUF, chan & 63, t);
       if constexpr (N >= 2) {
@@ -334,7 +336,11 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
 #pragma unroll
         for (int j = 0; j < CW_ROWS; ++j) dst[j] = t[j];
       }
-      asm volatile("s_nop 1");
+      // every row is in its register before the first DPP read (the hazard check of the compiler
+      // does not look into asm statements): the statement below takes all sixteen as operands
+      asm volatile("s_nop 1"
+                   : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7]),
+                     "+v"(t[8]), "+v"(t[9]), "+v"(t[10]), "+v"(t[11]), "+v"(t[12]), "+v"(t[13]), "+v"(t[14]), "+v"(t[15]));
 #pragma unroll
       for (int i = 0; i < CW_ROWS; ++i)
         asm volatile("v_fmac_f32_dpp %0, %0, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf" : "+v"(t[i]) : "v"(sg1));
