@@ -51,6 +51,7 @@ struct ColArgs {
   uint64_t seed;
   uint32_t stream;
   int32_t r, rpad, bits, store4, rounding, mode, tb, stats_cleared;
+  uint32_t gx, gy;     // logical grid: channel strips x runs of token blocks
   hipEvent_t after_stats;  // host only: recorded between the statistics and the quantise pass
   int8_t slot[COL_MAX_N];  // output position of natural row i, -1 = dropped
 };
@@ -187,9 +188,20 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   constexpr int CW_DEPTH = ring_depth<T>();
   uint8_t* const stage = lds + CW_DEPTH * BUF;               // PASS 1: codes [channel][k]
 
+  // One-dimensional launch.  The hardware deals consecutive workgroups to the eight XCDs in turn;
+  // each XCD takes a contiguous chunk of the logical order, which runs along the token blocks
+  // of one channel strip: the workgroups an XCD runs side by side then write neighbouring runs
+  // of the same output rows, and its L2 merges their partial lines.
+  // (The statistics pass stores nothing and keeps the plain order, strips fastest.)
+  const unsigned ngrid = a.gx * a.gy, chunk = (ngrid + 7u) >> 3;
+  const unsigned wg_lin = PASS == 1 ? (blockIdx.x & 7u) * chunk + (blockIdx.x >> 3) : blockIdx.x;
+  if (wg_lin >= ngrid) return;
+  const unsigned bx = PASS == 1 ? wg_lin / a.gy : wg_lin % a.gx;
+  const unsigned by = PASS == 1 ? wg_lin - bx * a.gy : wg_lin / a.gx;
+  const unsigned wg_id = by * a.gx + bx;     // the numbering the ordered reductions use
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int64_t cg0 = (int64_t)blockIdx.x * CW;
+  const int64_t cg0 = (int64_t)bx * CW;
   // Fused row statistic: within each group of 16 lanes the channels are dealt out so that the four
   // stages of the 16-point row transform pair lanes at the distances a single DPP operand reaches
   // (channel bit 0 <-> lane xor 1, bit 1 <-> xor 2, bit 2 <-> xor 15, bit 3 <-> xor 8).
@@ -197,7 +209,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   const int chan = RSP ? (tid ^ ((tid & 4) ? 0xB : 0)) : tid;   // channel of this thread within the workgroup
   const int64_t c = cg0 + chan;
   const bool active = c < a.C;
-  const int64_t blk0 = (int64_t)blockIdx.y * a.tb;
+  const int64_t blk0 = (int64_t)by * a.tb;
   int nblk = (int)((a.NB - blk0) < a.tb ? (a.NB - blk0) : a.tb);
   const int nsteps = (nblk * N + CW_ROWS - 1) / CW_ROWS;
   const int qmax = (1 << (a.bits - 1)) - 1;
@@ -237,11 +249,11 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       }
       const float sc = cm / (float)qmax;
       d = active ? sc + 1e-11f : 1.f;
-      if (active && blockIdx.y == 0) a.scales_out[c] = sc;
+      if (active && by == 0) a.scales_out[c] = sc;
     } else if (a.mode == HOT_SCALE_TENSOR) {
       const float sc = stat_slots_max(a.slots, lane) / (float)qmax;
       d = sc + 1e-11f;
-      if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) a.scales_out[0] = sc;
+      if (bx == 0 && by == 0 && tid == 0) a.scales_out[0] = sc;
     } else {
       d = a.stat[1] + 1e-11f;
       clip = a.stat[2];
@@ -396,12 +408,12 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       if (tid == 0) {
         float mm = s_max[0];
         for (int i = 1; i < CW / 64; ++i) mm = fmaxf(mm, s_max[i]);
-        stat_slot_update(a.row_absmax, blockIdx.y * gridDim.x + blockIdx.x, mm);
+        stat_slot_update(a.row_absmax, wg_id, mm);
       }
       __syncthreads();
     }
     if (a.mode == HOT_SCALE_ROW) {
-      if (active) atomic_max_nonneg(a.colmax + (blockIdx.y % COLMAX_COPIES) * a.C + c, cmax);
+      if (active) atomic_max_nonneg(a.colmax + (by % COLMAX_COPIES) * a.C + c, cmax);
       return;
     }
     if (a.mode == HOT_SCALE_TENSOR) {
@@ -411,7 +423,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       if (tid == 0) {
         float mm = s_max[0];
         for (int i = 1; i < CW / 64; ++i) mm = fmaxf(mm, s_max[i]);
-        stat_slot_update(a.slots, blockIdx.y * gridDim.x + blockIdx.x, mm);
+        stat_slot_update(a.slots, wg_id, mm);
       }
       return;
     }
@@ -423,7 +435,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     if (tid == 0) {
       double q = 0.0, b = 0.0;
       for (int i = 0; i < CW / 64; ++i) { q += s_sum[0][i]; b += s_sum[1][i]; }
-      const int64_t wg = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
+      const int64_t wg = (int64_t)wg_id;
       a.partial[2 * wg] = q;
       a.partial[2 * wg + 1] = b;
     }
@@ -432,7 +444,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     // flush: each channel's staged run is one contiguous global segment
     const bool last = blk0 + a.tb >= a.NB;
     const int out_sb = a.store4 ? sb / 2 : sb;
-    const int64_t seg0 = (int64_t)blockIdx.y * out_sb;      // byte offset in the output row
+    const int64_t seg0 = (int64_t)by * out_sb;      // byte offset in the output row
     const int64_t seg_end = last ? a.ld_out : seg0 + out_sb;
     const int ndw = (int)((seg_end - seg0) / 4);            // output dwords per channel
     const int sdw = out_sb / 4;                             // of which staged
@@ -547,7 +559,10 @@ static int launch_pass(const ColArgs& a, dim3 grid, size_t lds, hipStream_t st) 
     if (e != hipSuccess) return check_hip(e, "hipFuncSetAttribute(colwise_kernel)");
     attr_done = true;
   }
-  hipLaunchKernelGGL((colwise_kernel<T, N, PASS, ROUND, SAWB, SEL, RS>), grid, dim3(CW), lds, st, a);
+  ColArgs b = a;
+  b.gx = grid.x; b.gy = grid.y;
+  const unsigned total = grid.x * grid.y;
+  hipLaunchKernelGGL((colwise_kernel<T, N, PASS, ROUND, SAWB, SEL, RS>), dim3(((total + 7u) >> 3) << 3), dim3(CW), lds, st, b);
   return HOT_OK;
 }
 
