@@ -348,6 +348,12 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
 #pragma unroll
         for (int j = 0; j < CW_ROWS; ++j) dst[j] = t[j];
       }
+      // the first token-wise stage is complete before the rows are overwritten (else the compiler
+      // keeps copies of them)
+      asm volatile(""
+                   : "+v"(dst[0]), "+v"(dst[1]), "+v"(dst[2]), "+v"(dst[3]), "+v"(dst[4]), "+v"(dst[5]), "+v"(dst[6]),
+                     "+v"(dst[7]), "+v"(dst[8]), "+v"(dst[9]), "+v"(dst[10]), "+v"(dst[11]), "+v"(dst[12]),
+                     "+v"(dst[13]), "+v"(dst[14]), "+v"(dst[15]));
       // every row is in its register before the first DPP read (the hazard check of the compiler
       // does not look into asm statements): the statement below takes all sixteen as operands
       asm volatile("s_nop 1"
