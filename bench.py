@@ -71,13 +71,13 @@ def make_layer(L, O, I, dtype, dev, nsets, seed=0):
 # counter reads for a 512 MiB device copy (FETCH_SIZE reads half the bytes, WRITE_SIZE all of them).
 # Summary and commands: profiles/hot_linear_backward_vit_b_fc1_bf16.hbm_traffic.txt
 MEASURED_TRAFFIC_BYTES = {
-    "gy_stats": (2 * 37914.4 + 14.1) * 1024,
-    "gy_hla_quant": (2 * 37938.0 + 29271.0) * 1024,      # the g_y launches (the trace averages 4 launches on x in)
-    "gy_hq_quant": (2 * 37870.4 + 18912.0) * 1024,
-    "w_stats": (2 * 2333.0 + 4.5) * 1024,
-    "w_quant": (2 * 2362.5 + 1152.0) * 1024,
-    "gemm_gx": (2 * 19705.1 + 18912.0) * 1024,
-    "gemm_gw": (2 * 39547.4 + 27648.0 + 2 * 13863.0 + 4608.0) * 1024,   # K-range kernel + reduce kernel
+    "gy_stats": (2 * 37911.5 + 19.7) * 1024,
+    "gy_hla_quant": (2 * 37947.0 + 21683.0) * 1024,      # the g_y launches (the trace averages 4 launches on x in)
+    "gy_hq_quant": (2 * 37869.4 + 18912.0) * 1024,
+    "w_stats": (2 * 2333.7 + 4.5) * 1024,
+    "w_quant": (2 * 2363.5 + 1152.0) * 1024,
+    "gemm_gx": (2 * 19683.1 + 18912.0) * 1024,
+    "gemm_gw": (2 * 39542.7 + 27648.0 + 2 * 13863.0 + 4608.0) * 1024,   # K-range kernel + reduce kernel
 }
 
 
