@@ -11,6 +11,7 @@ low-rank rows), :228-254 (cache).
 """
 from __future__ import annotations
 
+import functools
 import math
 from typing import Dict, Tuple
 
@@ -84,12 +85,19 @@ def _kept_sequencies(n: int, percentile: float) -> np.ndarray:
     return np.concatenate(keep)
 
 
+@functools.lru_cache(maxsize=256)
+def _hla_rows_cached(n: int, percentile: float) -> np.ndarray:
+    order = np.argsort(_sequency(n), kind="stable")   # natural row of each sequency
+    rows = order[_kept_sequencies(n, percentile)]
+    rows.setflags(write=False)                        # shared between callers
+    return rows
+
+
 def hla_rows(size_m: int, percentile: float = 50) -> Tuple[int, np.ndarray]:
     """(n, natural-order row of each kept coefficient) for a token count: the
-    rule behind make_WHT, in the index form the kernels take."""
+    rule behind make_WHT, in the index form the kernels take (the array is cached and read-only)."""
     n = 1 if size_m == 1 else biggest_power2_factor(size_m)
-    order = np.argsort(_sequency(n), kind="stable")   # natural row of each sequency
-    return n, order[_kept_sequencies(n, percentile)]
+    return n, _hla_rows_cached(int(n), float(percentile))
 
 
 def paper_rows(n: int = 16, r: int = 8) -> Tuple[int, np.ndarray]:

@@ -7,7 +7,7 @@ all arithmetic happens in libhot_gfx950.so.
 from __future__ import annotations
 
 import ctypes as C
-from dataclasses import dataclass, field
+from dataclasses import dataclass, field, replace
 from typing import Optional, Sequence, Tuple
 
 import torch
@@ -52,7 +52,7 @@ def kpad(k: int) -> int:
     return int(_lib.lib().hot_kpad(int(k)))
 
 
-@dataclass
+@dataclass(frozen=True)
 class HotOptions:
     """Options of the fused path (struct hot_config); the fields FLinearQ reads
     from the reference's module-global ``args`` for scheme gih_gwlr."""
@@ -80,7 +80,28 @@ class HotOptions:
     def lprime(self, L: int) -> int:
         return (L // self.hla_n) * self.hla_r
 
+    def with_seed(self, seed: int) -> "HotOptions":
+        """The same options under another stochastic-rounding key; reuses the built C struct."""
+        seed = int(seed)
+        if seed == self.seed:
+            return self
+        other = replace(self, seed=seed)
+        base = self.to_c()
+        c = _lib.HotConfig.from_buffer_copy(base)
+        c.seed = seed & 0xFFFFFFFFFFFFFFFF
+        object.__setattr__(other, "_c", c)
+        object.__setattr__(other, "_keep", base)     # owner of what hla_rows_big points to
+        return other
+
     def to_c(self) -> _lib.HotConfig:
+        """struct hot_config for these options (built once per object; the library only reads it)."""
+        c = self.__dict__.get("_c")
+        if c is None:
+            c = self._build_c()
+            object.__setattr__(self, "_c", c)
+        return c
+
+    def _build_c(self) -> _lib.HotConfig:
         if self.hla_n > _lib.HOT_MAX_HLA_BIG:
             raise HotError("HLA block %d exceeds the native maximum %d" % (self.hla_n, _lib.HOT_MAX_HLA_BIG))
         c = _lib.HotConfig()

@@ -70,10 +70,32 @@ def hot_switched_off() -> bool:
             and all(getattr(args, k) in off for k in ("quantBWDGogi", "quantBWDWgt", "quantBWDGogw", "quantBWDAct")))
 
 
+_OPTIONS_CACHE: dict = {}
+
+
 def options_for(tokens: int, layer_name: str = " ", out_features: int = 16) -> ops.HotOptions:
     """args.* -> HotOptions, following the branch structure of FLinearQ.  The Hadamard block along the
     out-features is the reference's make_hadamard rule: the largest power of two dividing them, at
-    most 16 (utils/hadamard_matmul.py:57-59): 16 for the usual widths, 4 for a 100-class head."""
+    most 16 (utils/hadamard_matmul.py:57-59): 16 for the usual widths, 4 for a 100-class head.
+    The result is cached per state of the flags it reads (layers call this on every step)."""
+    auto = bool(args.quantAuto and len(args.layer_quant_dict) > 0)
+    key = (tokens, out_features, args.transform_scheme, args.TransformGogi, args.TransformWgt, args.TransformGogw,
+           args.TransformInput, args.quantBWDGogi, args.quantBWDWgt, args.quantBWDGogw, args.quantBWDAct,
+           args.GogiQuantBit, args.weightQuantBit, args.GogwQuantBit, args.actQuantBit, args.hla_rule,
+           args.hla_max_block, args.vectorPercentile,
+           (args.layer_quant_dict.get(layer_name + "_gx"), args.layer_quant_dict.get(layer_name + "_gw")) if auto else None)
+    seed = (int(args.sr_seed) << 20) + int(args.sr_step)
+    hit = _OPTIONS_CACHE.get(key)
+    if hit is not None:
+        return hit.with_seed(seed)
+    if len(_OPTIONS_CACHE) > 4096:
+        _OPTIONS_CACHE.clear()
+    opt = _options_uncached(tokens, layer_name, out_features)
+    _OPTIONS_CACHE[key] = opt
+    return opt.with_seed(seed)
+
+
+def _options_uncached(tokens: int, layer_name: str, out_features: int) -> ops.HotOptions:
     if args.transform_scheme != "gih_gwlr":
         raise NotImplementedError("transform scheme %r: only gih_gwlr runs natively" % args.transform_scheme)
     if not (args.TransformGogi and args.TransformWgt and args.TransformGogw and args.TransformInput):
@@ -110,17 +132,34 @@ def _pad8(t: Tensor) -> Tensor:
     return F.pad(t, (0, extra)).contiguous() if extra else t.contiguous()
 
 
+# torch keeps the transform check where Function.apply itself reads it; without it the class falls
+# back to the stock apply
+_PLAIN_APPLY = hasattr(torch._C, "_are_functorch_transforms_active")
+
+
 class FLinearQ(Function):
     """torch.autograd.Function with the reference's forward / setup_context /
     backward triple (utils/quant_matmul.py:169-348)."""
 
+    @classmethod
+    def apply(cls, x, w, h_out, h_bs, name, bias=None):
+        # Function.apply inspects the signature of forward on every call to fill in defaults
+        # (about 30 us); with all six arguments in hand there is nothing to fill in
+        if _PLAIN_APPLY and not torch._C._are_functorch_transforms_active():
+            return super(Function, cls).apply(x, w, h_out, h_bs, name, bias)
+        return super().apply(x, w, h_out, h_bs, name, bias)
+
     @staticmethod
-    def forward(x, w, h_out, h_bs, name):
-        return F.linear(x, w)
+    def forward(x, w, h_out, h_bs, name, bias=None):
+        # `bias` is an addition to the reference's five arguments (which adds the bias after the
+        # Function, utils/quant_matmul.py:419-420): inside, it rides in the GEMM epilogue instead of
+        # costing a pass over the output
+        return F.linear(x, w, bias)
 
     @staticmethod
     def setup_context(ctx, inputs, output):
-        x, w, _h_out, _h_bs, name = inputs
+        x, w, _h_out, _h_bs, name = inputs[:5]
+        ctx.has_bias = len(inputs) > 5 and inputs[5] is not None
         ctx.name = name
         ctx.x_shape = tuple(x.shape)
         ctx.full_precision = hot_switched_off()
@@ -153,7 +192,7 @@ class FLinearQ(Function):
             grad_w = go.mT @ x.to(w.dtype)
             if grad_w.dim() == 3:                    # [B, O, I]: the sum over samples autograd would take
                 grad_w = grad_w.sum(dim=0)
-            return go @ w, grad_w, None, None, None
+            return go @ w, grad_w, None, None, None, FLinearQ._bias_grad(ctx, grad_output)
         xq, w, sx = ctx.saved_tensors
         opt = ctx.opt
         go = grad_output
@@ -175,7 +214,13 @@ class FLinearQ(Function):
             grad_input = gx[:, :I].reshape(ctx.x_shape)
         if O % 8 or I % 8:
             grad_w = grad_w[:O, :I]
-        return grad_input, grad_w, None, None, None
+        return grad_input, grad_w, None, None, None, FLinearQ._bias_grad(ctx, grad_output)
+
+    @staticmethod
+    def _bias_grad(ctx, grad_output):
+        if not (ctx.has_bias and ctx.needs_input_grad[5]):
+            return None
+        return grad_output.reshape(-1, grad_output.shape[-1]).sum(dim=0)
 
 
 class HQ_Linear(nn.Linear):
@@ -207,7 +252,7 @@ class HQ_Linear(nn.Linear):
             self.hadamard_bs = torch.ones((1, 1), dtype=self.weight.dtype, device=self.weight.device)
             return
         # P = rows of H_n
-        idx = torch.as_tensor(np.asarray(rows), dtype=torch.long)
+        idx = torch.tensor(np.array(rows), dtype=torch.long)
         i = idx[:, None] & torch.arange(n)[None, :]
         par = torch.zeros_like(i)
         while bool(i.any()):
@@ -220,10 +265,7 @@ class HQ_Linear(nn.Linear):
             self._refresh_bs(input.shape[1])
         else:
             self._refresh_bs(input.numel() // input.shape[-1])
-        output = FLinearQ.apply(input, self.weight, self.hadamard_out, self.hadamard_bs, self.layer_name)
-        if self.bias is not None:
-            output = output + self.bias.to(output.device)
-        return output
+        return FLinearQ.apply(input, self.weight, self.hadamard_out, self.hadamard_bs, self.layer_name, self.bias)
 
 
 class HQ_Conv2d(nn.Conv2d):
@@ -242,14 +284,19 @@ class HQ_Conv2d(nn.Conv2d):
     def forward(self, input: Tensor) -> Tensor:
         if self.groups > 1:                          # depth-wise convolution
             raise NotImplementedError
-        B, _, H, W = input.shape
-        cols = F.unfold(input, self.kernel_size, dilation=self.dilation, padding=self.padding,
-                        stride=self.stride).transpose(1, 2)              # [B, H'W', C k k]
+        B, Cin, H, W = input.shape
+        kh, kw = self.kernel_size
+        if (tuple(self.stride) == (kh, kw) and tuple(self.padding) == (0, 0) and tuple(self.dilation) == (1, 1)
+                and self.padding_mode == "zeros" and H % kh == 0 and W % kw == 0):
+            # non-overlapping patches (a ViT patch embedding): unfold is a permutation, one copy
+            # instead of the im2col kernel
+            cols = (input.reshape(B, Cin, H // kh, kh, W // kw, kw).permute(0, 2, 4, 1, 3, 5)
+                    .reshape(B, (H // kh) * (W // kw), Cin * kh * kw))
+        else:
+            cols = F.unfold(input, self.kernel_size, dilation=self.dilation, padding=self.padding,
+                            stride=self.stride).transpose(1, 2)          # [B, H'W', C k k]
         weight = self.weight.view(self.weight.size(0), -1)
-        output = FLinearQ.apply(cols, weight, self.hadamard_out, self.hadamard_bs, self.layer_name)
+        output = FLinearQ.apply(cols, weight, self.hadamard_out, self.hadamard_bs, self.layer_name, self.bias)
         ho = (H + 2 * self.padding[0] - self.dilation[0] * (self.kernel_size[0] - 1) - 1) // self.stride[0] + 1
         wo = (W + 2 * self.padding[1] - self.dilation[1] * (self.kernel_size[1] - 1) - 1) // self.stride[1] + 1
-        output = output.transpose(1, 2).reshape(B, self.out_channels, ho, wo)
-        if self.bias is not None:
-            output = output + self.bias.view(1, -1, 1, 1)
-        return output
+        return output.transpose(1, 2).reshape(B, self.out_channels, ho, wo)

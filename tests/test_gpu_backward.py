@@ -314,6 +314,35 @@ def test_hq_conv2d_matches_oracle(gpu, fresh_args):
     assert torch.allclose(conv.bias.grad.cpu(), G.cpu().sum((0, 2, 3)), rtol=1e-4, atol=1e-7)
 
 
+def test_hq_conv2d_overlapping_patches(gpu, fresh_args):
+    """Kernel 3, stride 1, padding 1: the unfold path (the non-overlapping case above is a plain
+    permutation); the input gradient is the fold (a sum over overlapping patches) of the oracle's."""
+    from hot_amd.quant_matmul import HQ_Conv2d
+    B, C, H, W, O, k = 2, 8, 8, 8, 16, 3
+    torch.manual_seed(4)
+    conv = HQ_Conv2d(C, O, kernel_size=k, stride=1, padding=1).to(gpu)
+    x = torch.randn(B, C, H, W, device=gpu, requires_grad=True)
+    y = conv(x)
+    assert torch.allclose(y, torch.nn.functional.conv2d(x, conv.weight, conv.bias, padding=1), atol=1e-5, rtol=1e-5)
+    G = torch.randn_like(y) * 1e-3
+    y.backward(G)
+    L = H * W
+    ocfg, _ = both_configs(L)
+    cols = torch.nn.functional.unfold(x.detach().cpu(), k, padding=1).transpose(1, 2)      # [B, L, C k k]
+    gy = G.cpu().flatten(2).transpose(1, 2)
+    wn = conv.weight.detach().cpu().reshape(O, -1).numpy()
+    gw, gcols = 0, []
+    for b in range(B):
+        xq_ref, sx_ref = orc.abc_forward(cols[b].contiguous().numpy(), ocfg)
+        tr = orc.linear_backward(gy[b].contiguous().numpy(), wn, xq_ref, sx_ref, ocfg)
+        gw = gw + tr.g_w
+        gcols.append(torch.from_numpy(tr.g_x))
+    gx = torch.nn.functional.fold(torch.stack(gcols).transpose(1, 2), (H, W), k, padding=1)
+    assert rel(x.grad.cpu().numpy(), gx.numpy()) < 1e-6
+    assert rel(conv.weight.grad.cpu().reshape(O, -1).numpy(), gw) < 1e-6
+
+
+
 def test_lqs_then_hot_training_step(gpu, fresh_args):
     """Calibrate in the plain setting, then take a HOT step with the selected quantisers."""
     from hot_amd import lqs, utils as hutils
