@@ -19,8 +19,8 @@ class Attention(nn.Module):
 
     def forward(self, x):
         B, T, C = x.shape
-        qkv = self.qkv(x).reshape(B, T, 3, self.heads, C // self.heads).permute(2, 0, 3, 1, 4)
-        y = F.scaled_dot_product_attention(qkv[0], qkv[1], qkv[2])
+        q, k, v = self.qkv(x).reshape(B, T, 3, self.heads, C // self.heads).permute(2, 0, 3, 1, 4).unbind(0)
+        y = F.scaled_dot_product_attention(q, k, v)   # unbind: one gradient stack instead of three zero-filled ones
         return self.proj(y.transpose(1, 2).reshape(B, T, C))
 
 
