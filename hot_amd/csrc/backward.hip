@@ -183,7 +183,7 @@ enum {
 };
 
 // The two W kernels are small (a few MB) and cannot fill the chip; they run on a side stream beside
-// the g_y kernels.  One side stream and two events per device, created on first use (default
+// the g_y kernels.  One side stream and three events per device, created on first use (default
 // priority) and kept for the life of the process; a mutex keeps the fork / join of one call together.
 struct SideLane {
   hipStream_t stream = nullptr;
