@@ -110,8 +110,8 @@ def kernel_table(w, sets, bufs, opt, ws, iters, warm, traffic=None):
         ("w_stats", "hot::colwise_kernel<.., PASS 0> (W)", us[4], "hbm", O * I * e),
         ("w_quant", "hot::colwise_kernel<.., PASS 1> (W: Hadamard-16 + INT%d, transposed)" % opt.w_bits, us[5], "hbm",
          O * I * e + O * I * opt.w_bits // 8),
-        ("gemm_gx", "hot::gemm_i8_pipe_kernel<2, 2, %d, ..> (g_x)" % opt.gx_bits, us[6], "mfma", 2.0 * L * O * I),
-        ("gemm_gw", "hot::gemm_i8_pipe_kernel<2, 2, 8, ..> (g_W)" + (" in %d K ranges + gemm_i8_reduce_kernel" % gw_splits
+        ("gemm_gx", "hot::gemm_i8_pipe_kernel<.., %d, ..> (g_x)" % opt.gx_bits, us[6], "mfma", 2.0 * L * O * I),
+        ("gemm_gw", "hot::gemm_i8_pipe_kernel<.., 8, ..> (g_W)" + (" in %d K ranges + gemm_i8_reduce_kernel" % gw_splits
                                                                      if gw_splits > 1 else ""),
          us[7], "mfma", 2.0 * O * I * lp),
     ]
@@ -390,10 +390,13 @@ def main():
         pn, prow = paper_rows(16, 8)
         lopt = ops.HotOptions(n_o=16, hla_n=int(pn), hla_rows=tuple(int(v) for v in prow))
         lw, lsets = make_layer(Ll, Ol, Il, torch.bfloat16, dev, nsets=2, seed=1)
-        lsec, _, _ = step_time(lw, lsets, lopt, max(5, a.steps // 5), max(2, a.warmup // 5))
+        lsec, lbufs, lws = step_time(lw, lsets, lopt, max(5, a.steps // 5), max(2, a.warmup // 5))
+        ltable = kernel_table(lw, lsets, lbufs, lopt, lws, iters=6, warm=2)
         out["llama_gate_up"] = {"us_per_layer": round(lsec * 1e6, 1), "L": Ll, "O": Ol, "I": Il,
-                                "hla": "n=16 r=8", "int8_tops": round((2.0 * Ll * Ol * Il + 2.0 * Ol * Il * (Ll // 2)) / lsec / 1e12, 1)}
-        del lw, lsets
+                                "hla": "n=16 r=8", "int8_tops": round((2.0 * Ll * Ol * Il + 2.0 * Ol * Il * (Ll // 2)) / lsec / 1e12, 1),
+                                # kernels launched one after the other: [us, fraction of the 8 TB/s or 5 POP/s peak]
+                                "kernels_serial": {r["key"]: [r["us"], r["frac"]] for r in ltable}}
+        del lw, lsets, lbufs, lws
     if not a.no_extras and not a.table_only:
         try:
             out["hq_rowwise_sweep"] = hq_rowwise_sweep(dev)
