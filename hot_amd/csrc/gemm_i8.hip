@@ -59,11 +59,26 @@ struct GemmArgs {
 // tile grid in groups of group_m tile rows, row index fastest inside a group, so the workgroups that
 // are resident in one XCD at the same time form a compact block of tiles: they stream few distinct
 // A and B row panels, and most of their loads hit in that XCD's L2.
-__device__ __forceinline__ void tile_of(const GemmArgs& g, int wg, int& tm, int& tn) {
-  const int total = g.tiles_m * g.tiles_n;
+// Position of workgroup `wg` in a launch order of `total` units in which XCD x (= wg % 8) takes the
+// x-th contiguous chunk.
+__device__ __forceinline__ int xcd_chunk_position(int total, int wg) {
   const int x = wg & 7, idx = wg >> 3;
   const int q = total >> 3, rem = total & 7;
-  const int t = x * q + (x < rem ? x : rem) + idx;
+  return x * q + (x < rem ? x : rem) + idx;
+}
+
+// Tile of position t in the grouped walk of the tile grid.
+__device__ __forceinline__ void grouped_tile(const GemmArgs& g, int t, int& tm, int& tn) {
+  const int per_group = g.group_m * g.tiles_n;
+  const int grp = t / per_group, j = t - grp * per_group;
+  const int rows = min(g.group_m, g.tiles_m - grp * g.group_m);
+  tm = grp * g.group_m + j % rows;
+  tn = j / rows;
+}
+
+__device__ __forceinline__ void tile_of(const GemmArgs& g, int wg, int& tm, int& tn) {
+  const int total = g.tiles_m * g.tiles_n;
+  const int t = xcd_chunk_position(total, wg);
   const int per_group = g.group_m * g.tiles_n;
   const int grp = t / per_group, j = t - grp * per_group;
   const int rows = min(g.group_m, g.tiles_m - grp * g.group_m);
@@ -382,9 +397,18 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = wave >> 1, wn = wave & 1;
   const int tiles_total = g.tiles_m * g.tiles_n;
-  const int split = (int)blockIdx.x / tiles_total, tile_id = (int)blockIdx.x - split * tiles_total;
-  int tm, tn;
-  tile_of(g, tile_id, tm, tn);
+  // Split launches order their (K range, tile) units range-major and give each XCD a contiguous
+  // chunk: the workgroups sharing an L2 then work on ONE K range of a compact block of tiles, a
+  // fraction of the operand bytes that all ranges of fewer tiles would touch.
+  int split = 0, tile_id = (int)blockIdx.x, tm, tn;
+  if (g.splits > 1) {
+    const int u = xcd_chunk_position(tiles_total * g.splits, (int)blockIdx.x);
+    split = u / tiles_total;
+    tile_id = u - split * tiles_total;
+    grouped_tile(g, tile_id, tm, tn);
+  } else {
+    tile_of(g, tile_id, tm, tn);
+  }
   const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
   // The steps of this lane's rows: loaded here, behind the K loop's latency, when registers allow;
   // the 256 x 256 tile has none to spare and loads them in the epilogue.
@@ -588,7 +612,7 @@ __global__ void __launch_bounds__(64) gemm_i8_reduce_kernel(const GemmArgs g) {
   const int fi = frag / WN, fj = frag % WN;
   const int wm = wave >> 1, wn = wave & 1;
   int tm, tn;
-  tile_of(g, tile_id, tm, tn);
+  grouped_tile(g, tile_id, tm, tn);   // the numbering of the split launch
   const int64_t row0 = (int64_t)tm * BM + (wm * WM + fi) * 32, col0 = (int64_t)tn * BN + (wn * WN + fj) * 32;
   float sa_row[1];
   load_row_scales<1>(g, row0, lane, sa_row);
