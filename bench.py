@@ -77,7 +77,7 @@ MEASURED_TRAFFIC_BYTES = {
     "w_stats": (2 * 2333.7 + 4.5) * 1024,
     "w_quant": (2 * 2363.5 + 1152.0) * 1024,
     "gemm_gx": (2 * 19683.1 + 18912.0) * 1024,
-    "gemm_gw": (2 * 39542.7 + 27648.0 + 2 * 13863.0 + 4608.0) * 1024,   # K-range kernel + reduce kernel
+    "gemm_gw": (2 * 23058.7 + 27648.0 + 2 * 13862.0 + 4608.0) * 1024,   # K-range kernel + reduce kernel
 }
 
 
