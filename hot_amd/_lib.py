@@ -25,7 +25,7 @@ EXPORTS = (
     "hot_last_error", "hot_abi_version", "hot_kpad", "hot_hq_rowwise", "hot_hla_tokenwise",
     "hot_wq_colwise", "hot_colwise_workspace_bytes", "hot_gemm_i8", "hot_abc_workspace_bytes",
     "hot_abc_forward", "hot_backward_workspace_bytes", "hot_linear_backward", "hot_linear_backward_kernels",
-    "hot_gemm_splits", "hot_hla_workspace_bytes",
+    "hot_gemm_splits", "hot_hla_workspace_bytes", "hot_linear_backward_bias",
 )
 
 
@@ -84,6 +84,8 @@ def _declare(lib):
     lib.hot_gemm_splits.argtypes = [i64, i64, i64, i32]
     lib.hot_linear_backward_kernels.restype = i32
     lib.hot_linear_backward_kernels.argtypes = lib.hot_linear_backward.argtypes
+    lib.hot_linear_backward_bias.restype = i32
+    lib.hot_linear_backward_bias.argtypes = [vp, vp, i32, vp, vp, i64, i64, i64, cfgp, vp, vp, vp, i32, vp, sz, vp]
 
 
 def lib():

@@ -48,7 +48,8 @@ static int check_cfg(const hot_config* c, const char* who) {
 
 struct BwdLayout {
   int64_t ld_g, ld_w, ld_gp;                       // code pitches in bytes
-  size_t off_hq, off_colw, off_colg, off_sg, off_sw, off_sgp, off_qg, off_qw, off_qgp, off_split, total;
+  size_t off_hq, off_colw, off_colg, off_sg, off_sw, off_sgp, off_qg, off_qw, off_qgp, off_split, off_colsum, total;
+  int64_t colsum_strips;                         // rows of partial column sums of g_y (bias gradient)
   size_t split_bytes;                            // split-K workspace shared by the two GEMMs
 };
 
@@ -73,6 +74,8 @@ static BwdLayout bwd_layout(int64_t L, int64_t O, int64_t I, const hot_config* c
   const GemmSplit px = gemm_split_plan(L, I, O, c->gx_bits), pw = gemm_split_plan(O, I, lp, 8);
   b.split_bytes = px.ws_bytes > pw.ws_bytes ? px.ws_bytes : pw.ws_bytes;
   b.off_split = o; o += align256(b.split_bytes);
+  b.colsum_strips = colsum_strips_impl(L, O, c->hla_n, c->hla_r, 0, c->gw_scale);
+  b.off_colsum = o; o += align256((size_t)b.colsum_strips * (size_t)O * 4);
   b.total = o;
   return b;
 }
@@ -211,7 +214,8 @@ static SideLane* side_lane_locked() {
 static int run_backward(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,
                         int64_t O, int64_t I, const hot_config* cfg, void* gx, void* gw, int out_dtype,
                         void* workspace, size_t workspace_bytes, hipEvent_t* ev /* K_COUNT + 1 or null */,
-                        int* slot_of /* K_COUNT: kernel group measured by event pair i, i + 1 */, hipStream_t st) {
+                        int* slot_of /* K_COUNT: kernel group measured by event pair i, i + 1 */, hipStream_t st,
+                        void* gb = nullptr /* [O] of out_dtype: column sums of g_y, or null */) {
   const char* who = "hot_linear_backward";
   if (int e = check_cfg(cfg, who)) return e;
   if (!gy || !w || !xq || !sx || !gx || !gw) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
@@ -289,8 +293,15 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
                           cfg->seed, HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp,
                           ws + b.off_colg, hla_workspace_bytes_impl(L, O, cfg->hla_n, cfg->hla_r), st, who,
                           fuse ? (float*)(ws + b.off_hq) : nullptr, /*stats_cleared=*/true,
-                          hq_aside ? side->fork2 : mid(K_GY_STATS));
+                          hq_aside ? side->fork2 : mid(K_GY_STATS), gb ? (float*)(ws + b.off_colsum) : nullptr);
   if (rc) return rc;
+  // bias gradient: the partial column sums of the statistics pass, added up by a small kernel that
+  // rides on the side stream behind the row-wise quantise pass, beside the large kernels of the main
+  // stream (here, in order, when there is no side stream)
+  auto finish_bias = [&](hipStream_t s2) {
+    return gb ? colsum_finish_impl((const float*)(ws + b.off_colsum), b.colsum_strips, O, gb, out_dtype, s2) : HOT_OK;
+  };
+  if (!side && (rc = finish_bias(st))) return rc;
   mark(K_GY_HLA);
   // g_x operand of g_y on the side stream: a streaming kernel beside the g_W GEMM
   auto quantise_gy_rows = [&](hipStream_t s2) {
@@ -306,6 +317,7 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   if (hq_aside) {
     rc = check_hip(hipStreamWaitEvent(side->stream, side->fork2, 0), "hipStreamWaitEvent");   // statistics are in
     if (!rc) rc = quantise_gy_rows(side->stream);
+    if (!rc) rc = finish_bias(side->stream);
     if (!rc && gx_aside) rc = gemm_gx(side->stream);
     if (rc) return rc;
   }
@@ -379,6 +391,14 @@ int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq
   times4[2] = k[K_GEMM_GX];
   times4[3] = k[K_GEMM_GW];
   return HOT_OK;
+}
+
+int hot_linear_backward_bias(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,
+                             int64_t O, int64_t I, const hot_config* cfg, void* gx, void* gw, void* gb, int out_dtype,
+                             void* workspace, size_t workspace_bytes, void* hip_stream) {
+  if (!gb) return fail(HOT_ERR_INVALID, "hot_linear_backward_bias: null pointer");
+  return run_backward(gy, w, dtype, xq, sx, L, O, I, cfg, gx, gw, out_dtype, workspace, workspace_bytes, nullptr,
+                      nullptr, (hipStream_t)hip_stream, gb);
 }
 
 int hot_linear_backward_kernels(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,

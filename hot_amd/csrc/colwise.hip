@@ -48,6 +48,7 @@ struct ColArgs {
   float* colmax;      // ROW: per-channel absmax, COLMAX_COPIES arrays of C floats
   float* scales_out;
   float* row_absmax;  // statistics pass with RS != 0: absmax of the row-wise block Hadamard (STAT_SLOTS partial maxima)
+  float* colsum;      // statistics pass: NULL or per-channel sums of the input, one row of C floats per run of token blocks
   uint64_t seed;
   uint32_t stream;
   int32_t r, rpad, bits, store4, rounding, mode, tb, stats_cleared;
@@ -261,7 +262,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     rcp = 1.0f / d;
   }
 
-  float cmax = 0.f, rmax = 0.f;
+  float cmax = 0.f, rmax = 0.f, csum = 0.f;
   double ssq = 0.0, sab = 0.0;
   float x[XL];
 
@@ -272,6 +273,8 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     for (int g = 0; g < BPS; ++g) {
       const int blk = bl + g;
       if (blk < nblk) {
+        // coefficient 0 of a block is the sum of its tokens (row 0 of H is all ones)
+        if constexpr (PASS == 0) csum += x[g * N];
         int visited = 0;      // kept coefficients of this block quantised so far (stochastic rounding)
         float u[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -405,6 +408,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   }
 
   if constexpr (PASS == 0) {
+    if (a.colsum && active) a.colsum[(int64_t)by * a.C + c] = csum;
     if constexpr (RS != 0) {
       // rows past the end of the input were redirected to real rows and channels past C form whole
       // inactive blocks, so only the latter need masking
@@ -542,6 +546,64 @@ __global__ void colwise_clear_kernel(float* stat, float* colmax, int64_t C, floa
   if (colmax && i < C * COLMAX_COPIES) colmax[i] = 0.f;
 }
 
+// ---- column sums ------------------------------------------------------------------
+
+// Sums of a strip of rows per channel, thread = channel: the stand-alone form of what the statistics
+// pass of colwise_kernel delivers for free (used when the token blocks take the two-level path).
+template <typename T>
+__global__ void __launch_bounds__(256) colsum_strip_kernel(const void* in, int64_t R, int64_t C, int64_t rows_per_wg,
+                                                            float* partial) {
+  typedef typename raw_of<T>::type raw_t;
+  const int64_t c = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= C) return;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_wg;
+  const int64_t r1 = r0 + rows_per_wg < R ? r0 + rows_per_wg : R;
+  const raw_t* p = reinterpret_cast<const raw_t*>(in) + r0 * C + c;
+  float acc = 0.f;
+  int64_t r = r0;
+  for (; r + 8 <= r1; r += 8, p += 8 * C) {
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = cvt_raw<T>(p[i * C]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc += v[i];
+  }
+  for (; r < r1; ++r, p += C) acc += cvt_raw<T>(*p);
+  partial[(int64_t)blockIdx.y * C + c] = acc;
+}
+
+// out[c] = sum of partial[s][c] over the strips s, rounded once to the output type, in a fixed order:
+// eight groups of threads take the strips s = g, g + 8, g + 16, ... of a channel (eight loads in
+// flight each, added in strip order), then the eight group sums are added in group order.  A
+// workgroup covers 32 channels, so that a few hundred strips are a short chain of loads per thread.
+constexpr int CS_GROUPS = 8, CS_CHANS = 32;
+template <typename OutT>
+__global__ void __launch_bounds__(CS_GROUPS * CS_CHANS) colsum_finish_kernel(const float* partial, int strips, int64_t C, OutT* out) {
+  __shared__ float s_part[CS_GROUPS][CS_CHANS];
+  const int ch = threadIdx.x % CS_CHANS, g = threadIdx.x / CS_CHANS;
+  const int64_t c = (int64_t)blockIdx.x * CS_CHANS + ch;
+  float acc = 0.f;
+  if (c < C) {
+    int s = g;
+    for (; s + 7 * CS_GROUPS < strips; s += 8 * CS_GROUPS) {
+      float v[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] = partial[(int64_t)(s + i * CS_GROUPS) * C + c];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc += v[i];
+    }
+    for (; s < strips; s += CS_GROUPS) acc += partial[(int64_t)s * C + c];
+  }
+  s_part[g][ch] = acc;
+  __syncthreads();
+  if (g == 0 && c < C) {
+    float t = s_part[0][ch];
+#pragma unroll
+    for (int i = 1; i < CS_GROUPS; ++i) t += s_part[i][ch];
+    store_scalar<OutT>(out + c, t);
+  }
+}
+
 // ---- host ---------------------------------------------------------------------
 
 
@@ -572,22 +634,35 @@ static int launch_pass(const ColArgs& a, dim3 grid, size_t lds, hipStream_t st) 
   return HOT_OK;
 }
 
-template <typename T, int N, typename SEL>
-static int launch_colwise(ColArgs& a, hipStream_t st) {
-  constexpr int BPS = N >= CW_ROWS ? 1 : CW_ROWS / N;
-  // Token blocks per workgroup.  The staged run of a channel (tb * r codes) must be a whole number
-  // of output dwords and cover the blocks that share a 16-row step; beyond that, longer runs (up
-  // to 128 bytes) are taken only while they leave at least four workgroups per CU.
-  const int64_t gx0 = (a.C + CW - 1) / CW;
-  auto run_bytes = [&](int t) { return a.store4 ? t * a.r / 2 : t * a.r; };   // t * r is a multiple of 8 when store4
+// Token blocks per workgroup of the quantise pass (tb) and of an absmax statistics pass (tb0).
+// The staged run of a channel (tb * r codes) must be a whole number of output dwords and cover the
+// blocks that share a 16-row step; beyond that, longer runs (up to 128 bytes) are taken only while
+// they leave at least four workgroups per CU.  Absmax statistics stage nothing: while the grid has
+// fewer than 2048 workgroups they take shorter workgroups, down to 64 rows (measured 1 us faster at
+// 12608 x 3072).  The SAWB sums are order-sensitive and keep the partition of the quantise pass.
+struct ColPartition { int tb, tb0; };
+static ColPartition col_partition(int n, int r, int store4, int mode, int64_t C, int64_t NB) {
+  const int BPS = n >= CW_ROWS ? 1 : CW_ROWS / n;
+  const int64_t gx = (C + CW - 1) / CW;
+  auto run_bytes = [&](int t) { return store4 ? t * r / 2 : t * r; };   // t * r is a multiple of 8 when store4
   int tb = BPS;
-  while ((tb * a.r) % (a.store4 ? 8 : 4) != 0 || run_bytes(tb) < 32) tb <<= 1;
-  while (run_bytes(tb) < 128 && gx0 * ((a.NB + 2 * tb - 1) / (2 * tb)) >= 1024) tb <<= 1;
+  while ((tb * r) % (store4 ? 8 : 4) != 0 || run_bytes(tb) < 32) tb <<= 1;
+  while (run_bytes(tb) < 128 && gx * ((NB + 2 * tb - 1) / (2 * tb)) >= 1024) tb <<= 1;
   {
     static int forced = -1;   // experiments: HOT_COL_TB overrides the rule (must keep runs whole dwords)
     if (forced < 0) { const char* e = getenv("HOT_COL_TB"); forced = e ? atoi(e) : 0; }
-    if (forced > 0 && forced % BPS == 0 && (forced * a.r) % (a.store4 ? 8 : 4) == 0) tb = forced;
+    if (forced > 0 && forced % BPS == 0 && (forced * r) % (store4 ? 8 : 4) == 0) tb = forced;
   }
+  int tb0 = tb;
+  if (mode != HOT_SCALE_SAWB)
+    while (tb0 > BPS && (tb0 & 1) == 0 && tb0 * n > 64 && gx * ((NB + tb0 - 1) / tb0) < 2048) tb0 >>= 1;
+  return {tb, tb0};
+}
+
+template <typename T, int N, typename SEL>
+static int launch_colwise(ColArgs& a, hipStream_t st) {
+  const ColPartition part = col_partition(N, a.r, a.store4, a.mode, a.C, a.NB);
+  const int tb = part.tb;
   a.tb = tb;
   const size_t in_bytes = (size_t)ring_depth<T>() * CW_ROWS * CW * sizeof(T);
   const size_t lds_stats = in_bytes, lds_quant = in_bytes + (size_t)CW * (tb * a.r + 4);
@@ -604,10 +679,8 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   if (a.mode == HOT_SCALE_SAWB) {
     rc = launch_pass<T, N, 0, 0, true, SEL>(a, grid, lds_stats, st);   // same partition as ever: the sums are order-sensitive
   } else {
-    // absmax statistics stage nothing: while the grid has fewer than 2048 workgroups they take
-    // shorter ones, down to 64 rows (measured 1 us faster at 12608 x 3072)
     ColArgs a0 = a;
-    while (a0.tb > BPS && (a0.tb & 1) == 0 && a0.tb * N > 64 && gx * ((a.NB + a0.tb - 1) / a0.tb) < 2048) a0.tb >>= 1;
+    a0.tb = part.tb0;
     const dim3 grid0((unsigned)gx, (unsigned)((a.NB + a0.tb - 1) / a0.tb));
     if (a.row_absmax) rc = launch_pass<T, N, 0, 0, false, SEL, 16>(a0, grid0, lds_stats, st);
     else rc = launch_pass<T, N, 0, 0, false, SEL>(a0, grid0, lds_stats, st);
@@ -624,6 +697,38 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   }
   if (rc) return rc;
   return check_launch("colwise_kernel");
+}
+
+// Rows of the partial column sums a token-wise call writes: one per run of token blocks of its
+// statistics pass; the stand-alone kernel of the large-block path takes strips of at least 64 rows,
+// about 2048 workgroups in all.
+static int64_t colsum_strip_rows_big(int64_t R, int64_t C) {
+  const int64_t gx = (C + 255) / 256;
+  const int64_t want = 2048 / gx > 0 ? 2048 / gx : 1;
+  const int64_t rows = round_up((R + want - 1) / want, 16);
+  return rows < 64 ? 64 : rows;
+}
+
+int64_t colsum_strips_impl(int64_t R, int64_t C, int n, int r, int store4, int mode) {
+  if (R <= 0 || C <= 0 || n < 1 || r < 1) return 0;
+  if (n > COL_MAX_N) {
+    const int64_t rows = colsum_strip_rows_big(R, C);
+    return (R + rows - 1) / rows;
+  }
+  const int64_t NB = R / n;
+  const ColPartition part = col_partition(n, r, store4, mode, C, NB);
+  return (NB + part.tb0 - 1) / part.tb0;
+}
+
+int colsum_finish_impl(const float* partial, int64_t strips, int64_t C, void* out, int out_dtype, hipStream_t st) {
+  const dim3 grid((unsigned)((C + CS_CHANS - 1) / CS_CHANS)), block(CS_GROUPS * CS_CHANS);
+  switch (out_dtype) {
+    case HOT_F32: hipLaunchKernelGGL(colsum_finish_kernel<float>, grid, block, 0, st, partial, (int)strips, C, (float*)out); break;
+    case HOT_BF16: hipLaunchKernelGGL(colsum_finish_kernel<bf16_t>, grid, block, 0, st, partial, (int)strips, C, (bf16_t*)out); break;
+    case HOT_F16: hipLaunchKernelGGL(colsum_finish_kernel<f16_t>, grid, block, 0, st, partial, (int)strips, C, (f16_t*)out); break;
+    default: return fail(HOT_ERR_INVALID, "column sums: bad output dtype %d", out_dtype);
+  }
+  return check_launch("colsum_finish_kernel");
 }
 
 template <typename SEL, int N>
@@ -662,7 +767,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
                        int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
                        void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,
                        size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out,
-                       bool stats_cleared, hipEvent_t after_stats) {
+                       bool stats_cleared, hipEvent_t after_stats, float* colsum_partial) {
   if (!in || !codes_out || !scales_out || !rows) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
   if (R <= 0 || C <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape R=%lld C=%lld", who, (long long)R, (long long)C);
   if (n > COL_MAX_N) {
@@ -673,6 +778,16 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
     if (bits != 4 && bits != 8) return fail(HOT_ERR_UNSUPPORTED, "%s: bits=%d (4 or 8)", who, bits);
     if (rounding != HOT_ROUND_NEAREST && rounding != HOT_ROUND_STOCH) return fail(HOT_ERR_INVALID, "%s: bad rounding %d", who, rounding);
     if (scale_mode < HOT_SCALE_TENSOR || scale_mode > HOT_SCALE_SAWB) return fail(HOT_ERR_INVALID, "%s: bad scale mode %d", who, scale_mode);
+    if (colsum_partial) {
+      const int64_t rows = colsum_strip_rows_big(R, C);
+      const dim3 grid((unsigned)((C + 255) / 256), (unsigned)((R + rows - 1) / rows));
+      switch (dtype) {
+        case HOT_F32: hipLaunchKernelGGL(colsum_strip_kernel<float>, grid, dim3(256), 0, st, in, R, C, rows, colsum_partial); break;
+        case HOT_BF16: hipLaunchKernelGGL(colsum_strip_kernel<bf16_t>, grid, dim3(256), 0, st, in, R, C, rows, colsum_partial); break;
+        case HOT_F16: hipLaunchKernelGGL(colsum_strip_kernel<f16_t>, grid, dim3(256), 0, st, in, R, C, rows, colsum_partial); break;
+        default: return fail(HOT_ERR_INVALID, "%s: bad dtype %d", who, dtype);
+      }
+    }
     return hla_big_impl(in, dtype, R, C, n, rows, r, bits, rounding, seed, rng_stream, scale_mode, codes_out, ld_out,
                         scales_out, workspace, workspace_bytes, st, who, after_stats);
   }
@@ -712,6 +827,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   a.partial = (double*)(ws + COL_STAT_BYTES + round_up(C * 4 * COLMAX_COPIES, 256));
   a.scales_out = scales_out;
   // the fused row-wise statistic exists for block 16 and absmax steps, and needs whole 16-blocks of channels
+  a.colsum = colsum_partial;
   a.row_absmax = (row16_absmax_out && scale_mode != HOT_SCALE_SAWB && C % 16 == 0) ? row16_absmax_out : nullptr;
   if (row16_absmax_out && !a.row_absmax) return fail(HOT_ERR_UNSUPPORTED, "%s: fused row statistic unavailable for this configuration", who);
   switch (dtype) {

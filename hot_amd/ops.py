@@ -207,9 +207,12 @@ def abc_forward(x: torch.Tensor, opt: HotOptions):
 
 
 def linear_backward(gy: torch.Tensor, w: torch.Tensor, xq: torch.Tensor, sx: torch.Tensor, opt: HotOptions,
-                    out_dtype=None, timing: bool = False, workspace: Optional[torch.Tensor] = None):
+                    out_dtype=None, timing: bool = False, workspace: Optional[torch.Tensor] = None,
+                    bias_grad: bool = False):
     """g_x [L, I], g_W [O, I]; with timing=True also the four stage times (s), with
-    timing="kernels" the eight per-kernel times of hot_linear_backward_kernels."""
+    timing="kernels" the eight per-kernel times of hot_linear_backward_kernels; with
+    bias_grad=True also g_b [O], the sum of g_y over the tokens (hot_linear_backward_bias:
+    delivered by the statistics pass, no extra read of g_y; not combined with timing)."""
     _need_gpu_2d(gy, "Go")
     _need_gpu_2d(w, "Wt")
     L, O = gy.shape
@@ -230,6 +233,14 @@ def linear_backward(gy: torch.Tensor, w: torch.Tensor, xq: torch.Tensor, sx: tor
         workspace = _ws(need, gy.device)
     gx = torch.empty((L, I), dtype=out_dtype, device=gy.device)
     gw = torch.empty((O, I), dtype=out_dtype, device=gy.device)
+    if bias_grad:
+        if timing:
+            raise ValueError("bias_grad and timing are separate entry points")
+        gb = torch.empty((O,), dtype=out_dtype, device=gy.device)
+        _lib.check(_lib.lib().hot_linear_backward_bias(
+            gy.data_ptr(), w.data_ptr(), _dt(gy), xq.data_ptr(), sx.data_ptr(), L, O, I, C.byref(cfg), gx.data_ptr(),
+            gw.data_ptr(), gb.data_ptr(), _DTYPES[out_dtype], workspace.data_ptr(), workspace.numel(), _stream()))
+        return gx, gw, gb
     per_kernel = timing == "kernels"
     times = (C.c_float * (8 if per_kernel else 4))() if timing else None
     entry = _lib.lib().hot_linear_backward_kernels if per_kernel else _lib.lib().hot_linear_backward

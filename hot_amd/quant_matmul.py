@@ -210,6 +210,14 @@ class FLinearQ(Function):
             grad_w = gw.to(wc.dtype)
         else:
             go2 = go.reshape(-1, go.shape[-1])
+            if ctx.has_bias and ctx.needs_input_grad[5]:
+                # the statistics pass over g_y holds the sum of every token block: the bias gradient
+                # comes out of the same call instead of a reduction of its own over g_y
+                gx, grad_w, gb = ops.linear_backward(_pad8(go2), wc, xq, sx, opt, bias_grad=True)
+                grad_input = gx[:, :I].reshape(ctx.x_shape)
+                if O % 8 or I % 8:
+                    grad_w = grad_w[:O, :I]
+                return grad_input, grad_w, None, None, None, gb[:O].to(grad_output.dtype)
             gx, grad_w = ops.linear_backward(_pad8(go2), wc, xq, sx, opt)
             grad_input = gx[:, :I].reshape(ctx.x_shape)
         if O % 8 or I % 8:

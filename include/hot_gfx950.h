@@ -183,6 +183,21 @@ HOT_API int hot_linear_backward(const void* gy, const void* w, int dtype, const 
                         void* hip_stream);
 
 /*
+ * hot_linear_backward (without stage timings) that also returns the bias gradient
+ * gb[O] of out_dtype: the sum of g_y over the tokens, accumulated in fp32 in a fixed order
+ * (within a token block in the butterfly order of the transform, whose coefficient 0 it
+ * is; then block after block) and rounded once.  It costs no pass over g_y: the statistics
+ * pass of the token-wise kernel already holds every block's sum.  The reference adds the
+ * bias outside its autograd Function (utils/quant_matmul.py:419-420), so there the bias
+ * gradient is autograd's own reduction of g_y; this entry point folds that reduction into
+ * the backward of the layer.  Same workspace as hot_linear_backward.
+ */
+HOT_API int hot_linear_backward_bias(const void* gy, const void* w, int dtype, const void* xq,
+                             const float* sx, int64_t L, int64_t O, int64_t I,
+                             const hot_config* cfg, void* gx, void* gw, void* gb, int out_dtype,
+                             void* workspace, size_t workspace_bytes, void* hip_stream);
+
+/*
  * Number of K ranges into which the GEMMs inside hot_linear_backward cut a product of
  * M x N outputs over K codes of `bits` bits (1 = one kernel; more = a kernel per range
  * writing int32 partial tiles to the workspace, then a reduce kernel).  Products with

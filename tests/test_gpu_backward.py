@@ -518,3 +518,72 @@ def test_backward_exact_python_rule_on_large_blocks(gpu, L, O, I, variant):
     gx, gw, tr = run_both(x, w, gy, ocfg, opt, gpu)
     assert np.array_equal(gx.cpu().numpy(), tr.g_x)
     assert np.array_equal(gw.cpu().numpy(), tr.g_w)
+
+
+def _options_like(ocfg):
+    from hot_amd import ops
+    return ops.HotOptions(n_o=ocfg.n_o, hla_n=ocfg.hla_n, hla_rows=ocfg.hla_rows, gx_bits=ocfg.gx_bits,
+                          w_bits=ocfg.w_bits, gw_bits=ocfg.gw_bits, act_bits=ocfg.act_bits,
+                          gx_round=ocfg.gx_round, w_round=ocfg.w_round, gw_round=ocfg.gw_round,
+                          act_round=ocfg.act_round, gx_scale=ocfg.gx_scale, w_scale=ocfg.w_scale,
+                          gw_scale=ocfg.gw_scale, act_scale=ocfg.act_scale, seed=ocfg.seed)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L,O,I,rule,variant", [
+    (448, 192, 160, "python", dict()),                                             # n = 64, fused row statistic
+    (64 * 5, 208, 72, "python", dict()),                                           # O short of a workgroup's 256 channels
+    (64 * 37, 528, 64, "python", dict(gx_scale=orc.SCALE_ROW, gw_scale=orc.SCALE_ROW,
+                                      gx_round=orc.ROUND_STOCH, gw_round=orc.ROUND_STOCH, seed=5)),   # several strips
+    (448, 192, 160, "paper", dict()),                                              # n = 16, r = 8
+    (197, 96, 64, "python", dict()),                                               # n = 1
+    (384, 64, 40, "python", dict(gx_scale=orc.SCALE_ROW, gw_scale=orc.SCALE_ROW)),  # n = 128
+    (1024, 80, 48, "python", dict()),                                              # n = 1024: two-level path
+])
+def test_backward_with_bias_gradient(gpu, dtype, L, O, I, rule, variant):
+    """hot_linear_backward_bias: g_x and g_W are those of hot_linear_backward bit for bit, and g_b is
+    the sum of g_y over the tokens.  The reference has no code for it (autograd reduces g_y for the bias
+    added at utils/quant_matmul.py:419-420), so it is pinned by the mathematics: on integer-valued g_y
+    every fp32 partial sum is exact whatever the order and g_b must EQUAL the integer sum; on random
+    g_y it must lie within the fp32 accumulation bound (tokens * 2^-24 * sum |g_y|) of the float64 sum,
+    plus one rounding of the output type (2^-9 relative for bf16)."""
+    from hot_amd import ops
+    ocfg = orc.HotConfig.python_rule(L, **variant) if rule == "python" else orc.HotConfig.paper(16, 8, **variant)
+    opt = _options_like(ocfg)
+    x, w, gy = make_case(L, O, I, seed=3, dtype=dtype)
+    xq, sx = ops.abc_forward(x.to(gpu), opt)
+    gyd, wd = gy.to(gpu), w.to(gpu)
+    gx0, gw0 = ops.linear_backward(gyd, wd, xq, sx, opt)
+    gx1, gw1, gb = ops.linear_backward(gyd, wd, xq, sx, opt, bias_grad=True)
+    assert torch.equal(gx0, gx1) and torch.equal(gw0, gw1)
+    assert gb.shape == (O,) and gb.dtype == dtype
+    ref = gy.double().sum(dim=0).numpy()
+    bound = L * 2.0 ** -24 * gy.double().abs().sum(dim=0).numpy()
+    if dtype == torch.bfloat16:
+        bound = bound + 2.0 ** -8 * np.abs(ref)
+    assert np.all(np.abs(gb.double().cpu().numpy() - ref) <= bound + 1e-30)
+    # integer-valued g_y: exact sums (|sum| < 2^24), any dropped, doubled or misplaced block shows
+    g = torch.Generator().manual_seed(11)
+    gi = torch.randint(-8, 9, (L, O), generator=g).to(dtype)
+    _, _, gbi = ops.linear_backward(gi.to(gpu), wd, xq, sx, opt, out_dtype=torch.float32, bias_grad=True)
+    assert np.array_equal(gbi.cpu().numpy(), gi.double().sum(dim=0).numpy().astype(np.float32))
+    # a second call on the same workspace with other data: nothing of the first call is left over
+    _, _, gb2 = ops.linear_backward(gyd * 2, wd, xq, sx, opt, out_dtype=torch.float32, bias_grad=True)
+    _, _, gb1 = ops.linear_backward(gyd, wd, xq, sx, opt, out_dtype=torch.float32, bias_grad=True)
+    assert torch.equal(gb2, gb1 * 2)
+
+
+def test_hq_linear_bias_gradient_from_fused_call(gpu, fresh_args):
+    """HQ_Linear with a bias: its bias gradient comes from the fused call and equals torch's
+    reduction of g_y up to the fp32 accumulation bound."""
+    from hot_amd.quant_matmul import HQ_Linear
+    torch.manual_seed(0)
+    lin = HQ_Linear(96, 200).to(gpu)              # 200 = 8 * 25: n_o = 8
+    x = torch.randn(4, 64, 96, device=gpu, requires_grad=True)
+    fresh_args.batched_mode = "flatten"
+    y = lin(x)
+    gy = torch.randn_like(y)
+    y.backward(gy)
+    ref = gy.reshape(-1, 200).double().sum(dim=0)
+    assert lin.bias.grad.shape == (200,)
+    assert float((lin.bias.grad.double() - ref).abs().max()) <= 256 * 2.0 ** -24 * float(gy.abs().sum(dim=(0, 1)).max())
