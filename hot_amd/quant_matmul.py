@@ -51,7 +51,12 @@ def _scheme(flag: str, what: str, allowed) -> Tuple[int, int]:
 
 
 def token_rule(tokens: int):
-    """(n, rows) of the low-rank projection for a token count under args.hla_rule."""
+    """(n, rows) of the token-wise transform for a token count: the low-rank projection under
+    args.hla_rule, or, with the reference's scheme "hadamard", the whole block Hadamard of make_hadamard
+    along the tokens (utils/quant_matmul.py:182-183,294-295,353-355: every coefficient, natural order)."""
+    if args.transform_scheme == "hadamard":
+        n = int(biggest_power2_factor_max16(int(tokens)))
+        return n, np.arange(n)
     if args.hla_rule == "paper":
         if tokens % 16:
             return 1, np.array([0])
@@ -96,8 +101,10 @@ def options_for(tokens: int, layer_name: str = " ", out_features: int = 16) -> o
 
 
 def _options_uncached(tokens: int, layer_name: str, out_features: int) -> ops.HotOptions:
-    if args.transform_scheme != "gih_gwlr":
-        raise NotImplementedError("transform scheme %r: only gih_gwlr runs natively" % args.transform_scheme)
+    # "hadamard" differs from "gih_gwlr" in the token-wise transform only (token_rule); the low-rank
+    # schemes on the g_x side (low_rank, gilr_gwh, gilro_gwh) need an expansion pass that is not built
+    if args.transform_scheme not in ("gih_gwlr", "hadamard"):
+        raise NotImplementedError("transform scheme %r: gih_gwlr and hadamard run natively" % args.transform_scheme)
     if not (args.TransformGogi and args.TransformWgt and args.TransformGogw and args.TransformInput):
         raise NotImplementedError("the native path needs all four Transform* flags on")
     n, rows = token_rule(tokens)
@@ -249,7 +256,7 @@ class HQ_Linear(nn.Linear):
         self.layer_name = " "
 
     def _refresh_bs(self, tokens: int) -> None:
-        key = (tokens, args.hla_rule, args.hla_max_block, args.vectorPercentile)
+        key = (tokens, args.transform_scheme, args.hla_rule, args.hla_max_block, args.vectorPercentile)
         if self._bs_tokens == key:
             return
         n, rows = token_rule(tokens)

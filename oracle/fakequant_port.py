@@ -87,18 +87,25 @@ def setup_context(x: torch.Tensor, h_bs: torch.Tensor, cfg: PortConfig):
 
 
 def backward(grad_output: torch.Tensor, w: torch.Tensor, xq: torch.Tensor, scale_x, h_out: torch.Tensor,
-             h_bs: torch.Tensor, cfg: PortConfig):
-    """quant_matmul.py:215-348, branch gih_gwlr, 2-D tensors."""
+             h_bs: torch.Tensor, cfg: PortConfig, scheme: str = "gih_gwlr"):
+    """quant_matmul.py:215-348, branch gih_gwlr, 2-D tensors; with scheme "hadamard" (h_bs = the block
+    Hadamard of make_hadamard for the token count) the g_W branch of that scheme (:294-295, :338-339)."""
     g = _front(grad_output, h_out)                              # :238
     g, s_g = _quant(g, cfg.gx_bits, cfg.gx_kind)                # :244-257
     wh = _back(h_out, w)                                        # :270
     wh, s_w = _quant(wh, cfg.w_bits, cfg.w_kind)                # :276-285
     grad_input = (g @ wh) * s_g * s_w                           # :288-290
-    gp = _back(h_bs, grad_output).T                             # :301
+    if scheme == "hadamard":
+        gp = _front(grad_output.T.contiguous(), h_bs)           # :295
+    else:
+        gp = _back(h_bs, grad_output).T                         # :301
     gp, s_gp = _quant(gp, cfg.gw_bits, cfg.gw_kind)             # :307-320
     grad_w = (gp @ xq.to(gp.dtype)) * s_gp * scale_x            # :322-324
     grad_input = grad_input / orc.pow2_factor_max16(h_out.shape[0])   # :343
-    grad_w = grad_w / orc.pow2_factor(h_bs.shape[1])                  # :344
+    if scheme == "hadamard":
+        grad_w = grad_w / orc.pow2_factor_max16(h_bs.shape[0])        # :339
+    else:
+        grad_w = grad_w / orc.pow2_factor(h_bs.shape[1])              # :344
     return grad_input, grad_w
 
 

@@ -587,3 +587,34 @@ def test_hq_linear_bias_gradient_from_fused_call(gpu, fresh_args):
     ref = gy.reshape(-1, 200).double().sum(dim=0)
     assert lin.bias.grad.shape == (200,)
     assert float((lin.bias.grad.double() - ref).abs().max()) <= 256 * 2.0 ** -24 * float(gy.abs().sum(dim=(0, 1)).max())
+
+
+@pytest.mark.parametrize("L", [448, 200])
+def test_hq_linear_scheme_hadamard(gpu, fresh_args, L):
+    """transform_scheme "hadamard" (utils/quant_matmul.py:182-183,229-230,262-263,294-295,337-339): both
+    token-wise transforms are the whole block Hadamard of make_hadamard(tokens) instead of the low-rank
+    projection, everything else as in gih_gwlr.  Bit-exact against the oracle configured with every
+    coefficient kept, and within the tolerance against the op-for-op port of that branch."""
+    from hot_amd.quant_matmul import HQ_Linear
+    I, O = 96, 128
+    fresh_args.transform_scheme = "hadamard"
+    torch.manual_seed(1)
+    lin = HQ_Linear(I, O).to(gpu)
+    x = torch.randn(L, I, device=gpu, requires_grad=True)
+    gy = torch.randn(L, O, device=gpu) * 1e-3
+    lin(x).backward(gy)
+    n = orc.pow2_factor_max16(L)
+    assert n == (16 if L == 448 else 8) and lin.hadamard_bs.shape == (n, n)
+    assert np.array_equal(lin.hadamard_bs.cpu().numpy(), orc.hadamard(n))
+    ocfg = orc.HotConfig(hla_n=n, hla_rows=tuple(range(n)))
+    xq_ref, sx_ref = orc.abc_forward(x.detach().cpu().numpy(), ocfg)
+    tr = orc.linear_backward(gy.cpu().numpy(), lin.weight.detach().cpu().numpy(), xq_ref, sx_ref, ocfg)
+    assert np.array_equal(x.grad.cpu().numpy(), tr.g_x)
+    assert np.array_equal(lin.weight.grad.cpu().numpy(), tr.g_w)
+    h_out = torch.tensor(orc.make_hadamard(O), dtype=torch.float32)
+    h_bs = torch.tensor(orc.make_hadamard(L), dtype=torch.float32)
+    xq, sx = fq.setup_context(x.detach().cpu(), h_bs, fq.PortConfig())
+    gi_ref, gw_ref = fq.backward(gy.cpu(), lin.weight.detach().cpu(), xq, sx, h_out, h_bs, fq.PortConfig(),
+                                 scheme="hadamard")
+    assert rel(x.grad.cpu().numpy(), gi_ref.numpy()) < REL_TOL
+    assert rel(lin.weight.grad.cpu().numpy(), gw_ref.numpy()) < REL_TOL

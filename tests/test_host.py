@@ -111,7 +111,11 @@ def test_options_follow_args(fresh_args):
     with pytest.raises(NotImplementedError):
         options_for(64)
     a.quantBWDGogi = "int"
-    a.transform_scheme = "hadamard"
+    a.transform_scheme = "hadamard"                 # block Hadamard along the tokens, nothing dropped
+    o = options_for(12608)
+    assert (o.hla_n, o.hla_r, o.hla_rows) == (16, 16, tuple(range(16)))
+    assert options_for(197).hla_n == 1 and options_for(200).hla_n == 8
+    a.transform_scheme = "low_rank"
     with pytest.raises(NotImplementedError):
         options_for(64)
     a.transform_scheme = "gih_gwlr"
