@@ -318,6 +318,9 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 512 MiB device-to-device copies (a kernel of known traffic, for scaling "
                          "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
+    ap.add_argument("--llama-table", action="store_true",
+                    help="only the per-kernel pass at the Llama-7B gate/up shape (kernels launched one after the "
+                         "other), printed as one JSON line; for profiling runs of that shape")
     a = ap.parse_args()
     if a.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus %d is not supported (no collectives, no sharding)"
@@ -340,6 +343,18 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    if a.llama_table:
+        Ll, Ol, Il = 8192, 11008, 4096
+        pn, prow = paper_rows(16, 8)
+        lopt = ops.HotOptions(n_o=16, hla_n=int(pn), hla_rows=tuple(int(v) for v in prow))
+        lw, lsets = make_layer(Ll, Ol, Il, torch.bfloat16, dev, nsets=2, seed=1)
+        lsec, lbufs, lws = step_time(lw, lsets, lopt, a.steps, a.warmup)
+        ltable = kernel_table(lw, lsets, lbufs, lopt, lws, iters=6, warm=2)
+        print(json.dumps({"workload": "Llama-7B gate/up linear backward (L=8192, O=11008, I=4096), bf16, HLA n=16 r=8",
+                          "us_per_layer": round(lsec * 1e6, 1), "steps": a.steps, "warmup": a.warmup,
+                          "kernels_serial": ltable}))
+        return
 
     L, O, I = 12608, 3072, 768
     n, rows = hla_rows(L)
