@@ -49,7 +49,7 @@ static int check_cfg(const hot_config* c, const char* who) {
 struct BwdLayout {
   int64_t ld_g, ld_w, ld_gp;                       // code pitches in bytes
   size_t off_hq, off_colw, off_colg, off_sg, off_sw, off_sgp, off_qg, off_qw, off_qgp, off_split, off_colsum, total;
-  int64_t colsum_strips;                         // rows of partial column sums of g_y (bias gradient)
+  int64_t colsum_strips;                         // room for that many rows of partial column sums of g_y (bias gradient)
   size_t split_bytes;                            // split-K workspace shared by the two GEMMs
 };
 
@@ -74,7 +74,11 @@ static BwdLayout bwd_layout(int64_t L, int64_t O, int64_t I, const hot_config* c
   const GemmSplit px = gemm_split_plan(L, I, O, c->gx_bits), pw = gemm_split_plan(O, I, lp, 8);
   b.split_bytes = px.ws_bytes > pw.ws_bytes ? px.ws_bytes : pw.ws_bytes;
   b.off_split = o; o += align256(b.split_bytes);
-  b.colsum_strips = colsum_strips_impl(L, O, c->hla_n, c->hla_r, 0, c->gw_scale);
+  {  // the workspace query knows no input type: room for the larger partition of the two element sizes
+    const int64_t s2 = colsum_strips_impl(L, O, c->hla_n, c->hla_r, 0, c->gw_scale, 2);
+    const int64_t s4 = colsum_strips_impl(L, O, c->hla_n, c->hla_r, 0, c->gw_scale, 4);
+    b.colsum_strips = s2 > s4 ? s2 : s4;
+  }
   b.off_colsum = o; o += align256((size_t)b.colsum_strips * (size_t)O * 4);
   b.total = o;
   return b;
@@ -299,7 +303,9 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   // rides on the side stream behind the row-wise quantise pass, beside the large kernels of the main
   // stream (here, in order, when there is no side stream)
   auto finish_bias = [&](hipStream_t s2) {
-    return gb ? colsum_finish_impl((const float*)(ws + b.off_colsum), b.colsum_strips, O, gb, out_dtype, s2) : HOT_OK;
+    if (!gb) return (int)HOT_OK;
+    const int64_t strips = colsum_strips_impl(L, O, cfg->hla_n, cfg->hla_r, 0, cfg->gw_scale, dtype == HOT_F32 ? 4 : 2);
+    return colsum_finish_impl((const float*)(ws + b.off_colsum), strips, O, gb, out_dtype, s2);
   };
   if (!side && (rc = finish_bias(st))) return rc;
   mark(K_GY_HLA);

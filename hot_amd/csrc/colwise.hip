@@ -636,18 +636,31 @@ static int launch_pass(const ColArgs& a, dim3 grid, size_t lds, hipStream_t st) 
 
 // Token blocks per workgroup of the quantise pass (tb) and of an absmax statistics pass (tb0).
 // The staged run of a channel (tb * r codes) must be a whole number of output dwords and cover the
-// blocks that share a 16-row step; beyond that, longer runs (up to 128 bytes) are taken only while
-// they leave at least four workgroups per CU.  Absmax statistics stage nothing: while the grid has
-// fewer than 2048 workgroups they take shorter workgroups, down to 64 rows (measured 1 us faster at
-// 12608 x 3072).  The SAWB sums are order-sensitive and keep the partition of the quantise pass.
+// blocks that share a 16-row step, and is at least 32 bytes long.  Beyond that, runs grow (up to 128
+// bytes) only while the grid keeps four workgroups per CU and the staging area does not cost a
+// resident workgroup: with the ring of a 16-bit input three workgroups share a CU up to 80 staged
+// bytes per channel, and the quantise pass lost a quarter of its speed each time a longer run took
+// one away (measured at 8192 x 11008 and 11008 x 4096; the L2 of an XCD merges the short runs of
+// neighbouring workgroups anyway).  (Runs below 32 bytes make a small W kernel faster on its own,
+// 8 us instead of 11 at 3072 x 768, but its four times as many workgroups then get in the way of the
+// g_y statistics pass it runs beside: the step came out 2 us slower.)  Absmax statistics stage nothing: while the grid has fewer than 2048
+// workgroups they take shorter workgroups, down to 64 rows (measured 1 us faster at 12608 x 3072).
+// The SAWB sums are order-sensitive and keep the partition of the quantise pass.
 struct ColPartition { int tb, tb0; };
-static ColPartition col_partition(int n, int r, int store4, int mode, int64_t C, int64_t NB) {
+static ColPartition col_partition(int n, int r, int store4, int mode, int64_t C, int64_t NB, int elem_bytes) {
   const int BPS = n >= CW_ROWS ? 1 : CW_ROWS / n;
   const int64_t gx = (C + CW - 1) / CW;
+  const size_t ring = (size_t)(elem_bytes == 4 ? 3 : 4) * CW_ROWS * CW * elem_bytes;
   auto run_bytes = [&](int t) { return store4 ? t * r / 2 : t * r; };   // t * r is a multiple of 8 when store4
+  auto wgs = [&](int t) { return gx * ((NB + t - 1) / t); };
+  auto resident = [&](int t) {   // workgroups of the quantise pass per CU, as far as LDS decides (three are enough)
+    const size_t per = ring + (size_t)CW * (t * r + 4) + 256;
+    const int k = (int)((160u * 1024u) / per);
+    return k > 3 ? 3 : k;
+  };
   int tb = BPS;
   while ((tb * r) % (store4 ? 8 : 4) != 0 || run_bytes(tb) < 32) tb <<= 1;
-  while (run_bytes(tb) < 128 && gx * ((NB + 2 * tb - 1) / (2 * tb)) >= 1024) tb <<= 1;
+  while (run_bytes(tb) < 128 && wgs(2 * tb) >= 1024 && resident(2 * tb) >= resident(tb)) tb <<= 1;
   {
     static int forced = -1;   // experiments: HOT_COL_TB overrides the rule (must keep runs whole dwords)
     if (forced < 0) { const char* e = getenv("HOT_COL_TB"); forced = e ? atoi(e) : 0; }
@@ -655,13 +668,13 @@ static ColPartition col_partition(int n, int r, int store4, int mode, int64_t C,
   }
   int tb0 = tb;
   if (mode != HOT_SCALE_SAWB)
-    while (tb0 > BPS && (tb0 & 1) == 0 && tb0 * n > 64 && gx * ((NB + tb0 - 1) / tb0) < 2048) tb0 >>= 1;
+    while (tb0 > BPS && (tb0 & 1) == 0 && tb0 * n > 64 && wgs(tb0) < 2048) tb0 >>= 1;
   return {tb, tb0};
 }
 
 template <typename T, int N, typename SEL>
 static int launch_colwise(ColArgs& a, hipStream_t st) {
-  const ColPartition part = col_partition(N, a.r, a.store4, a.mode, a.C, a.NB);
+  const ColPartition part = col_partition(N, a.r, a.store4, a.mode, a.C, a.NB, (int)sizeof(T));
   const int tb = part.tb;
   a.tb = tb;
   const size_t in_bytes = (size_t)ring_depth<T>() * CW_ROWS * CW * sizeof(T);
@@ -709,14 +722,14 @@ static int64_t colsum_strip_rows_big(int64_t R, int64_t C) {
   return rows < 64 ? 64 : rows;
 }
 
-int64_t colsum_strips_impl(int64_t R, int64_t C, int n, int r, int store4, int mode) {
+int64_t colsum_strips_impl(int64_t R, int64_t C, int n, int r, int store4, int mode, int elem_bytes) {
   if (R <= 0 || C <= 0 || n < 1 || r < 1) return 0;
   if (n > COL_MAX_N) {
     const int64_t rows = colsum_strip_rows_big(R, C);
     return (R + rows - 1) / rows;
   }
   const int64_t NB = R / n;
-  const ColPartition part = col_partition(n, r, store4, mode, C, NB);
+  const ColPartition part = col_partition(n, r, store4, mode, C, NB, elem_bytes);
   return (NB + part.tb0 - 1) / part.tb0;
 }
 

@@ -41,10 +41,11 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
                        size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out = nullptr,
                        bool stats_cleared = false, hipEvent_t after_stats = nullptr, float* colsum_partial = nullptr);
 // Column sums of the input of a colwise_quant_impl call (the bias gradient when the input is g_y):
-// with colsum_partial the call also writes colsum_strips_impl(...) rows of C partial sums (fp32, one
+// with colsum_partial the call also writes colsum_strips_impl(...) rows of C partial sums (fp32; elem_bytes
+// = size of an input element, on which the partition of the passes depends; one
 // row per run of token blocks of its statistics pass, which holds the sum of every block as
 // coefficient 0); colsum_finish_impl adds the rows in a fixed order and rounds once to the output type.
-int64_t colsum_strips_impl(int64_t R, int64_t C, int n, int r, int store4, int mode);
+int64_t colsum_strips_impl(int64_t R, int64_t C, int n, int r, int store4, int mode, int elem_bytes);
 int colsum_finish_impl(const float* partial, int64_t strips, int64_t C, void* out, int out_dtype, hipStream_t st);
 size_t colwise_workspace_bytes_impl(int64_t C);
 size_t colwise_stats_bytes_impl(int64_t C);  // leading part of the workspace that must be zero before the statistics pass
