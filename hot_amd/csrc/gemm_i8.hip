@@ -717,17 +717,28 @@ static int pick_tile(GemmArgs& g, hipStream_t st) {
     case 22: return launch_gemm<2, 2, BITS, OutT>(g, st);
     default: break;
   }
-  // 128 x 128 tiles by default.  With more tiles than CUs, three LDS stages let three workgroups
-  // share a CU and hide each other's stalls; with fewer, a lone workgroup per CU prefers the deeper
-  // prefetch of four stages.  Problems with at least two full rounds of 256 x 256 tiles take those:
-  // half the operand traffic per multiply-add.  The DMA kernel addresses operands with 32-bit
+  // 128 x 128 tiles (three or four LDS stages: with more tiles than CUs three workgroups share a
+  // CU and hide each other's stalls; with fewer, a lone workgroup prefers the deeper prefetch) or
+  // 256 x 256 tiles (one workgroup per CU, half the operand traffic per multiply-add, but 10 us of
+  // fill and epilogue per tile that nothing overlaps).  The choice follows the measured time of a
+  // tile as a function of K, times the rounds of 256 tiles a launch needs:
+  //   128 x 128: INT4 0.9 + 0.0037 K us, INT8 0.5 + 0.0052 K us
+  //   256 x 256: INT4 10 + 0.0131 K us,  INT8 10 + 0.0136 K us
+  // (fitted on 8192..25216 x 768..11008 outputs with K = 768..11008: INT8 operands take the large
+  // tiles from K of about 1100 on, packed INT4 operands only from about 7000 on, and a product of
+  // exactly 256 large tiles beats 1024 small ones).  The DMA kernel addresses operands with 32-bit
   // offsets; larger operands take the register-staged kernel.
   if (g.M * g.lda < (1ll << 32) && g.N * g.ldb < (1ll << 32)) {
     if (g.splits > 1) return launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st);
     const int64_t tiles = ((g.M + 127) / 128) * ((g.N + 127) / 128);
     const int64_t big = ((g.M + 255) / 256) * ((g.N + 255) / 256);
-    if (big >= 512) return launch_gemm_pipe<4, 4, BITS, 4, OutT>(g, st);
-    return tiles > 256 ? launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st) : launch_gemm_pipe<2, 2, BITS, 4, OutT>(g, st);
+    const double k = (double)g.ktiles * (double)G_BK;   // codes along K
+    const double t_small = (BITS == 4 ? 0.9 + 0.0037 * k : 0.5 + 0.0052 * k) * (double)((tiles + 255) / 256);
+    const double t_big = (10.0 + (BITS == 4 ? 0.0131 : 0.0136) * k) * (double)((big + 255) / 256);
+    if (big >= 256 && t_big < t_small) return launch_gemm_pipe<4, 4, BITS, 4, OutT>(g, st);
+    // three stages (three workgroups per CU) pay for packed INT4 operands only: INT8 stages are twice
+    // as many bytes per multiply-add and the deeper ring measured 2-12 % faster there
+    return (tiles > 256 && BITS == 4) ? launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st) : launch_gemm_pipe<2, 2, BITS, 4, OutT>(g, st);
   }
   return launch_gemm<2, 2, BITS, OutT>(g, st);
 }
