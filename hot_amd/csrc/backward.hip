@@ -321,8 +321,12 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
                         s2 == st && b.split_bytes ? ws + b.off_split : nullptr, s2 == st ? b.split_bytes : 0);
   };
   if (hq_aside) {
-    rc = check_hip(hipStreamWaitEvent(side->stream, side->fork2, 0), "hipStreamWaitEvent");   // statistics are in
+    // The statistics pass on the main stream feeds the row-wise quantiser only when it delivers the
+    // fused absmax; with per-token steps (or an absmax pass of its own) the row-wise kernel starts
+    // at once, beside the statistics pass.  The partial column sums always come from that pass.
+    if (fuse) rc = check_hip(hipStreamWaitEvent(side->stream, side->fork2, 0), "hipStreamWaitEvent");
     if (!rc) rc = quantise_gy_rows(side->stream);
+    if (!rc && gb && !fuse) rc = check_hip(hipStreamWaitEvent(side->stream, side->fork2, 0), "hipStreamWaitEvent");
     if (!rc) rc = finish_bias(side->stream);
     if (!rc && gx_aside) rc = gemm_gx(side->stream);
     if (rc) return rc;
