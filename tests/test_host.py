@@ -199,3 +199,11 @@ def test_library_argument_checks_need_no_gpu():
     assert lib.hot_backward_workspace_bytes(12608, 3072, 768, C.byref(cfg)) == 0
     with pytest.raises(_lib.HotError):
         _lib.check(-2)
+
+
+def test_bench_refuses_more_than_one_gpu():
+    """Every box has one GPU: the benchmark says so instead of running a second rank."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True)
+    assert r.returncode != 0 and "ONE GPU" in r.stderr and r.stdout.strip() == ""
