@@ -19,6 +19,7 @@ Prints ONE JSON line.  Besides the contract fields it carries
                 (oracle/fakequant_port.py) on the same layer, on the host cores
   kernels       per-kernel microseconds and achieved rates for this layer
   llama_gate_up the same step at the Llama-7B gate/up shape (reported only)
+  quantiser_grid the same step over bits x rounding x step granularity x low-rank setting (reported only)
 This run uses one GPU; --gpus above 1 is refused.
 """
 from __future__ import annotations
@@ -248,6 +249,25 @@ def hq_rowwise_sweep(dev):
             "note": "per-token steps, round-to-nearest; includes the Python wrapper (about 14 us floor)"}
 
 
+def quantiser_grid(w, sets, steps=60, warmup=10):
+    """Extra: the same step at the headline shape over the quantiser settings of the g_x path (bits x
+    rounding x step granularity; the g_W path follows rounding and granularity at INT8) and the two
+    low-rank settings; us per layer, inputs rotated as in the headline measurement."""
+    from hot_amd import ops
+    from hot_amd.hadamard_matmul import hla_rows, paper_rows
+    L = sets[0][1].shape[0]
+    rows = []
+    for hla, (n, sel) in (("n=64 r=36", hla_rows(L)), ("n=16 r=8", paper_rows(16, 8))):
+        for bits in (4, 8):
+            for rnd, rname in ((ops.ROUND_NEAREST, "nearest"), (ops.ROUND_STOCH, "stochastic")):
+                for sc, sname in ((ops.SCALE_TENSOR, "per-tensor"), (ops.SCALE_ROW, "per-token")):
+                    opt = ops.HotOptions(n_o=16, hla_n=int(n), hla_rows=tuple(int(v) for v in sel), gx_bits=bits,
+                                         w_bits=bits, gx_round=rnd, gw_round=rnd, gx_scale=sc, gw_scale=sc, seed=1)
+                    sec, _, _ = step_time(w, sets, opt, steps, warmup)
+                    rows.append([hla, bits, rname, sname, round(sec * 1e6, 1)])
+    return {"columns": ["hla", "gx_bits", "rounding", "steps", "us_per_layer"], "rows": rows}
+
+
 def vit_b16_backward(dev, batch=128, steps=3):
     """Whole-model extra: ViT-B/16 (hot_amd/vit.py, random weights, bf16) on synthetic images, every
     Linear / Conv2d swapped for the HOT layers, quantisers chosen per layer by the calibration pass;
@@ -417,6 +437,10 @@ def main():
             out["hq_rowwise_sweep"] = hq_rowwise_sweep(dev)
         except Exception as e:
             out["hq_rowwise_sweep"] = {"error": repr(e)[:200]}
+        try:
+            out["quantiser_grid"] = quantiser_grid(w, sets)
+        except Exception as e:
+            out["quantiser_grid"] = {"error": repr(e)[:200]}
         try:
             out["vit_b16"] = vit_b16_backward(dev)
         except Exception as e:          # an extra: never costs the headline line
