@@ -154,6 +154,17 @@ def test_vit_fc1_full_size(gpu):
     gi_ref, gw_ref = fq.backward(gy, w, xq, sx, h_out, h_bs, fq.PortConfig())
     assert rel(gx.cpu().numpy(), gi_ref.numpy()) < REL_TOL
     assert rel(gw.cpu().numpy(), gw_ref.numpy()) < REL_TOL
+    # the entry point that also returns the bias gradient: same gradients; on integer-valued g_y the
+    # column sums are exact whatever the order of the additions
+    from hot_amd import ops
+    xq_d, sx_d = ops.abc_forward(x.to(gpu), opt)
+    gx_b, gw_b, gb = ops.linear_backward(gy.to(gpu), w.to(gpu), xq_d, sx_d, opt, bias_grad=True)
+    assert torch.equal(gx_b, gx) and torch.equal(gw_b, gw)
+    ref = gy.double().sum(dim=0)
+    assert float((gb.double().cpu() - ref).abs().max()) <= L * 2.0 ** -24 * float(gy.double().abs().sum(dim=0).max())
+    gi = torch.randint(-8, 9, (L, O), generator=torch.Generator().manual_seed(5)).float()
+    _, _, gbi = ops.linear_backward(gi.to(gpu), w.to(gpu), xq_d, sx_d, opt, bias_grad=True)
+    assert torch.equal(gbi.cpu(), gi.sum(dim=0))
 
 
 @pytest.mark.parametrize("shape", [(8192, 11008, 4096), (8192, 4096, 11008)])
