@@ -629,3 +629,17 @@ def test_hq_linear_scheme_hadamard(gpu, fresh_args, L):
                                  scheme="hadamard")
     assert rel(x.grad.cpu().numpy(), gi_ref.numpy()) < REL_TOL
     assert rel(lin.weight.grad.cpu().numpy(), gw_ref.numpy()) < REL_TOL
+
+
+@pytest.mark.parametrize("variant", [dict(), dict(gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW,
+                                                 gw_round=orc.ROUND_STOCH, gw_scale=orc.SCALE_ROW, seed=3)])
+def test_backward_fp16(gpu, variant):
+    """fp16 tensors (the reference's op dispatches them, cuda_measure/HLQ_backward_kernel.cu:474-515): the
+    codes and steps are those of the oracle on the fp16 values, the outputs its fp32 results rounded once."""
+    L, O, I = 448, 192, 160
+    x, w, gy = make_case(L, O, I, seed=21, dtype=torch.float16)
+    ocfg, opt = both_configs(L, **variant)
+    gx, gw, tr = run_both(x, w, gy, ocfg, opt, gpu)
+    assert gx.dtype == torch.float16 and gw.dtype == torch.float16
+    assert torch.equal(gx.cpu(), torch.from_numpy(tr.g_x).to(torch.float16))
+    assert torch.equal(gw.cpu(), torch.from_numpy(tr.g_w).to(torch.float16))
