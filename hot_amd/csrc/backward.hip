@@ -94,10 +94,9 @@ __global__ void clear3_kernel(uint32_t* p0, int n0, uint32_t* p1, int n1, uint32
 }
 
 static const int32_t* identity_rows() {
-  static int32_t rows[HOT_MAX_HLA_N];
-  static bool init = false;
-  if (!init) { for (int i = 0; i < HOT_MAX_HLA_N; ++i) rows[i] = i; init = true; }
-  return rows;
+  struct Rows { int32_t v[HOT_MAX_HLA_N]; Rows() { for (int i = 0; i < HOT_MAX_HLA_N; ++i) v[i] = i; } };
+  static const Rows rows;   // initialised once, thread-safe
+  return rows.v;
 }
 
 }  // namespace hot
@@ -153,6 +152,23 @@ int hot_gemm_i8(const void* A, int64_t lda, const void* B, int64_t ldb, int bits
                 void* out, int out_dtype, int64_t ldo, int32_t* acc_out, void* hip_stream) {
   return gemm_i8_impl(A, lda, B, ldb, bits, M, N, K, scale_a, a_per_row, scale_b, post_scale, out, out_dtype,
                       ldo, acc_out, (hipStream_t)hip_stream);
+}
+
+int hot_gemm_plan(int64_t M, int64_t N, int64_t K, int bits, int64_t lda, int64_t ldb, size_t workspace_bytes) {
+  return gemm_plan_impl(M, N, K, bits, lda, ldb, workspace_bytes);
+}
+
+size_t hot_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits) {
+  if (bits != 4 && bits != 8) return 0;
+  return gemm_split_plan(M, N, K, bits).ws_bytes;
+}
+
+int hot_gemm_i8_variant(const void* A, int64_t lda, const void* B, int64_t ldb, int bits, int64_t M, int64_t N,
+                        int64_t K, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
+                        void* out, int out_dtype, int64_t ldo, int32_t* acc_out, int variant, void* workspace,
+                        size_t workspace_bytes, void* hip_stream) {
+  return gemm_i8_impl(A, lda, B, ldb, bits, M, N, K, scale_a, a_per_row, scale_b, post_scale, out, out_dtype,
+                      ldo, acc_out, (hipStream_t)hip_stream, workspace, workspace_bytes, variant);
 }
 
 size_t hot_abc_workspace_bytes(int64_t L, int64_t I, const hot_config* cfg) {
@@ -230,6 +246,12 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   if (cfg->gx_scale == HOT_SCALE_SAWB) return fail(HOT_ERR_UNSUPPORTED, "%s: SAWB applies to W and x only", who);
   if (cfg->w_scale == HOT_SCALE_ROW) return fail(HOT_ERR_UNSUPPORTED, "%s: W uses one step per tensor", who);
   if (cfg->gw_scale == HOT_SCALE_SAWB) return fail(HOT_ERR_UNSUPPORTED, "%s: SAWB applies to W and x only", who);
+  // limits of the stages, checked here so that nothing has been launched when one of them refuses
+  if (O % 8 || I % 8) return fail(HOT_ERR_UNSUPPORTED, "%s: O=%lld and I=%lld must be multiples of 8", who, (long long)O, (long long)I);
+  if (O * I * 4 >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "%s: W of %lld x %lld elements exceeds the 32-bit offsets of the loader", who, (long long)O, (long long)I);
+  if (cfg->hla_n <= COL_MAX_N && L * O * 4 >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "%s: g_y of %lld x %lld elements exceeds the 32-bit offsets of the loader", who, (long long)L, (long long)O);
+  if (L >= (1ll << 31)) return fail(HOT_ERR_UNSUPPORTED, "%s: L too large", who);
+  if (((uintptr_t)gy & 15) || ((uintptr_t)w & 15) || ((uintptr_t)xq & 15)) return fail(HOT_ERR_INVALID, "%s: gy, w and xq must be 16-byte aligned", who);
   const BwdLayout b = bwd_layout(L, O, I, cfg);
   if (!workspace || workspace_bytes < b.total) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, b.total, workspace_bytes);
   if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
@@ -276,11 +298,26 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
     side = side_lane_locked();
     if (!side) side_guard.unlock();
   }
+  // Once the side stream has been forked, every way out of this function joins it again: the
+  // caller's stream waits for what the side stream was given, also when a later stage refuses, so
+  // that no kernel of the call still runs (on the workspace) behind work the caller queues next,
+  // and a capture of the caller's stream is never left with an unjoined branch.
+  struct SideJoin {
+    SideLane* side = nullptr;
+    hipStream_t st = nullptr;
+    bool forked = false, joined = false;
+    ~SideJoin() {
+      if (!forked || joined) return;
+      if (hipEventRecord(side->join, side->stream) == hipSuccess) (void)hipStreamWaitEvent(st, side->join, 0);
+    }
+  } side_join;
   int rc = HOT_OK;
   if (side) {
     rc = check_hip(hipEventRecord(side->fork, st), "hipEventRecord");
     if (!rc) rc = check_hip(hipStreamWaitEvent(side->stream, side->fork, 0), "hipStreamWaitEvent");
-    if (!rc) rc = quantise_w(side->stream);
+    if (rc) return rc;
+    side_join.side = side; side_join.st = st; side_join.forked = true;
+    rc = quantise_w(side->stream);
     if (rc) return rc;
   }
   // g_y: HLA along tokens + quantise, transposed (g_W operand); Hadamard along O + quantise (g_x
@@ -349,6 +386,7 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   if (side) {
     rc = check_hip(hipStreamWaitEvent(st, side->join, 0), "hipStreamWaitEvent");
     if (rc) return rc;
+    side_join.joined = true;
   } else {
     rc = quantise_w(st);
     if (rc) return rc;
@@ -396,10 +434,11 @@ int hot_linear_backward(const void* gy, const void* w, int dtype, const void* xq
   const int rc = run_backward_timed(gy, w, dtype, xq, sx, L, O, I, cfg, gx, gw, out_dtype, workspace, workspace_bytes,
                                     k, (hipStream_t)hip_stream);
   if (rc) return rc;
-  times4[0] = k[K_CLEAR] + k[K_GY_STATS] + k[K_GY_HLA] + k[K_GY_HQ];
-  times4[1] = k[K_W_STATS] + k[K_W_QUANT];
-  times4[2] = k[K_GEMM_GX];
-  times4[3] = k[K_GEMM_GW];
+  // the reference op returns {fwht, quant, gemm, dequant} (HLQ_backward_kernel.cu:729-733)
+  times4[0] = k[K_CLEAR] + k[K_GY_STATS] + k[K_W_STATS];          // transform passes that only measure
+  times4[1] = k[K_GY_HLA] + k[K_GY_HQ] + k[K_W_QUANT];            // transform + quantise passes
+  times4[2] = k[K_GEMM_GX] + k[K_GEMM_GW];                        // both GEMMs
+  times4[3] = 0.f;                                                // dequantisation: fused into the GEMMs' epilogues
   return HOT_OK;
 }
 

@@ -23,7 +23,7 @@
 // input (statistics, then quantise): the step of a tensor depends on all of it.
 //
 // HBM traffic per input element: 2 * sizeof(in) read + (r/n) * bits/8 written.
-#include <stdlib.h>
+#include <mutex>
 
 #include "hot_device.h"
 #include "hot_host.h"
@@ -620,13 +620,14 @@ size_t colwise_workspace_bytes_impl(int64_t C) {
 
 template <typename T, int N, int PASS, int ROUND, bool SAWB, typename SEL, int RS = 0>
 static int launch_pass(const ColArgs& a, dim3 grid, size_t lds, hipStream_t st) {
-  static bool attr_done = false;  // one-time, read-only afterwards
-  if (!attr_done && lds > 48 * 1024) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&colwise_kernel<T, N, PASS, ROUND, SAWB, SEL, RS>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-    if (e != hipSuccess) return check_hip(e, "hipFuncSetAttribute(colwise_kernel)");
-    attr_done = true;
-  }
+  // one-time per instantiation; later calls only read the outcome
+  static std::once_flag attr_once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(attr_once, [] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&colwise_kernel<T, N, PASS, ROUND, SAWB, SEL, RS>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+  });
+  if (attr_err != hipSuccess) return check_hip(attr_err, "hipFuncSetAttribute(colwise_kernel)");
   ColArgs b = a;
   b.gx = grid.x; b.gy = grid.y;
   const unsigned total = grid.x * grid.y;
@@ -661,11 +662,6 @@ static ColPartition col_partition(int n, int r, int store4, int mode, int64_t C,
   int tb = BPS;
   while ((tb * r) % (store4 ? 8 : 4) != 0 || run_bytes(tb) < 32) tb <<= 1;
   while (run_bytes(tb) < 128 && wgs(2 * tb) >= 1024 && resident(2 * tb) >= resident(tb)) tb <<= 1;
-  {
-    static int forced = -1;   // experiments: HOT_COL_TB overrides the rule (must keep runs whole dwords)
-    if (forced < 0) { const char* e = getenv("HOT_COL_TB"); forced = e ? atoi(e) : 0; }
-    if (forced > 0 && forced % BPS == 0 && (forced * r) % (store4 ? 8 : 4) == 0) tb = forced;
-  }
   int tb0 = tb;
   if (mode != HOT_SCALE_SAWB)
     while (tb0 > BPS && (tb0 & 1) == 0 && tb0 * n > 64 && wgs(tb0) < 2048) tb0 >>= 1;

@@ -19,8 +19,7 @@
 // Tiling: 256 threads = 2x2 waves; each wave owns (32 WM) x (32 WN) outputs as
 // WM x WN MFMA tiles; K advances 128 codes per stage with the next stage's
 // global loads in flight during the MFMAs (double-buffered LDS).
-#include <stdlib.h>
-
+#include <mutex>
 #include <type_traits>
 #include <utility>
 
@@ -88,9 +87,6 @@ __device__ __forceinline__ void tile_of(const GemmArgs& g, int wg, int& tm, int&
 
 // Rows per group: about the square root of the tiles one XCD holds at a time.
 static int pick_group_m(int tiles_m, int tiles_n, int wgs_per_cu) {
-  static int forced = -1;   // experiments: HOT_GEMM_GROUP_M overrides the rule
-  if (forced < 0) { const char* e = getenv("HOT_GEMM_GROUP_M"); forced = e ? atoi(e) : 0; }
-  if (forced > 0) return forced < tiles_m ? forced : tiles_m;
   const int64_t total = (int64_t)tiles_m * tiles_n;
   int64_t conc = total / 8 < 32 * wgs_per_cu ? total / 8 : 32 * wgs_per_cu;
   if (conc < 1) conc = 1;
@@ -657,23 +653,18 @@ static int launch_gemm(GemmArgs& g, hipStream_t st) {
   g.tiles_n = (int)((g.N + BN - 1) / BN);
   g.group_m = pick_group_m(g.tiles_m, g.tiles_n, 1);
   const size_t lds = (size_t)2 * (BM + BN) * G_PITCH;
-  static bool attr_done = false;  // one-time, read-only afterwards
-  if (!attr_done) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_i8_kernel<WM, WN, BITS, OutT>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return check_hip(e, "hipFuncSetAttribute(gemm_i8_kernel)");
-    attr_done = true;
-  }
+  // one-time per instantiation; later calls only read the outcome
+  static std::once_flag attr_once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(attr_once, [&] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_i8_kernel<WM, WN, BITS, OutT>),
+                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  });
+  if (attr_err != hipSuccess) return check_hip(attr_err, "hipFuncSetAttribute(gemm_i8_kernel)");
   const int64_t total = (int64_t)g.tiles_m * g.tiles_n;
   if (total > (1 << 30)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: too many tiles");
   hipLaunchKernelGGL((gemm_i8_kernel<WM, WN, BITS, OutT>), dim3((unsigned)total), dim3(G_THREADS), lds, st, g);
   return check_launch("gemm_i8_kernel");
-}
-
-static int forced_tile() {   // experiments: HOT_GEMM_TILE picks one kernel variant for every problem
-  static int forced = -1;
-  if (forced < 0) { const char* e = getenv("HOT_GEMM_TILE"); forced = e ? atoi(e) : 0; }
-  return forced;
 }
 
 // Split K when the 128 x 128 tiles cannot fill the chip: up to two workgroups per CU, at least 16
@@ -683,14 +674,11 @@ GemmSplit gemm_split_plan(int64_t M, int64_t N, int64_t K, int bits) {
   if (M <= 0 || N <= 0 || K <= 0) return p;
   const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
   const int64_t stages = round_up(K, GEMM_KTILE) / (bits == 8 ? 64 : 128);
-  static int forced = -1;   // experiments: HOT_GEMM_SPLITK overrides the rule (1 = never split)
-  if (forced < 0) { const char* e = getenv("HOT_GEMM_SPLITK"); forced = e ? atoi(e) : 0; }
   int64_t sk = 1;
   if (tiles < 256) {
     sk = 512 / tiles;                        // about two workgroups per CU
     if (sk > stages / 16) sk = stages / 16;
     if (sk > 8) sk = 8;
-    if (forced > 0) sk = forced;
   }
   if (sk > stages) sk = stages;
   if (sk < 2) return p;
@@ -702,53 +690,52 @@ GemmSplit gemm_split_plan(int64_t M, int64_t N, int64_t K, int bits) {
   return p;
 }
 
+// Which kernel a product takes.  128 x 128 tiles (three or four LDS stages: with more tiles than CUs
+// three workgroups share a CU and hide each other's stalls; with fewer, a lone workgroup prefers the
+// deeper prefetch) or 256 x 256 tiles (one workgroup per CU, half the operand traffic per
+// multiply-add, but 10 us of fill and epilogue per tile that nothing overlaps).  The choice follows
+// the measured time of a tile as a function of K, times the rounds of 256 tiles a launch needs:
+//   128 x 128: INT4 0.9 + 0.0037 K us, INT8 0.5 + 0.0052 K us
+//   256 x 256: INT4 10 + 0.0131 K us,  INT8 10 + 0.0136 K us
+// (fitted on 8192..25216 x 768..11008 outputs with K = 768..11008: INT8 operands take the large
+// tiles from K of about 1100 on, packed INT4 operands only from about 7000 on, and a product of
+// exactly 256 large tiles beats 1024 small ones).  The DMA kernels address operands with 32-bit
+// offsets; larger operands take the register-staged kernel.  With a workspace, products of few
+// tiles and a long K are cut into K ranges.
+int gemm_plan_impl(int64_t M, int64_t N, int64_t K, int bits, int64_t lda, int64_t ldb, size_t ws_bytes) {
+  if (M <= 0 || N <= 0 || K <= 0 || (bits != 4 && bits != 8)) return HOT_GEMM_AUTO;
+  if (M * lda >= (1ll << 32) || N * ldb >= (1ll << 32)) return HOT_GEMM_REG_128;
+  const GemmSplit sp = gemm_split_plan(M, N, K, bits);
+  if (sp.splits > 1 && ws_bytes >= sp.ws_bytes) return HOT_GEMM_DMA_128_SPLITK;
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+  const int64_t big = ((M + 255) / 256) * ((N + 255) / 256);
+  const double k = (double)round_up(K, GEMM_KTILE);   // codes along K
+  const double t_small = (bits == 4 ? 0.9 + 0.0037 * k : 0.5 + 0.0052 * k) * (double)((tiles + 255) / 256);
+  const double t_big = (10.0 + (bits == 4 ? 0.0131 : 0.0136) * k) * (double)((big + 255) / 256);
+  if (big >= 256 && t_big < t_small) return HOT_GEMM_DMA_256_S4;
+  // three stages (three workgroups per CU) pay for packed INT4 operands only: INT8 stages are twice
+  // as many bytes per multiply-add and the deeper ring measured 2-12 % faster there
+  return (tiles > 256 && bits == 4) ? HOT_GEMM_DMA_128_S3 : HOT_GEMM_DMA_128_S4;
+}
+
 template <int BITS, typename OutT>
-static int pick_tile(GemmArgs& g, hipStream_t st) {
-  const int forced = forced_tile();
-  switch (forced) {
-    case 144: return launch_gemm_pipe<4, 4, BITS, 4, OutT>(g, st);
-    case 142: return launch_gemm_pipe<4, 2, BITS, 4, OutT>(g, st);
-    case 124: return launch_gemm_pipe<2, 4, BITS, 4, OutT>(g, st);
-    case 122: return launch_gemm_pipe<2, 2, BITS, 4, OutT>(g, st);
-    case 322: return launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st);
-    case 44: return launch_gemm<4, 4, BITS, OutT>(g, st);
-    case 42: return launch_gemm<4, 2, BITS, OutT>(g, st);
-    case 24: return launch_gemm<2, 4, BITS, OutT>(g, st);
-    case 22: return launch_gemm<2, 2, BITS, OutT>(g, st);
-    default: break;
+static int launch_variant(int variant, GemmArgs& g, hipStream_t st) {
+  switch (variant) {
+    case HOT_GEMM_DMA_128_S3: return launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st);
+    case HOT_GEMM_DMA_128_S4: return launch_gemm_pipe<2, 2, BITS, 4, OutT>(g, st);
+    case HOT_GEMM_DMA_256_S4: return launch_gemm_pipe<4, 4, BITS, 4, OutT>(g, st);
+    case HOT_GEMM_DMA_128_SPLITK: return launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st);
+    case HOT_GEMM_REG_128: return launch_gemm<2, 2, BITS, OutT>(g, st);
+    default: return fail(HOT_ERR_INVALID, "hot_gemm_i8: unknown kernel variant %d", variant);
   }
-  // 128 x 128 tiles (three or four LDS stages: with more tiles than CUs three workgroups share a
-  // CU and hide each other's stalls; with fewer, a lone workgroup prefers the deeper prefetch) or
-  // 256 x 256 tiles (one workgroup per CU, half the operand traffic per multiply-add, but 10 us of
-  // fill and epilogue per tile that nothing overlaps).  The choice follows the measured time of a
-  // tile as a function of K, times the rounds of 256 tiles a launch needs:
-  //   128 x 128: INT4 0.9 + 0.0037 K us, INT8 0.5 + 0.0052 K us
-  //   256 x 256: INT4 10 + 0.0131 K us,  INT8 10 + 0.0136 K us
-  // (fitted on 8192..25216 x 768..11008 outputs with K = 768..11008: INT8 operands take the large
-  // tiles from K of about 1100 on, packed INT4 operands only from about 7000 on, and a product of
-  // exactly 256 large tiles beats 1024 small ones).  The DMA kernel addresses operands with 32-bit
-  // offsets; larger operands take the register-staged kernel.
-  if (g.M * g.lda < (1ll << 32) && g.N * g.ldb < (1ll << 32)) {
-    if (g.splits > 1) return launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st);
-    const int64_t tiles = ((g.M + 127) / 128) * ((g.N + 127) / 128);
-    const int64_t big = ((g.M + 255) / 256) * ((g.N + 255) / 256);
-    const double k = (double)g.ktiles * (double)G_BK;   // codes along K
-    const double t_small = (BITS == 4 ? 0.9 + 0.0037 * k : 0.5 + 0.0052 * k) * (double)((tiles + 255) / 256);
-    const double t_big = (10.0 + (BITS == 4 ? 0.0131 : 0.0136) * k) * (double)((big + 255) / 256);
-    if (big >= 256 && t_big < t_small) return launch_gemm_pipe<4, 4, BITS, 4, OutT>(g, st);
-    // three stages (three workgroups per CU) pay for packed INT4 operands only: INT8 stages are twice
-    // as many bytes per multiply-add and the deeper ring measured 2-12 % faster there
-    return (tiles > 256 && BITS == 4) ? launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st) : launch_gemm_pipe<2, 2, BITS, 4, OutT>(g, st);
-  }
-  return launch_gemm<2, 2, BITS, OutT>(g, st);
 }
 
 template <int BITS>
-static int dispatch_out(int out_dtype, GemmArgs& g, hipStream_t st) {
+static int dispatch_out(int out_dtype, int variant, GemmArgs& g, hipStream_t st) {
   switch (out_dtype) {
-    case HOT_F32: return pick_tile<BITS, float>(g, st);
-    case HOT_BF16: return pick_tile<BITS, bf16_t>(g, st);
-    case HOT_F16: return pick_tile<BITS, f16_t>(g, st);
+    case HOT_F32: return launch_variant<BITS, float>(variant, g, st);
+    case HOT_BF16: return launch_variant<BITS, bf16_t>(variant, g, st);
+    case HOT_F16: return launch_variant<BITS, f16_t>(variant, g, st);
     default: return fail(HOT_ERR_INVALID, "hot_gemm_i8: bad out dtype %d", out_dtype);
   }
 }
@@ -756,7 +743,7 @@ static int dispatch_out(int out_dtype, GemmArgs& g, hipStream_t st) {
 int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bits, int64_t M, int64_t N,
                  int64_t K, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
                  void* out, int out_dtype, int64_t ldo, int32_t* acc_out, hipStream_t st, void* split_ws,
-                 size_t split_ws_bytes) {
+                 size_t split_ws_bytes, int variant) {
   if (!A || !B || !scale_a || !scale_b || !out) return fail(HOT_ERR_INVALID, "hot_gemm_i8: null pointer");
   if (M < 0 || N < 0 || K <= 0) return fail(HOT_ERR_INVALID, "hot_gemm_i8: bad shape %lld x %lld x %lld", (long long)M, (long long)N, (long long)K);
   if (bits != 4 && bits != 8) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: bits=%d (4 or 8)", bits);
@@ -768,7 +755,13 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
   if (ldo < N) return fail(HOT_ERR_INVALID, "hot_gemm_i8: ldo=%lld < N", (long long)ldo);
   if (bits == 4 && K > (int64_t)(0x7FFFFFFF / (112 * 112))) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: K too large for the scaled INT4 accumulator");
   if (bits == 8 && K > (int64_t)(0x7FFFFFFF / (127 * 127))) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: K too large for int32 accumulation");
+  if (variant < HOT_GEMM_AUTO || variant >= HOT_GEMM_VARIANTS) return fail(HOT_ERR_INVALID, "hot_gemm_i8: unknown kernel variant %d", variant);
   if (M == 0 || N == 0) return HOT_OK;
+  const size_t ws_have = split_ws ? split_ws_bytes : 0;
+  if (variant == HOT_GEMM_AUTO) variant = gemm_plan_impl(M, N, K, bits, lda, ldb, ws_have);
+  const bool small_ptrs = M * lda < (1ll << 32) && N * ldb < (1ll << 32);
+  if (variant != HOT_GEMM_REG_128 && !small_ptrs)
+    return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: operands of 4 GiB or more take the register-staged kernel only");
   GemmArgs g;
   g.A = (const uint8_t*)A; g.B = (const uint8_t*)B; g.lda = lda; g.ldb = ldb; g.M = M; g.N = N;
   g.ktiles = (int)(kpad / G_BK);
@@ -777,13 +770,15 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
   g.vec_out = ((ldo & 3) == 0 && ((uintptr_t)out & 15) == 0) ? 1 : 0;
   g.vec16 = (((uintptr_t)out & 15) == 0 && ((ldo * (out_dtype == HOT_F32 ? 4 : 2)) & 15) == 0) ? 1 : 0;
   g.splits = 1; g.partials = nullptr;
-  const GemmSplit plan = gemm_split_plan(M, N, K, bits);
-  if (plan.splits > 1 && split_ws && split_ws_bytes >= plan.ws_bytes && M * lda < (1ll << 32) && N * ldb < (1ll << 32) &&
-      forced_tile() == 0) {
+  if (variant == HOT_GEMM_DMA_128_SPLITK) {
+    const GemmSplit plan = gemm_split_plan(M, N, K, bits);
+    if (plan.splits < 2) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: the split-K kernel needs a product of fewer than 256 tiles of 128 x 128 and a long K");
+    if (ws_have < plan.ws_bytes) return fail(HOT_ERR_WORKSPACE, "hot_gemm_i8: split-K workspace of %zu bytes needed, %zu given", plan.ws_bytes, ws_have);
+    if ((uintptr_t)split_ws & 15) return fail(HOT_ERR_INVALID, "hot_gemm_i8: workspace must be 16-byte aligned");
     g.splits = plan.splits;
     g.partials = (v4i*)split_ws;
   }
-  return bits == 4 ? dispatch_out<4>(out_dtype, g, st) : dispatch_out<8>(out_dtype, g, st);
+  return bits == 4 ? dispatch_out<4>(out_dtype, variant, g, st) : dispatch_out<8>(out_dtype, variant, g, st);
 }
 
 }  // namespace hot

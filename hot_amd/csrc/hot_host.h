@@ -63,7 +63,9 @@ size_t hla_workspace_bytes_impl(int64_t R, int64_t C, int n, int r);
 int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bits, int64_t M, int64_t N,
                  int64_t K, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
                  void* out, int out_dtype, int64_t ldo, int32_t* acc_out, hipStream_t st, void* split_ws = nullptr,
-                 size_t split_ws_bytes = 0);
+                 size_t split_ws_bytes = 0, int variant = HOT_GEMM_AUTO);
+// The hot_gemm_variant that gemm_i8_impl picks for a product when `ws_bytes` of workspace come with it.
+int gemm_plan_impl(int64_t M, int64_t N, int64_t K, int bits, int64_t lda, int64_t ldb, size_t ws_bytes);
 
 // Split-K plan of gemm_i8_impl for a problem: `splits` K ranges (1 = none) and the bytes of workspace
 // that hold their partial accumulators (16-byte aligned; contents need no initialisation).

@@ -150,8 +150,8 @@ def hla_tokenwise(x: torch.Tensor, n: int, rows: Sequence[int], bits: int = 8, r
     mode = _SCALE[scale]
     codes = torch.empty((Cc, ld), dtype=torch.int8, device=x.device)
     scales = torch.empty((Cc if mode == SCALE_ROW else 1,), dtype=torch.float32, device=x.device)
-    ws = _ws(_lib.lib().hot_hla_workspace_bytes(R, Cc, n, r), x.device)
     rows_c = (C.c_int32 * r)(*[int(v) for v in rows])
+    ws = _ws(_lib.lib().hot_hla_workspace_bytes(R, Cc, n, r), x.device)
     _lib.check(_lib.lib().hot_hla_tokenwise(x.data_ptr(), _dt(x), R, Cc, n, rows_c, r, bits, _ROUND[rounding], seed,
                                             rng_stream, mode, codes.data_ptr(), ld, scales.data_ptr(),
                                             ws.data_ptr(), ws.numel(), _stream()))
@@ -173,11 +173,20 @@ def wq_colwise(w: torch.Tensor, n: int = 16, bits: int = 4, rounding="nearest", 
     return codes, scales
 
 
+def gemm_plan(M: int, N: int, k: int, bits: int, lda: Optional[int] = None, ldb: Optional[int] = None,
+              workspace_bytes: int = 0) -> int:
+    """The kernel variant (enum hot_gemm_variant) the library runs for this product."""
+    pitch = kpad(k) * bits // 8
+    return int(_lib.lib().hot_gemm_plan(M, N, k, bits, lda or pitch, ldb or pitch, int(workspace_bytes)))
+
+
 def gemm_i8(a: torch.Tensor, b: torch.Tensor, k: int, bits: int, scale_a: torch.Tensor, scale_b: torch.Tensor,
-            post_scale: float = 1.0, out_dtype=torch.float32, return_acc: bool = False):
+            post_scale: float = 1.0, out_dtype=torch.float32, return_acc: bool = False,
+            variant: Optional[int] = None):
     """out[M,N] = ((A . B^T) * scale_a) * scale_b * post_scale on K-major codes.
     a [M, lda bytes], b [N, ldb bytes] int8 tensors whose rows hold k codes of
-    `bits` bits, zero-padded to kpad(k)."""
+    `bits` bits, zero-padded to kpad(k).  `variant` (enum hot_gemm_variant) names the kernel
+    (hot_gemm_i8_variant, with the workspace the variant asks for); None = hot_gemm_i8."""
     _need_gpu_2d(a, "A")
     _need_gpu_2d(b, "B")
     M, N = a.shape[0], b.shape[0]
@@ -186,10 +195,20 @@ def gemm_i8(a: torch.Tensor, b: torch.Tensor, k: int, bits: int, scale_a: torch.
     per_row = 1 if scale_a.numel() > 1 else 0
     if per_row and scale_a.numel() != M:
         raise RuntimeError("scale_a must have 1 or M entries")
-    _lib.check(_lib.lib().hot_gemm_i8(a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), bits, M, N, k,
-                                      scale_a.data_ptr(), per_row, scale_b.data_ptr(), float(post_scale),
-                                      out.data_ptr(), _DTYPES[out_dtype], N,
-                                      acc.data_ptr() if acc is not None else None, _stream()))
+    if variant is None:
+        _lib.check(_lib.lib().hot_gemm_i8(a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), bits, M, N, k,
+                                          scale_a.data_ptr(), per_row, scale_b.data_ptr(), float(post_scale),
+                                          out.data_ptr(), _DTYPES[out_dtype], N,
+                                          acc.data_ptr() if acc is not None else None, _stream()))
+    else:
+        need = int(_lib.lib().hot_gemm_workspace_bytes(M, N, k, bits))
+        ws = _ws(need, a.device) if need else None
+        _lib.check(_lib.lib().hot_gemm_i8_variant(a.data_ptr(), a.stride(0), b.data_ptr(), b.stride(0), bits, M, N, k,
+                                                  scale_a.data_ptr(), per_row, scale_b.data_ptr(), float(post_scale),
+                                                  out.data_ptr(), _DTYPES[out_dtype], N,
+                                                  acc.data_ptr() if acc is not None else None, int(variant),
+                                                  ws.data_ptr() if ws is not None else None,
+                                                  ws.numel() if ws is not None else 0, _stream()))
     return (out, acc) if return_acc else out
 
 

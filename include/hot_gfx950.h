@@ -41,7 +41,7 @@
 extern "C" {
 #endif
 
-#define HOT_ABI_VERSION 2
+#define HOT_ABI_VERSION 3
 #define HOT_API __attribute__((visibility("default")))
 
 enum hot_status {
@@ -98,7 +98,7 @@ HOT_API int64_t hot_kpad(int64_t k);
 /*
  * Block-Hadamard along the contiguous dimension + absmax step + quantise.
  *   in          device, [M, K] row-major, dtype
- *   n           Hadamard block, 16 | 32 | 64; K % n == 0
+ *   n           Hadamard block, a power of two 1 .. 64; K % n == 0 and K % 8 == 0
  *   bits        4: codes_out is [M, K/2] bytes, element 2j in bits 3:0 of byte j
  *               8: codes_out is [M, K] int8
  *   scale_mode  HOT_SCALE_TENSOR -> scales_out[1]; HOT_SCALE_ROW -> scales_out[M]
@@ -164,10 +164,13 @@ HOT_API int hot_abc_forward(const void* x, int dtype, int64_t L, int64_t I, cons
 /*
  * The fused backward: g_x[L, I] and g_W[O, I] (both of out_dtype, dense).
  *   gy [L, O], w [O, I] of dtype; xq / sx as written by hot_abc_forward
- *   times4      host, NULL or 4 floats receiving the seconds spent in
- *               {transform+quantise of g_y (both operands), transform+quantise
- *               of W, g_x GEMM+dequant, g_W GEMM+dequant}; non-NULL makes the
- *               call synchronise the stream
+ *   times4      host, NULL or 4 floats in the order of the reference op's time
+ *               vector {fwht, quant, gemm, dequant} (HLQ_backward_kernel.cu:729-733):
+ *               seconds spent in {the transform passes that only measure (statistics
+ *               of g_y and W), the transform+quantise passes (g_y twice, W), both
+ *               GEMMs, 0: dequantisation is the GEMMs' epilogue}; non-NULL makes
+ *               the call synchronise the stream and run its kernels one after the
+ *               other on `hip_stream`
  * Without timing, independent kernels of the call (the two W kernels, the row-wise
  * quantise pass of g_y and, for products too small to fill the chip, the g_x GEMM) run
  * on a side stream of the library (one per device, created on first use, default
@@ -206,6 +209,39 @@ HOT_API int hot_linear_backward_bias(const void* gy, const void* w, int dtype, c
  * reference (its CUTLASS GEMMs run without split-K, HLQ_backward_kernel.cu:236-250).
  */
 HOT_API int hot_gemm_splits(int64_t M, int64_t N, int64_t K, int bits);
+
+/*
+ * Kernel variants of the integer GEMM.  hot_gemm_i8 and the GEMMs inside hot_linear_backward pick
+ * one per product (hot_gemm_plan tells which); hot_gemm_i8_variant runs a named one, so that tests
+ * and measurements can cover every kernel whatever the rule picks.  The reference has no
+ * counterpart: its two CUTLASS instantiations are fixed at compile time
+ * (cuda_measure/HLQ_backward_kernel.cu:181-280,309-384).
+ */
+enum hot_gemm_variant {
+  HOT_GEMM_AUTO = 0,           /* let the library choose                                        */
+  HOT_GEMM_DMA_128_S3 = 1,     /* 128 x 128 tiles, operands HBM -> LDS directly, ring of 3 stages */
+  HOT_GEMM_DMA_128_S4 = 2,     /* the same with 4 stages                                        */
+  HOT_GEMM_DMA_256_S4 = 3,     /* 256 x 256 tiles, ring of 4 stages                             */
+  HOT_GEMM_REG_128 = 4,        /* 128 x 128 tiles staged through registers (operands >= 4 GiB)  */
+  HOT_GEMM_DMA_128_SPLITK = 5, /* 128 x 128 tiles, K cut into ranges + reduce kernel; needs a
+                                  workspace of hot_gemm_workspace_bytes                         */
+  HOT_GEMM_VARIANTS = 6
+};
+/* The variant hot_gemm_i8 (workspace_bytes = 0) or a GEMM inside hot_linear_backward
+ * (workspace_bytes = what the call can spare) runs for this product; lda, ldb in bytes. */
+HOT_API int hot_gemm_plan(int64_t M, int64_t N, int64_t K, int bits, int64_t lda, int64_t ldb,
+                          size_t workspace_bytes);
+/* Workspace with which the split-K variant runs for this product (0: it does not apply). */
+HOT_API size_t hot_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K, int bits);
+/* hot_gemm_i8 with the kernel named by `variant` (HOT_GEMM_AUTO: the library's choice given the
+ * workspace); `workspace` may be NULL for the variants that need none.  A variant that does not
+ * apply to the product (split-K without a long K, a DMA kernel on operands of 4 GiB or more) is
+ * refused with HOT_ERR_UNSUPPORTED. */
+HOT_API int hot_gemm_i8_variant(const void* A, int64_t lda, const void* B, int64_t ldb, int bits,
+                        int64_t M, int64_t N, int64_t K, const float* scale_a, int a_per_row,
+                        const float* scale_b, float post_scale, void* out, int out_dtype,
+                        int64_t ldo, int32_t* acc_out, int variant, void* workspace,
+                        size_t workspace_bytes, void* hip_stream);
 
 /*
  * hot_linear_backward with a HIP event after every kernel group; synchronises

@@ -318,18 +318,117 @@ def test_gemm_i8_epilogues(gpu, out_dtype, bits, M, N, K, per_row):
     assert torch.equal(out.cpu(), torch.from_numpy(ref.astype(np.float32)).to(out_dtype))
 
 
-@pytest.mark.parametrize("bits", [4, 8])
-def test_gemm_i8_large_tiles(gpu, bits):
-    """Enough 256 x 256 tiles for the large-tile kernel (20 x 26 of them, ragged on both edges)."""
-    from hot_amd import ops
-    M, N, K = 5000, 6600, 192
+def exact_acc(a, b):
+    """int32 accumulators of A . B^T through BLAS: float32 while every partial sum stays below 2^24
+    (then each addition is exact), float64 otherwise."""
+    bound = int(np.abs(a).max()) * int(np.abs(b).max()) * a.shape[1]
+    dt = np.float32 if bound < 2 ** 24 else np.float64
+    return np.rint(a.astype(dt) @ b.astype(dt).T).astype(np.int64).astype(np.int32)
+
+
+def dequant_ref(acc, sa, sb, post):
+    """The epilogue, operation for operation: ((float(acc) * s_a[row]) * s_b) * post."""
+    return ((acc.astype(np.float32) * np.asarray(sa, np.float32).reshape(-1, 1)).astype(np.float32)
+            * np.float32(sb)).astype(np.float32) * np.float32(post)
+
+
+# (variant name, bits, M, N, K): shapes ragged on both edges of the variant's own tile, K not a
+# multiple of the K tile; the split-K kernel needs fewer than 256 tiles and at least 32 stages.
+VARIANT_CASES = [
+    ("GEMM_DMA_128_S3", 8, 515, 390, 1000), ("GEMM_DMA_128_S3", 4, 515, 390, 1000),
+    ("GEMM_DMA_128_S4", 8, 515, 390, 1000), ("GEMM_DMA_128_S4", 4, 515, 390, 1000),
+    ("GEMM_DMA_128_S3", 8, 130, 72, 100), ("GEMM_DMA_128_S4", 4, 1, 1, 16),          # shorter than the ring is deep
+    ("GEMM_DMA_256_S4", 8, 700, 530, 600), ("GEMM_DMA_256_S4", 4, 700, 530, 600),
+    ("GEMM_DMA_256_S4", 8, 257, 255, 100), ("GEMM_DMA_256_S4", 4, 300, 100, 3000),
+    ("GEMM_REG_128", 8, 515, 390, 1000), ("GEMM_REG_128", 4, 515, 390, 1000), ("GEMM_REG_128", 8, 77, 130, 90),
+    ("GEMM_DMA_128_SPLITK", 8, 260, 200, 2500), ("GEMM_DMA_128_SPLITK", 4, 260, 200, 5000),
+    ("GEMM_DMA_128_SPLITK", 8, 1000, 900, 2100),
+]
+
+
+@pytest.mark.parametrize("name,bits,M,N,K", VARIANT_CASES)
+def test_gemm_every_variant_exact(gpu, name, bits, M, N, K):
+    """Every GEMM kernel by name (hot_gemm_i8_variant): int32 accumulators bit-exact, and the
+    dequantised output (the other store path: no int32 side output) equal to the epilogue formula."""
+    from hot_amd import _lib, ops
+    variant = getattr(_lib, name)
+    a, b = rand_codes(M, K, bits, 31), rand_codes(N, K, bits, 32)
+    kp = ops.kpad(K)
+    rng = np.random.default_rng(33)
+    sa = rng.uniform(1e-4, 2e-4, size=M).astype(np.float32)
+    sb = rng.uniform(1e-3, 2e-3, size=1).astype(np.float32)
+    A, B = to_operand(a, bits, kp).to(gpu), to_operand(b, bits, kp).to(gpu)
+    acc_ref = exact_acc(a, b)
+    assert np.array_equal(acc_ref, orc.int_gemm_nt(a, b))
+    out, acc = ops.gemm_i8(A, B, K, bits, torch.from_numpy(sa).to(gpu), torch.from_numpy(sb).to(gpu), post_scale=1 / 16,
+                           return_acc=True, variant=variant)
+    ref = dequant_ref(acc_ref, sa, sb[0], 1 / 16)
+    assert np.array_equal(acc.cpu().numpy(), acc_ref)
+    assert np.array_equal(out.cpu().numpy(), ref)
+    for dt in (torch.float32, torch.bfloat16):
+        out2 = ops.gemm_i8(A, B, K, bits, torch.from_numpy(sa).to(gpu), torch.from_numpy(sb).to(gpu), post_scale=1 / 16,
+                           out_dtype=dt, variant=variant)
+        assert torch.equal(out2.cpu(), torch.from_numpy(ref).to(dt))
+
+
+@pytest.mark.parametrize("bits,M,N,K,expect", [
+    (8, 4000, 4090, 2048, "GEMM_DMA_256_S4"),      # 16 x 16 large tiles, ragged on both edges
+    (4, 4000, 4090, 8192, "GEMM_DMA_256_S4"),
+    (4, 5000, 6600, 192, "GEMM_DMA_128_S3"),       # short K: many small tiles, three workgroups per CU
+    (8, 5000, 6600, 192, "GEMM_DMA_128_S4"),
+    (8, 384, 256, 4000, "GEMM_DMA_128_S4"),        # few tiles, no workspace: one deep-ring workgroup per tile
+])
+def test_gemm_plan_and_result(gpu, bits, M, N, K, expect):
+    """hot_gemm_i8 picks its kernel by the rule hot_gemm_plan reports; the test names the kernel it
+    means to cover, so a change of the rule cannot silently move it to another one."""
+    from hot_amd import _lib, ops
+    assert ops.gemm_plan(M, N, K, bits) == getattr(_lib, expect)
     a, b = rand_codes(M, K, bits, 21), rand_codes(N, K, bits, 22)
     kp = ops.kpad(K)
     one = torch.ones(1, device=gpu)
-    out = ops.gemm_i8(to_operand(a, bits, kp).to(gpu), to_operand(b, bits, kp).to(gpu), K, bits, one, one,
-                      out_dtype=torch.float32)
-    ref = (a.astype(np.float64) @ b.astype(np.float64).T).astype(np.float32)      # exact: |acc| < 2^24
-    assert np.array_equal(out.cpu().numpy(), ref)
+    A, B = to_operand(a, bits, kp).to(gpu), to_operand(b, bits, kp).to(gpu)
+    acc_ref = exact_acc(a, b)
+    _, acc = ops.gemm_i8(A, B, K, bits, one, one, return_acc=True)
+    assert np.array_equal(acc.cpu().numpy(), acc_ref)
+    sa = torch.full((M,), 2.0 ** -9, device=gpu)
+    out = ops.gemm_i8(A, B, K, bits, sa, one, post_scale=1 / 16, out_dtype=torch.bfloat16)    # the staged epilogue
+    ref = torch.from_numpy(dequant_ref(acc_ref, np.full(M, 2.0 ** -9, np.float32), 1.0, 1 / 16)).to(torch.bfloat16)
+    assert torch.equal(out.cpu(), ref)
+
+
+@pytest.mark.parametrize("bits,M,N,K,expect", [
+    (4, 8192, 4096, 11008, "GEMM_DMA_256_S4"),     # Llama-7B gate/up: g_x
+    (8, 11008, 4096, 4096, "GEMM_DMA_256_S4"),     # Llama-7B gate/up: g_W at the paper rule (L' = 4096)
+    (4, 8192, 11008, 4096, "GEMM_DMA_128_S3"),     # Llama-7B down: g_x (packed INT4, K below the large tiles' break-even)
+    (8, 4096, 11008, 4096, "GEMM_DMA_256_S4"),     # Llama-7B down: g_W
+    (8, 4096, 4096, 4096, "GEMM_DMA_256_S4"),      # Llama-7B q/k/v/o: g_W
+    (4, 8192, 4096, 4096, "GEMM_DMA_256_S4"),      # Llama-7B q/k/v/o: g_x (exactly 256 large tiles)
+])
+def test_gemm_llama_products_sampled_rows_and_columns(gpu, bits, M, N, K, expect):
+    """The products of the Llama-7B shapes, on the kernel the library picks for them (named, so the
+    test cannot drift off it), checked on whole sampled rows and whole sampled columns of the
+    output, so that every output tile is touched: int32 accumulators and the bf16 results bit for bit."""
+    from hot_amd import _lib, ops
+    assert ops.gemm_plan(M, N, K, bits) == getattr(_lib, expect)
+    a, b = rand_codes(M, K, bits, 41), rand_codes(N, K, bits, 42)
+    kp = ops.kpad(K)
+    A, B = to_operand(a, bits, kp).to(gpu), to_operand(b, bits, kp).to(gpu)
+    rng = np.random.default_rng(43)
+    sa = rng.uniform(1e-4, 2e-4, size=M).astype(np.float32)
+    sb = np.float32(1.5e-3)
+    rows = np.unique(np.concatenate([[0, 255, 256, M - 1], rng.integers(0, M, 40)]))
+    cols = np.unique(np.concatenate([[0, 255, 256, N - 1], rng.integers(0, N, 40)]))
+    acc_rows, acc_cols = exact_acc(a[rows], b), exact_acc(a, b[cols])
+    out, acc = ops.gemm_i8(A, B, K, bits, torch.from_numpy(sa).to(gpu), torch.tensor([sb], device=gpu), post_scale=1 / 16,
+                           return_acc=True)
+    acc = acc.cpu().numpy()
+    assert np.array_equal(acc[rows], acc_rows) and np.array_equal(acc[:, cols], acc_cols)
+    del acc
+    out16 = ops.gemm_i8(A, B, K, bits, torch.from_numpy(sa).to(gpu), torch.tensor([sb], device=gpu), post_scale=1 / 16,
+                        out_dtype=torch.bfloat16).cpu()
+    assert torch.equal(out16[rows], torch.from_numpy(dequant_ref(acc_rows, sa[rows], sb, 1 / 16)).to(torch.bfloat16))
+    assert torch.equal(out16[:, cols], torch.from_numpy(dequant_ref(acc_cols, sa, sb, 1 / 16)).to(torch.bfloat16))
+    assert np.array_equal(out.cpu().numpy()[rows], dequant_ref(acc_rows, sa[rows], sb, 1 / 16))
 
 
 def test_gemm_splits_rule():
@@ -341,6 +440,7 @@ def test_gemm_splits_rule():
     assert f(11008, 4096, 4096, 8) == 1
     assert f(256, 256, 128, 8) == 1            # short K
     assert f(256, 256, 2304, 8) == 2
+    assert _lib.lib().hot_gemm_workspace_bytes(256, 256, 2304, 8) == 4 * 2 * 128 * 128 * 4
 
 
 

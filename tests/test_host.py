@@ -68,6 +68,7 @@ def test_transform_dict_caches():
 def fresh_args():
     from hot_amd import args
     saved = {k: getattr(args, k) for k in dir(args) if not k.startswith("_")}
+    args.hot_recipe()          # the module defaults describe a plain layer, as the reference's do
     yield args
     for k, v in saved.items():
         setattr(args, k, v)
@@ -124,7 +125,7 @@ def test_options_follow_args(fresh_args):
         options_for(64)
 
 
-def test_hq_linear_surface_and_no_cpu_fallback():
+def test_hq_linear_surface_and_no_cpu_fallback(fresh_args):
     import torch.nn as nn
     from hot_amd.quant_matmul import FLinearQ, HQ_Linear
     lin = HQ_Linear(48, 64)
@@ -133,6 +134,29 @@ def test_hq_linear_surface_and_no_cpu_fallback():
     assert {"forward", "setup_context", "backward"} <= set(vars(FLinearQ))
     with pytest.raises(RuntimeError):           # the native path refuses CPU tensors, it never falls back
         lin(torch.randn(128, 48))
+    # the module defaults are the reference's: a plain full-precision layer, which runs anywhere
+    fresh_args.plain_recipe()
+    x = torch.randn(128, 48, requires_grad=True)
+    lin(x).sum().backward()
+    assert x.grad is not None and lin.weight.grad.shape == (64, 48)
+
+
+def test_args_defaults_are_the_reference_defaults():
+    """args.py:29-49 of the reference: widths 0, quantisers "no", transforms off, scheme gih_gwlr."""
+    import importlib
+    from hot_amd import args
+    fresh = importlib.reload(args)
+    try:
+        assert (fresh.GogiQuantBit, fresh.weightQuantBit, fresh.GogwQuantBit, fresh.actQuantBit) == (0, 0, 0, 0)
+        assert (fresh.quantBWDGogi, fresh.quantBWDWgt, fresh.quantBWDGogw, fresh.quantBWDAct) == ("no",) * 4
+        assert not (fresh.TransformGogi or fresh.TransformWgt or fresh.TransformGogw or fresh.TransformInput)
+        assert fresh.transform_scheme == "gih_gwlr" and fresh.quantAuto is False and fresh.eps == 1e-11
+        fresh.canonical_recipe()
+        assert (fresh.quantBWDGogi, fresh.quantBWDWgt, fresh.quantBWDGogw, fresh.quantBWDAct) == ("nq", "sawb", "nq", "sawb")
+        assert (fresh.GogiQuantBit, fresh.weightQuantBit, fresh.GogwQuantBit, fresh.actQuantBit) == (4, 4, 8, 8)
+        assert fresh.quantAuto and fresh.TransformGogi and fresh.TransformInput
+    finally:
+        fresh.plain_recipe()
 
 
 def test_replace_layers_style_surgery():
@@ -171,10 +195,14 @@ def test_library_exports_every_declared_symbol():
     lib = C.CDLL(_lib.LIB_PATH)
     for n in names:
         assert hasattr(lib, n), n
-    assert _lib.lib().hot_abi_version() == 2
+    assert _lib.lib().hot_abi_version() == 3
     header = open(os.path.join(ROOT, "include", "hot_gfx950.h")).read()
-    for name in ("HOT_MAX_HLA_N", "HOT_MAX_HLA_BIG", "HOT_HQ_WORKSPACE_BYTES"):     # the binding repeats these constants
+    for name in ("HOT_MAX_HLA_N", "HOT_MAX_HLA_BIG", "HOT_HQ_WORKSPACE_BYTES"):   # the binding repeats these constants
         assert int(re.search(r"#define\s+%s\s+(\d+)" % name, header).group(1)) == getattr(_lib, name)
+    enum = re.search(r"enum hot_gemm_variant \{(.*?)\};", header, re.S).group(1)
+    for name, val in re.findall(r"HOT_(GEMM_\w+)\s*=\s*(\d+)", enum):
+        if name != "GEMM_VARIANTS":
+            assert getattr(_lib, name) == int(val), name
     assert [_lib.lib().hot_kpad(k) for k in (1, 128, 129, 7092)] == [128, 128, 256, 7168]
 
 
@@ -191,6 +219,17 @@ def test_library_argument_checks_need_no_gpu():
     rows = (C.c_int32 * 2)(0, 0)
     assert lib.hot_hla_tokenwise(one, 0, 64, 8, 16, rows, 2, 8, 0, 0, 0, 0, one, 128, one, one, 1 << 30, None) == -1
     assert b"listed twice" in lib.hot_last_error()
+    # the variant query and the named-variant entry point validate before they touch anything
+    assert lib.hot_gemm_plan(12608, 768, 3072, 4, 1536, 1536, 0) == _lib.GEMM_DMA_128_S3
+    assert lib.hot_gemm_plan(3072, 768, 7092, 8, 7168, 7168, 0) == _lib.GEMM_DMA_128_S4
+    assert lib.hot_gemm_plan(3072, 768, 7092, 8, 7168, 7168, 1 << 30) == _lib.GEMM_DMA_128_SPLITK
+    assert lib.hot_gemm_plan(8192, 4096, 11008, 4, 5504, 5504, 0) == _lib.GEMM_DMA_256_S4
+    assert lib.hot_gemm_plan(1 << 20, 128, 8192, 8, 8192, 8192, 0) == _lib.GEMM_REG_128     # A is 8 GiB
+    assert lib.hot_gemm_workspace_bytes(3072, 768, 7092, 8) == 144 * 3 * 128 * 128 * 4
+    assert lib.hot_gemm_i8_variant(one, 128, one, 128, 8, 4, 4, 100, one, 0, one, 1.0, one, 0, 4, None, 99, None, 0, None) == -1
+    assert b"variant" in lib.hot_last_error()
+    assert lib.hot_gemm_i8_variant(one, 128, one, 128, 8, 4, 4, 100, one, 0, one, 1.0, one, 0, 4, None,
+                                   _lib.GEMM_DMA_128_SPLITK, None, 0, None) == -2      # nothing to split
     cfg = ops.HotOptions(hla_n=64, hla_rows=tuple(range(36))).to_c()
     need = lib.hot_backward_workspace_bytes(12608, 3072, 768, C.byref(cfg))
     # packed g_y codes + packed W codes + int8 low-rank g_y codes dominate
