@@ -54,10 +54,13 @@ def backward(Go: torch.Tensor, W: torch.Tensor, X: torch.Tensor, reorder_idx_go=
     """Go [L, O], W [O, I], X [L, I] -> (gx [L, I], gw [O, I], [t0, t1, t2, t3]).
 
     ``reorder_idx_*`` are accepted and ignored, as in the reference (its C++
-    never dereferences them).  time_list = seconds spent in {transform+quantise
-    of Go, transform+quantise of W and X, g_x GEMM+dequantise, g_W
-    GEMM+dequantise}, measured with HIP events on the current stream; their sum
-    is the op's device time."""
+    never dereferences them).  time_list follows the reference's
+    [fwht, quant, gemm, dequant] (HLQ_backward_kernel.cu:729-733) as far as
+    fused kernels allow: seconds spent in {the transform passes that only
+    measure (statistics of Go and W), the transform + quantise passes (Go
+    twice, W, X), both GEMMs, 0.0 -- dequantisation is the GEMMs' epilogue},
+    measured with HIP events on the current stream; their sum is the op's
+    device time."""
     _check(Go, "Go")
     _check(W, "Wt")
     _check(X, "X")

@@ -89,10 +89,16 @@ def select_for_layer(grad: torch.Tensor, bits: int = 4, generator=None):
 
 
 class GradCapture:
-    """Keeps, per hooked layer, the most recent output gradient (and weight) of a backward pass:
-    the role of the reference's tensor dictionary during calibration (ViT_main.py:41-56)."""
+    """Keeps, per hooked layer, the output gradient (and weight) of the FIRST backward pass that
+    reaches it: the role of the reference's tensor dictionary during calibration (ViT_main.py:41-56),
+    whose register() returns early once a slot is filled (utils/plot.py:175-177), so that the
+    selection judges the gradients before any weight update.  ``keep="last"`` keeps the most recent
+    pass instead."""
 
-    def __init__(self, model: nn.Module, layer_types) -> None:
+    def __init__(self, model: nn.Module, layer_types, keep: str = "first") -> None:
+        if keep not in ("first", "last"):
+            raise ValueError("keep must be 'first' or 'last'")
+        self.keep = keep
         self.grads: Dict[str, torch.Tensor] = {}
         self.weights: Dict[str, torch.Tensor] = {}
         self._handles = []
@@ -102,6 +108,8 @@ class GradCapture:
 
     def _hook(self, name, module):
         def fn(_mod, _grad_in, grad_out):
+            if self.keep == "first" and name in self.grads:
+                return
             self.grads[name] = grad_out[0].detach()
             self.weights[name] = module.weight.detach()
         return fn
@@ -121,17 +129,18 @@ def _as_tokens(grad: torch.Tensor) -> torch.Tensor:
 
 
 def calibrate(model: nn.Module, batches: Iterable, criterion: Callable, optimizer: Optional[torch.optim.Optimizer] = None,
-              layer_types=None, bits: int = 4, generator=None) -> Dict[str, str]:
+              layer_types=None, bits: int = 4, generator=None, keep: str = "first") -> Dict[str, str]:
     """Runs the calibration batches through `model` with the HOT path switched off (full-precision
     backward), then fills and returns ``args.layer_quant_dict``.
 
-    `batches` yields (inputs, target) pairs already on the model's device.  The quantiser and
-    transform flags of ``args`` are restored afterwards."""
+    `batches` yields (inputs, target) pairs already on the model's device; the selection judges the
+    gradients of the first batch, as the reference does (``keep="last"``: of the last one).  The
+    quantiser and transform flags of ``args`` are restored afterwards."""
     from .quant_matmul import HQ_Conv2d, HQ_Linear
     layer_types = layer_types or (HQ_Linear, HQ_Conv2d)
     saved = {k: getattr(args, k) for k in ("TransformGogi", "TransformWgt", "TransformGogw", "TransformInput",
                                            "quantBWDGogi", "quantBWDWgt", "quantBWDGogw", "quantBWDAct", "quantAuto")}
-    cap = GradCapture(model, layer_types)
+    cap = GradCapture(model, layer_types, keep)
     try:
         args.TransformGogi = args.TransformWgt = args.TransformGogw = args.TransformInput = False
         args.quantBWDGogi = args.quantBWDWgt = args.quantBWDGogw = args.quantBWDAct = "no"

@@ -139,6 +139,41 @@ def test_backward_against_fakequant_port(gpu):
     assert rel(gw.cpu().numpy(), gw_ref.numpy()) < REL_TOL
 
 
+def test_bf16_inputs_against_the_reference_bf16_evaluation(gpu):
+    """With bf16 weights the reference evaluates the whole backward in bf16 (utils/quant_matmul.py:218-220:
+    H cast to bf16, transform matmuls, quantiser arithmetic and the "integer" matmuls in bf16, whose
+    results are rounded to 8 significant bits); the native path widens the same bf16 inputs to fp32,
+    transforms and quantises in fp32 and accumulates in int32.  The two therefore differ by the
+    reference's own bf16 rounding noise.  Pinned here at the ViT-B fc1 size:
+      * native (fp32 out) is within 1e-3 of the reference's evaluation order run in fp32 on the same
+        bf16 inputs;
+      * the distance native <-> reference-in-bf16 is no larger than the distance of the reference's
+        bf16 evaluation from its own fp32 evaluation (it IS that noise), and stays below 10 %."""
+    from hot_amd import ops
+    L, O, I = 12608, 3072, 768
+    x, w, gy = fq.config1_inputs(L, O, I, seed=0)
+    xb, wb, gb = x.to(torch.bfloat16), w.to(torch.bfloat16), gy.to(torch.bfloat16)
+    ocfg, opt = both_configs(L)
+    xq, sx = ops.abc_forward(xb.to(gpu), opt)
+    gx, gw = ops.linear_backward(gb.to(gpu), wb.to(gpu), xq, sx, opt, out_dtype=torch.float32)
+    gx, gw = gx.cpu().numpy(), gw.cpu().numpy()
+    out = {}
+    for dt in (torch.float32, torch.bfloat16):
+        h_out, h_bs = fq.matrices(L, O, dt)
+        xq_r, sx_r = fq.setup_context(xb.to(dt), h_bs, fq.PortConfig())
+        gi, gwr = fq.backward(gb.to(dt), wb.to(dt), xq_r, sx_r, h_out, h_bs, fq.PortConfig())
+        assert gi.dtype == dt and gwr.dtype == dt
+        out[dt] = (gi.float().numpy(), gwr.float().numpy())
+    d32 = (rel(gx, out[torch.float32][0]), rel(gw, out[torch.float32][1]))
+    d16 = (rel(gx, out[torch.bfloat16][0]), rel(gw, out[torch.bfloat16][1]))
+    own = (rel(out[torch.bfloat16][0], out[torch.float32][0]), rel(out[torch.bfloat16][1], out[torch.float32][1]))
+    print("native vs reference order in fp32: g_x %.2e g_W %.2e; vs its bf16 evaluation: g_x %.2e g_W %.2e; "
+          "reference bf16 vs fp32: g_x %.2e g_W %.2e" % (d32 + d16 + own))
+    assert d32[0] < REL_TOL and d32[1] < REL_TOL
+    assert d16[0] <= own[0] * 1.05 + 1e-3 and d16[1] <= own[1] * 1.05 + 1e-3
+    assert d16[0] < 0.1 and d16[1] < 0.1
+
+
 def test_vit_fc1_full_size(gpu):
     """BASELINE configuration 1 at full size (L = 12608, O = 3072, I = 768):
     bit-exact against the canonical oracle, 1e-3 against the fake-quant port."""
@@ -207,7 +242,9 @@ def test_hlq_backward_op_surface(gpu):
     for per_token in (True, False):
         gx, gw, times = HLQ_backward.backward(Go.to(gpu), W.to(gpu), X.to(gpu), 0, 0, 16, per_token)
         assert gx.shape == (L, I) and gw.shape == (O, I) and gx.dtype == Go.dtype
-        assert isinstance(times, list) and len(times) == 4 and all(isinstance(t, float) and t > 0 for t in times)
+        # [transform-only passes, transform + quantise passes, both GEMMs, 0: dequantisation is fused]
+        assert isinstance(times, list) and len(times) == 4 and all(isinstance(t, float) for t in times)
+        assert all(t > 0 for t in times[:3]) and times[3] == 0.0
         opt = HLQ_backward.options(L, 16, per_token)
         ocfg = orc.HotConfig(n_o=16, hla_n=opt.hla_n, hla_rows=opt.hla_rows, gx_round=orc.ROUND_STOCH,
                              gx_scale=orc.SCALE_ROW if per_token else orc.SCALE_TENSOR, seed=HLQ_backward.seed)
@@ -224,6 +261,7 @@ def test_hlq_backward_op_surface(gpu):
 def fresh_args():
     from hot_amd import args
     saved = {k: getattr(args, k) for k in dir(args) if not k.startswith("_")}
+    args.hot_recipe()          # the module defaults describe a plain layer, as the reference's do
     yield args
     for k, v in saved.items():
         setattr(args, k, v)

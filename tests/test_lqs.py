@@ -17,6 +17,7 @@ from hot_amd import ops
 def fresh_args():
     keys = [k for k in vars(args) if not k.startswith("_") and k not in ("defaultdict",)]
     saved = {k: copy.copy(getattr(args, k)) for k in keys}
+    args.hot_recipe()          # the module defaults describe a plain layer, as the reference's do
     yield args
     for k, v in saved.items():
         setattr(args, k, v)
@@ -192,3 +193,31 @@ def test_calibrate_fills_dict_and_restores_args(fresh_args):
     o = options_for(128, "block.0")
     assert (o.gx_round, o.gx_scale, o.gw_round, o.gw_scale) == (ops.ROUND_STOCH, ops.SCALE_ROW, ops.ROUND_STOCH, ops.SCALE_TENSOR)
     assert o.gw_bits == args.GogiQuantBit       # the reference's g_W branch reads GogiQuantBit under quantAuto
+
+
+def test_calibration_judges_the_first_batch(fresh_args):
+    """The reference's tensor dictionary fills each slot once (utils/plot.py:175-177), so with several
+    calibration batches the selection sees the gradients of the first one, taken before any weight
+    update; keep="last" is the explicit alternative."""
+    torch.manual_seed(1)
+    m = nn.Sequential(nn.Linear(8, 8))
+    hutils.replace_layers(m, nn.Linear, HQ_Linear)
+    hutils.name_layers(m)
+    args.plain_recipe()
+    batches = [torch.randn(16, 8), 100.0 * torch.randn(16, 8)]
+    seen = []
+    for keep in ("first", "last"):
+        cap = lqs.GradCapture(m, (HQ_Linear,), keep=keep)
+        grads = []
+        for b in batches:
+            y = m(b.clone().requires_grad_(True))
+            g = torch.randn_like(y)
+            grads.append(g)
+            y.backward(g)
+        cap.close()
+        (got,) = cap.grads.values()
+        assert torch.equal(got, grads[0] if keep == "first" else grads[1])
+        seen.append(got)
+    assert not torch.equal(seen[0], seen[1])
+    with pytest.raises(ValueError):
+        lqs.GradCapture(m, (HQ_Linear,), keep="middle")
