@@ -22,6 +22,7 @@ SCALE_TENSOR, SCALE_ROW, SCALE_SAWB = 0, 1, 2
 STREAM_GX, STREAM_GW, STREAM_W, STREAM_ACT = 0, 1, 2, 3
 # enum hot_gemm_variant
 GEMM_AUTO, GEMM_DMA_128_S3, GEMM_DMA_128_S4, GEMM_DMA_256_S4, GEMM_REG_128, GEMM_DMA_128_SPLITK = range(6)
+HOT_STATIC_MAX_CHANNELS = 16384
 
 EXPORTS = (
     "hot_last_error", "hot_abi_version", "hot_kpad", "hot_hq_rowwise", "hot_hla_tokenwise",
@@ -29,6 +30,7 @@ EXPORTS = (
     "hot_abc_forward", "hot_backward_workspace_bytes", "hot_linear_backward", "hot_linear_backward_kernels",
     "hot_gemm_splits", "hot_hla_workspace_bytes", "hot_linear_backward_bias",
     "hot_gemm_plan", "hot_gemm_workspace_bytes", "hot_gemm_i8_variant",
+    "hot_hla_tokenwise_static",
 )
 
 
@@ -94,6 +96,9 @@ def _declare(lib):
     lib.hot_gemm_i8_variant.restype = i32
     lib.hot_gemm_i8_variant.argtypes = [vp, i64, vp, i64, i32, i64, i64, i64, vp, i32, vp, fp, vp, i32, i64, vp,
                                         i32, vp, sz, vp]
+    lib.hot_hla_tokenwise_static.restype = i32
+    lib.hot_hla_tokenwise_static.argtypes = [vp, i32, i64, i64, i32, C.POINTER(C.c_int32), i32, i32, i32, u64, u32,
+                                             i32, vp, i64, vp, vp]
     lib.hot_linear_backward_bias.restype = i32
     lib.hot_linear_backward_bias.argtypes = [vp, vp, i32, vp, vp, i64, i64, i64, cfgp, vp, vp, vp, i32, vp, sz, vp]
 

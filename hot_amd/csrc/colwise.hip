@@ -847,4 +847,55 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   }
 }
 
+// ---- the entry point that allocates nothing ---------------------------------------
+//
+// hot_hla_tokenwise needs a workspace (statistics words, per-channel maxima, per-workgroup sums).
+// For callers that cannot allocate one, the same kernels run on a fixed array in device memory
+// that is part of the library's code object: every GPU that loads the library holds one copy of
+// it until the process ends.  Its size fixes the largest channel count the entry point takes.
+constexpr int64_t STATIC_MAX_C = HOT_STATIC_MAX_CHANNELS;
+constexpr size_t STATIC_SCRATCH_BYTES =
+    COL_STAT_BYTES + (size_t)STATIC_MAX_C * 4 * COLMAX_COPIES + (size_t)(2 * sizeof(double)) * 65536;
+static_assert((STATIC_MAX_C * 4 * COLMAX_COPIES) % 256 == 0, "the per-channel maxima end on a 256-byte boundary");
+static __device__ __align__(256) uint8_t scratch[STATIC_SCRATCH_BYTES];
+
+// Device address of `scratch` on the current device.  In host code the array's name is only a
+// handle for the runtime, never an address a kernel could use; the address is asked for once per
+// device (with that device current) and kept.
+static int static_scratch_ptr(uint8_t** out, const char* who) {
+  static std::mutex mu;
+  static uint8_t* ptr[64] = {};
+  int dev = -1;
+  if (int rc = check_hip(hipGetDevice(&dev), "hipGetDevice")) return rc;
+  if (dev < 0 || dev >= 64) return fail(HOT_ERR_UNSUPPORTED, "%s: device index %d outside [0, 64)", who, dev);
+  std::lock_guard<std::mutex> lock(mu);
+  if (!ptr[dev]) {
+    void* p = nullptr;
+    if (int rc = check_hip(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)), "hipGetSymbolAddress(scratch)")) return rc;
+    if (!p || ((uintptr_t)p & 255)) return fail(HOT_ERR_HIP, "%s: the scratch array has no usable device address", who);
+    ptr[dev] = (uint8_t*)p;
+  }
+  *out = ptr[dev];
+  return HOT_OK;
+}
+
 }  // namespace hot
+
+extern "C" int hot_hla_tokenwise_static(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows,
+                                        int r, int bits, int rounding, uint64_t seed, uint32_t rng_stream,
+                                        int scale_mode, void* codes_out, int64_t ld_out, float* scales_out,
+                                        void* hip_stream) {
+  using namespace hot;
+  const char* who = "hot_hla_tokenwise_static";
+  if (n > COL_MAX_N)
+    return fail(HOT_ERR_UNSUPPORTED, "%s: token blocks above %d need a workspace as large as the input; use hot_hla_tokenwise", who, COL_MAX_N);
+  if (C > STATIC_MAX_C)
+    return fail(HOT_ERR_UNSUPPORTED, "%s: %lld channels exceed the %lld the built-in scratch array holds; use hot_hla_tokenwise", who,
+                (long long)C, (long long)STATIC_MAX_C);
+  uint8_t* ws = nullptr;
+  if (int rc = static_scratch_ptr(&ws, who)) return rc;
+  // the statistics words at the head of the array are cleared by the first kernel of the call
+  // (stats_cleared = false), everything else is written before it is read
+  return colwise_quant_impl(in, dtype, R, C, n, rows, r, bits, rounding, seed, rng_stream, scale_mode, codes_out,
+                            ld_out, /*store4=*/0, scales_out, ws, STATIC_SCRATCH_BYTES, (hipStream_t)hip_stream, who);
+}

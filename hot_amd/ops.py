@@ -139,9 +139,10 @@ def hq_rowwise(x: torch.Tensor, n: int = 16, bits: int = 4, rounding="nearest", 
 
 
 def hla_tokenwise(x: torch.Tensor, n: int, rows: Sequence[int], bits: int = 8, rounding="nearest",
-                  scale="tensor", seed: int = 0, rng_stream: int = STREAM_GW):
+                  scale="tensor", seed: int = 0, rng_stream: int = STREAM_GW, static_scratch: bool = False):
     """HLA along dim 0 + quantise, stored transposed.
-    Returns (codes int8 [C, kpad(L')], steps fp32 [1] or [C], L')."""
+    Returns (codes int8 [C, kpad(L')], steps fp32 [1] or [C], L').  With static_scratch the call goes
+    through hot_hla_tokenwise_static: no workspace, the library's built-in scratch array."""
     _need_gpu_2d(x, "input")
     R, Cc = x.shape
     r = len(rows)
@@ -151,6 +152,11 @@ def hla_tokenwise(x: torch.Tensor, n: int, rows: Sequence[int], bits: int = 8, r
     codes = torch.empty((Cc, ld), dtype=torch.int8, device=x.device)
     scales = torch.empty((Cc if mode == SCALE_ROW else 1,), dtype=torch.float32, device=x.device)
     rows_c = (C.c_int32 * r)(*[int(v) for v in rows])
+    if static_scratch:
+        _lib.check(_lib.lib().hot_hla_tokenwise_static(x.data_ptr(), _dt(x), R, Cc, n, rows_c, r, bits,
+                                                       _ROUND[rounding], seed, rng_stream, mode, codes.data_ptr(), ld,
+                                                       scales.data_ptr(), _stream()))
+        return codes, scales, kout
     ws = _ws(_lib.lib().hot_hla_workspace_bytes(R, Cc, n, r), x.device)
     _lib.check(_lib.lib().hot_hla_tokenwise(x.data_ptr(), _dt(x), R, Cc, n, rows_c, r, bits, _ROUND[rounding], seed,
                                             rng_stream, mode, codes.data_ptr(), ld, scales.data_ptr(),

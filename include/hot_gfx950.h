@@ -135,6 +135,24 @@ HOT_API int hot_wq_colwise(const void* in, int dtype, int64_t O, int64_t I, int 
                    void* codes_out, int64_t ld_out, float* scales_out, void* workspace,
                    size_t workspace_bytes, void* hip_stream);
 
+/*
+ * hot_hla_tokenwise without a workspace argument and without any allocation: for callers that
+ * cannot allocate (code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc).  No counterpart in the reference, whose op allocates every intermediate per call
+ * (HLQ_backward_kernel.cu:518-522,557-563).  The kernels' scratch (statistics words, per-channel
+ * maxima, per-workgroup sums: about 1.5 MiB) is a fixed array in the library's device code; each GPU
+ * the library runs on holds it until the process ends.  Limits: C <= HOT_STATIC_MAX_CHANNELS and
+ * n <= 128 (larger blocks need a workspace as large as the input); anything beyond is refused with
+ * HOT_ERR_UNSUPPORTED.  All calls on one GPU share the array: calls that overlap on one GPU (two
+ * streams, two threads) race and must be serialised by the caller.  Same results as
+ * hot_hla_tokenwise, bit for bit.
+ */
+#define HOT_STATIC_MAX_CHANNELS 16384
+HOT_API int hot_hla_tokenwise_static(const void* in, int dtype, int64_t R, int64_t C, int n,
+                             const int32_t* rows, int r, int bits, int rounding, uint64_t seed,
+                             uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_out,
+                             float* scales_out, void* hip_stream);
+
 HOT_API size_t hot_colwise_workspace_bytes(int64_t C);
 /* Workspace of hot_hla_tokenwise for any block size: hot_colwise_workspace_bytes(C)
  * up to 128 tokens, plus an fp32 copy of the input above. */

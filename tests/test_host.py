@@ -197,7 +197,7 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, n), n
     assert _lib.lib().hot_abi_version() == 3
     header = open(os.path.join(ROOT, "include", "hot_gfx950.h")).read()
-    for name in ("HOT_MAX_HLA_N", "HOT_MAX_HLA_BIG", "HOT_HQ_WORKSPACE_BYTES"):   # the binding repeats these constants
+    for name in ("HOT_MAX_HLA_N", "HOT_MAX_HLA_BIG", "HOT_HQ_WORKSPACE_BYTES", "HOT_STATIC_MAX_CHANNELS"):   # the binding repeats these constants
         assert int(re.search(r"#define\s+%s\s+(\d+)" % name, header).group(1)) == getattr(_lib, name)
     enum = re.search(r"enum hot_gemm_variant \{(.*?)\};", header, re.S).group(1)
     for name, val in re.findall(r"HOT_(GEMM_\w+)\s*=\s*(\d+)", enum):
@@ -230,6 +230,10 @@ def test_library_argument_checks_need_no_gpu():
     assert b"variant" in lib.hot_last_error()
     assert lib.hot_gemm_i8_variant(one, 128, one, 128, 8, 4, 4, 100, one, 0, one, 1.0, one, 0, 4, None,
                                    _lib.GEMM_DMA_128_SPLITK, None, 0, None) == -2      # nothing to split
+    # the entry point without a workspace: limits checked before anything else
+    assert lib.hot_hla_tokenwise_static(one, 0, 512, 64, 256, rows, 2, 8, 0, 0, 0, 0, one, 128, one, None) == -2
+    assert lib.hot_hla_tokenwise_static(one, 0, 64, _lib.HOT_STATIC_MAX_CHANNELS + 8, 16, rows, 2, 8, 0, 0, 0, 0, one, 128, one, None) == -2
+    assert b"channels exceed" in lib.hot_last_error()
     cfg = ops.HotOptions(hla_n=64, hla_rows=tuple(range(36))).to_c()
     need = lib.hot_backward_workspace_bytes(12608, 3072, 768, C.byref(cfg))
     # packed g_y codes + packed W codes + int8 low-rank g_y codes dominate
