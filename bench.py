@@ -304,8 +304,9 @@ def vit_b16_backward(dev, batch=128, steps=3):
         return best, best_all
 
     plain, plain_all = backward_ms(model)
-    saved = {k: getattr(args, k) for k in ("batched_mode", "quantAuto")}
+    saved = {k: getattr(args, k) for k in dir(args) if not k.startswith("_") and not callable(getattr(args, k))}
     try:
+        args.hot_recipe(gx="stoch", gw="stoch")
         hutils.replace_layers(model, nn.Conv2d, HQ_Conv2d)
         hutils.replace_layers(model, nn.Linear, HQ_Linear)
         hutils.name_layers(model)

@@ -21,7 +21,8 @@ ROUND_NEAREST, ROUND_STOCH = 0, 1
 SCALE_TENSOR, SCALE_ROW, SCALE_SAWB = 0, 1, 2
 STREAM_GX, STREAM_GW, STREAM_W, STREAM_ACT = 0, 1, 2, 3
 # enum hot_gemm_variant
-GEMM_AUTO, GEMM_DMA_128_S3, GEMM_DMA_128_S4, GEMM_DMA_256_S4, GEMM_REG_128, GEMM_DMA_128_SPLITK = range(6)
+(GEMM_AUTO, GEMM_DMA_128_S3, GEMM_DMA_128_S4, GEMM_DMA_256_S4, GEMM_REG_128, GEMM_DMA_128_SPLITK, GEMM_SLOT_256,
+ GEMM_SLOT_128, GEMM_SLOT_160X256) = range(9)
 HOT_STATIC_MAX_CHANNELS = 16384
 
 EXPORTS = (

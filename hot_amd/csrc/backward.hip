@@ -111,7 +111,9 @@ int64_t hot_kpad(int64_t k) { return round_up(k, GEMM_KTILE); }
 
 int hot_gemm_splits(int64_t M, int64_t N, int64_t K, int bits) {
   if (bits != 4 && bits != 8) return 1;
-  return gemm_split_plan(M, N, K, bits).splits;
+  const GemmSplit sp = gemm_split_plan(M, N, K, bits);
+  const int64_t pitch = round_up(K, GEMM_KTILE) * bits / 8;
+  return gemm_plan_impl(M, N, K, bits, pitch, pitch, sp.ws_bytes) == HOT_GEMM_DMA_128_SPLITK ? sp.splits : 1;
 }
 
 int hot_hq_rowwise(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, int rounding,

@@ -344,14 +344,20 @@ __device__ __forceinline__ void wait_dma() {
   __builtin_amdgcn_s_waitcnt((VM & 0xF) | ((VM >> 4) << 14) | (0x7 << 4) | (0xF << 8));
 }
 
+// s_waitcnt vmcnt(VM) lgkmcnt(0): the DMA wait plus "this wave's LDS reads have all returned"
+template <int VM>
+__device__ __forceinline__ void wait_dma_lds() {
+  __builtin_amdgcn_s_waitcnt((VM & 0xF) | ((VM >> 4) << 14) | (0x7 << 4) | (0x0 << 8));
+}
+
 // vmcnt wait that lets `tiles` (0 .. MAXT) groups of LPW loads stay in flight
-template <int MAXT, int LPW>
+template <int MAXT, int LPW, bool LDS = false>
 __device__ __forceinline__ void wait_dma_upto(int tiles) {
   if constexpr (MAXT <= 0) {
-    wait_dma<0>();
+    if constexpr (LDS) wait_dma_lds<0>(); else wait_dma<0>();
   } else {
-    if (tiles >= MAXT) wait_dma<MAXT * LPW>();
-    else wait_dma_upto<MAXT - 1, LPW>(tiles);
+    if (tiles >= MAXT) { if constexpr (LDS) wait_dma_lds<MAXT * LPW>(); else wait_dma<MAXT * LPW>(); }
+    else wait_dma_upto<MAXT - 1, LPW, LDS>(tiles);
   }
 }
 
@@ -597,6 +603,226 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
   gemm_epilogue<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb);
 }
 
+// ---------------------------------------------------------------------------
+// Slot-scheduled variant.  Same data path as the pipelined kernel above (operand tiles HBM -> LDS by
+// DMA through a ring of S stages, packed INT4 expanded after the fragment read), but the K loop is
+// laid out by hand as a sequence of "slots", one MFMA each, fenced from one another, so that
+// everything else rides in the shadow of the matrix pipe instead of between its blocks:
+//   * the fragment reads of the NEXT round are issued in the first slots of the current round (in
+//     the order the next round first uses them), so they have all returned when it starts;
+//   * packed INT4: the low-nibble operands of the next round are expanded in the second half of the
+//     current round, the high-nibble operands (in place) in the first half of their own round;
+//   * the DMA instructions that refill a stage go out one per slot behind the barrier;
+//   * a stage is refilled as soon as its second round is in registers (S - 1 tiles in flight).
+// The wave grid is GM x GN (2 x 2, 1 x 4 or 4 x 1), a wave owns (32 WM) x (32 WN) outputs, so
+// block tiles of any multiple of 32 rows exist (160 x 256 gives ViT-B's 12608 tokens x 768 one
+// balanced round of 237 tiles on 256 CUs).  A stage holds (BM + BN) / 16 KiB chunks dealt round-
+// robin to the four waves; when that is not a multiple of four the spare DMA slots fetch into a
+// spare KiB, so that every wave issues the same number of loads and one vmcnt serves all.
+// ---------------------------------------------------------------------------
+template <int WM, int WN, int GM, int GN, int BITS, int S, int RB, typename OutT>
+__global__ void __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(1, (WM * WN <= 8 ? 2 : 1))))
+gemm_i8_slot_kernel(const GemmArgs g) {
+  static_assert(GM * GN == 4, "four waves");
+  static_assert(RB == 64 || RB == 128, "stage rows of 64 or 128 bytes");
+  constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN;
+  constexpr int SPR = RB / 16;                      // 16-byte slots per stage row
+  constexpr int RPC = 1024 / RB;                    // rows per KiB chunk (one DMA instruction)
+  constexpr int RPS = RB / 32;                      // rounds per stage: a round consumes 32 bytes of every row
+  constexpr int ROWS = BM + BN, CHUNKS = ROWS / RPC, LPW = (CHUNKS + 3) / 4;
+  constexpr bool SPARE = LPW * 4 != CHUNKS;
+  constexpr int STAGE_BYTES = ROWS * RB;
+  constexpr int RING_BYTES = S * STAGE_BYTES + (SPARE ? 1024 : 0);
+  static_assert(S >= 2 && RING_BYTES <= 160 * 1024, "two or more LDS stages within 160 KiB");
+  constexpr int NF = WM * WN;                       // accumulator fragments per wave
+  constexpr int NM = NF * (BITS == 8 ? 1 : 2);      // MFMAs (slots) per round
+  constexpr int NR = WM + WN;                       // fragment reads per round
+  constexpr int H = NM / 2;                         // slots per half round
+  constexpr int DPS = (LPW + NM - 1) / NM;          // DMA instructions per slot of the refilling round
+  static_assert(NR <= H || BITS == 8, "the reads of a round fit the first half of the round before");
+  __shared__ __attribute__((aligned(1024))) uint8_t ring[RING_BYTES];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / GN, wn = wave % GN;
+  int tm, tn;
+  tile_of(g, (int)blockIdx.x, tm, tn);
+  const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
+  constexpr bool EARLY_SCALES = NF <= 4;
+  float sa_row[WM];
+  float sb = 0.f;
+  if constexpr (EARLY_SCALES) {
+    load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
+    sb = g.scale_b[0];
+  }
+
+  // LDS stage layout: rows of RB bytes = SPR slots of 16 bytes; logical slot s of row r sits at
+  // physical slot s ^ swz(r), swz(r) = (r >> 2) & 3 for 64-byte rows, (r >> 1) & 7 for 128-byte
+  // rows: the fragment reads of 16 consecutive rows (same logical slot) then fall into 16 different
+  // 16-byte bank groups.  DMA instruction i of this wave fills KiB chunk c = 4 i + wave of the
+  // stage: rows RPC c .. RPC c + RPC - 1 (A rows first, then B rows); lane l fills physical slot
+  // l % SPR of row l / SPR of the chunk.  Chunks past the end of the stage go to the spare KiB.
+  uint32_t goff[LPW], ldst[LPW];
+  uint32_t is_b = 0;                                // bit i: instruction i reads B
+#pragma unroll
+  for (int i = 0; i < LPW; ++i) {
+    int c = 4 * i + wave;
+    const bool spare = SPARE && c >= CHUNKS;
+    ldst[i] = spare ? (uint32_t)(S * STAGE_BYTES) : (uint32_t)c * 1024u;
+    if (spare) c = 0;
+    const int r = c * RPC + lane / SPR;
+    const int swz = RB == 64 ? (r >> 2) & 3 : (r >> 1) & 7;
+    const int slot = (lane % SPR) ^ swz;
+    if (c * RPC < BM) {
+      int64_t gr = row0 + r;
+      if (gr >= g.M) gr = g.M - 1;
+      goff[i] = (uint32_t)(gr * g.lda + slot * 16);
+    } else {
+      int64_t gr = col0 + (r - BM);
+      if (gr >= g.N) gr = g.N - 1;
+      goff[i] = (uint32_t)(gr * g.ldb + slot * 16);
+      is_b |= 1u << i;
+    }
+  }
+  is_b = __builtin_amdgcn_readfirstlane(is_b);
+  const uint32_t ring0 = lds_offset(ring);
+  const int KT = g.ktiles * (G_BK * BITS / 8) / RB;               // stages of RB bytes per row
+  auto dma_one = [&](int stage_off, int kt, int i) {
+    const uint8_t* base = ((is_b >> i) & 1u ? g.B : g.A) + (int64_t)kt * RB;
+    const bool spare = SPARE && ldst[i] == (uint32_t)(S * STAGE_BYTES);
+    dma16(ring0 + (spare ? 0u : (uint32_t)stage_off) + ldst[i], goff[i], base);
+  };
+
+  v16i acc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
+
+  // Fragments of two consecutive rounds: fr[p][t], p = parity of the round within its stage, t in the
+  // order of first use by the MFMAs (A fragment 0, the WN B fragments, then A fragments 1 .. WM - 1).
+  // Packed INT4: lo[p][t] holds the low-nibble operands, fr[p][t] turns into the high-nibble operands
+  // in place.  In round d of a stage the lanes of half h (= lane / 32) read logical slot 2 d + h of
+  // their row: 16 int8 codes (one MFMA) or 32 packed INT4 codes (two MFMAs: the low nibbles, then the
+  // high nibbles; both operands alike, so every product pairs equal k).
+  v4i fr[2][NR], lo[2][BITS == 4 ? NR : 1];
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int sw = RB == 64 ? (frow >> 2) & 3 : (frow >> 1) & 7;     // same for rows r and r + 32 k
+  const int offA = (wm * 32 * WM + frow) * RB, offB = (BM + wn * 32 * WN + frow) * RB;
+  auto frag_off = [&](int t) {            // byte offset of fragment t within a stage, without the slot
+    return t == 0 ? offA : (t <= WN ? offB + (t - 1) * 32 * RB : offA + (t - WN) * 32 * RB);
+  };
+  auto read_frag = [&](const uint8_t* stage, int d, int t) {
+    const int so = ((2 * d + fhalf) ^ sw) * 16;
+    fr[d & 1][t] = *reinterpret_cast<const v4i*>(stage + frag_off(t) + so);
+  };
+  auto a_of = [](int i) { return i == 0 ? 0 : WN + i; };   // fragment index of A fragment i
+  auto b_of = [](int j) { return 1 + j; };
+  // MFMA m of a round of parity p
+  auto mfma_slot = [&](int p, int m) {
+    const int mm = m % NF, i = mm / WN, j = mm % WN;
+    if constexpr (BITS == 8) {
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[p][b_of(j)], fr[p][a_of(i)], acc[i][j], 0, 0, 0);
+    } else {
+      if (m < NF) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(lo[p][b_of(j)], lo[p][a_of(i)], acc[i][j], 0, 0, 0);
+      else acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[p][b_of(j)], fr[p][a_of(i)], acc[i][j], 0, 0, 0);
+    }
+  };
+  // dword items [e0, e1) of the expansions of the round of parity p: e = 4 t + dword
+  auto expand_lo = [&](int p, int e0, int e1) {
+#pragma unroll
+    for (int e = e0; e < e1 && e < 4 * NR; ++e) lo[p][e >> 2][e & 3] = (fr[p][e >> 2][e & 3] << 4) & (int)0xF0F0F0F0;
+  };
+  auto expand_hi = [&](int p, int e0, int e1) {
+#pragma unroll
+    for (int e = e0; e < e1 && e < 4 * NR; ++e) fr[p][e >> 2][e & 3] &= (int)0xF0F0F0F0;
+  };
+  constexpr int EPS_ = BITS == 4 ? (4 * NR + H - 1) / H : 0;     // expansion items per slot of a half round
+
+  // prologue: S tiles in flight, tile 0 landed and visible, its first round in registers
+  static_for<S>([&](auto k) {
+    if (k.value < KT) {
+#pragma unroll
+      for (int i = 0; i < LPW; ++i) dma_one(k.value * STAGE_BYTES, k.value, i);
+    }
+  });
+  wait_dma_upto<S - 1, LPW>((KT < S ? KT : S) - 1);
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int t = 0; t < NR; ++t) read_frag(ring, 0, t);
+  if constexpr (BITS == 4) expand_lo(0, 0, 4 * NR);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // One K tile in stage `cur` (tile kt + 1 in `nxt`).  `steady`: every predicate below is true.
+  auto ktile = [&](auto steady, auto cur_off, auto nxt_off, int kt) {
+    constexpr bool ST = decltype(steady)::value;
+    constexpr int CUR = decltype(cur_off)::value, NXT = decltype(nxt_off)::value;
+    const uint8_t* cur = ring + CUR;
+    const uint8_t* nxt = ring + NXT;
+    const bool more = ST || kt + 1 < KT;        // there is a tile kt + 1
+    const bool refill = ST || kt + S < KT;      // ... and a tile kt + S to fetch into this stage
+    static_for<RPS>([&](auto rc) {
+      constexpr int r = decltype(rc)::value, p = r & 1;
+      constexpr bool LAST = r == RPS - 1;
+      if constexpr (LAST) {
+        if (more) {
+          // tile kt + 1 has landed (this wave's share) and this wave's reads of the stage are in ...
+          if constexpr (ST) wait_dma_lds<(S - 2) * LPW>();
+          else wait_dma_upto<S - 2, LPW, true>((kt + S - 1 < KT - 1 ? kt + S - 1 : KT - 1) - (kt + 1));
+          __builtin_amdgcn_s_barrier();         // ... and everybody's: tile kt + 1 is visible, stage `cur` is free
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      // a round: reads of the next round (of this stage, or round 0 of the next tile), the refill of
+      // this stage behind the barrier; INT4: high nibbles of this round, then low nibbles of the next
+      static_for<NM>([&](auto mc) {
+        constexpr int m = decltype(mc)::value;
+        if constexpr (LAST) {
+#pragma unroll
+          for (int i = m * DPS; i < (m + 1) * DPS && i < LPW; ++i)
+            if (refill) dma_one(CUR, kt + S, i);
+        }
+        if constexpr (m < NR) {
+          if constexpr (!LAST) read_frag(cur, r + 1, m);
+          else if (more) read_frag(nxt, 0, m);
+        }
+        if constexpr (BITS == 4) {
+          if constexpr (m < H) expand_hi(p, m * EPS_, (m + 1) * EPS_);
+          else if (!LAST || more) expand_lo(p ^ 1, (m - H) * EPS_, (m - H + 1) * EPS_);
+        }
+        mfma_slot(p, m);
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    });
+  };
+  auto rotation = [&](auto steady, int kt0) {
+    static_for<S>([&](auto k) {
+      constexpr int K = decltype(k)::value;
+      if (decltype(steady)::value || kt0 + K < KT)
+        ktile(steady, std::integral_constant<int, K * STAGE_BYTES>{}, std::integral_constant<int, ((K + 1) % S) * STAGE_BYTES>{},
+              kt0 + K);
+    });
+  };
+  int kt0 = 0;
+  for (; kt0 + 2 * S - 1 < KT; kt0 += S) rotation(std::true_type{}, kt0);   // every tile inside has a tile kt + S
+  for (; kt0 < KT; kt0 += S) rotation(std::false_type{}, kt0);
+
+  if constexpr (!EARLY_SCALES) {
+    load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
+    sb = g.scale_b[0];
+  }
+  constexpr int AREA = 32 * (WN * 32 * (int)sizeof(OutT) + 16);
+  if (4 * AREA <= S * STAGE_BYTES && g.vec16 && !g.acc_out && row0 + BM <= g.M && col0 + BN <= g.N) {
+    __syncthreads();                                     // every wave is done with the ring
+    gemm_epilogue_staged<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb,
+                                             ring + wave * AREA);
+    return;
+  }
+  gemm_epilogue<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb);
+}
+
 // Second kernel of a split-K product: one single-wave workgroup per 32 x 32 accumulator fragment,
 // lane for lane the layout of the pipelined kernel, so each lane adds up the accumulators its twins
 // left in the workspace (integer sums: any order gives the same result) and runs the same epilogue.
@@ -646,6 +872,20 @@ static int launch_gemm_pipe(GemmArgs& g, hipStream_t st) {
   return check_launch("gemm_i8_pipe_kernel");
 }
 
+template <int WM, int WN, int GM, int GN, int BITS, int S, int RB, typename OutT>
+static int launch_gemm_slot(GemmArgs& g, hipStream_t st) {
+  constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN;
+  g.tiles_m = (int)((g.M + BM - 1) / BM);
+  g.tiles_n = (int)((g.N + BN - 1) / BN);
+  g.group_m = pick_group_m(g.tiles_m, g.tiles_n, 1);
+  const int64_t total = (int64_t)g.tiles_m * g.tiles_n;
+  if (total > (1 << 30)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: too many tiles");
+  if (g.M * g.lda >= (1ll << 32) || g.N * g.ldb >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: operand larger than 4 GiB");
+  if (((int64_t)g.ktiles * (G_BK * BITS / 8)) % RB) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: this kernel takes rows of a multiple of %d bytes", RB);
+  hipLaunchKernelGGL((gemm_i8_slot_kernel<WM, WN, GM, GN, BITS, S, RB, OutT>), dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
+  return check_launch("gemm_i8_slot_kernel");
+}
+
 template <int WM, int WN, int BITS, typename OutT>
 static int launch_gemm(GemmArgs& g, hipStream_t st) {
   constexpr int BM = 64 * WM, BN = 64 * WN;
@@ -690,32 +930,46 @@ GemmSplit gemm_split_plan(int64_t M, int64_t N, int64_t K, int bits) {
   return p;
 }
 
-// Which kernel a product takes.  128 x 128 tiles (three or four LDS stages: with more tiles than CUs
-// three workgroups share a CU and hide each other's stalls; with fewer, a lone workgroup prefers the
-// deeper prefetch) or 256 x 256 tiles (one workgroup per CU, half the operand traffic per
-// multiply-add, but 10 us of fill and epilogue per tile that nothing overlaps).  The choice follows
-// the measured time of a tile as a function of K, times the rounds of 256 tiles a launch needs:
-//   128 x 128: INT4 0.9 + 0.0037 K us, INT8 0.5 + 0.0052 K us
-//   256 x 256: INT4 10 + 0.0131 K us,  INT8 10 + 0.0136 K us
-// (fitted on 8192..25216 x 768..11008 outputs with K = 768..11008: INT8 operands take the large
-// tiles from K of about 1100 on, packed INT4 operands only from about 7000 on, and a product of
-// exactly 256 large tiles beats 1024 small ones).  The DMA kernels address operands with 32-bit
-// offsets; larger operands take the register-staged kernel.  With a workspace, products of few
-// tiles and a long K are cut into K ranges.
+// Which kernel a product takes.  Measured time of one round of up to 256 tiles (one per CU) as a
+// function of K, in microseconds, on 8192..25216 x 768..11008 outputs with K = 768..11008:
+//   128 x 128, pipelined, 2-3 workgroups per CU:  INT4 0.9 + 0.0037 K,   INT8 0.5 + 0.0052 K
+//   128 x 128, slot-scheduled, one per CU:        INT4 1.0 + 0.0045 K,   INT8 1.5 + 0.0038 K
+//   256 x 256, slot-scheduled:                    INT4 9 + 0.0108 K,     INT8 9 + 0.0122 K
+//   256 x 256, pipelined:                         INT4 10 + 0.0131 K,    INT8 10 + 0.0136 K
+//   160 x 256, slot-scheduled (INT4):             14.3 + 0.0064 K
+// times the rounds a launch needs.  The 9-14 us of the large tiles are fill and epilogue that a lone
+// workgroup per CU cannot overlap: INT8 operands take them from K of about 1100 on, packed INT4
+// operands only from about 7000 on, and a product of exactly 256 large tiles beats 1024 small ones.
+// Products of at most 256 small tiles with a long K take the slot-scheduled small kernel (one
+// workgroup per CU, four 32 KiB stages) or, when they are few and a workspace is at hand, the
+// split-K pair.  The slot-scheduled kernels stage 128 bytes of every row at a time and take rows of
+// a multiple of 128 bytes only.  The DMA kernels address operands with 32-bit offsets; larger
+// operands take the register-staged kernel.
 int gemm_plan_impl(int64_t M, int64_t N, int64_t K, int bits, int64_t lda, int64_t ldb, size_t ws_bytes) {
   if (M <= 0 || N <= 0 || K <= 0 || (bits != 4 && bits != 8)) return HOT_GEMM_AUTO;
   if (M * lda >= (1ll << 32) || N * ldb >= (1ll << 32)) return HOT_GEMM_REG_128;
-  const GemmSplit sp = gemm_split_plan(M, N, K, bits);
-  if (sp.splits > 1 && ws_bytes >= sp.ws_bytes) return HOT_GEMM_DMA_128_SPLITK;
+  const int64_t kpad = round_up(K, GEMM_KTILE);
+  const bool rows128 = (kpad * bits / 8) % 128 == 0;
   const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
   const int64_t big = ((M + 255) / 256) * ((N + 255) / 256);
-  const double k = (double)round_up(K, GEMM_KTILE);   // codes along K
-  const double t_small = (bits == 4 ? 0.9 + 0.0037 * k : 0.5 + 0.0052 * k) * (double)((tiles + 255) / 256);
-  const double t_big = (10.0 + (bits == 4 ? 0.0131 : 0.0136) * k) * (double)((big + 255) / 256);
-  if (big >= 256 && t_big < t_small) return HOT_GEMM_DMA_256_S4;
-  // three stages (three workgroups per CU) pay for packed INT4 operands only: INT8 stages are twice
-  // as many bytes per multiply-add and the deeper ring measured 2-12 % faster there
-  return (tiles > 256 && bits == 4) ? HOT_GEMM_DMA_128_S3 : HOT_GEMM_DMA_128_S4;
+  const int64_t mid = ((M + 159) / 160) * ((N + 255) / 256);
+  const double k = (double)kpad;   // codes along K
+  const GemmSplit sp = gemm_split_plan(M, N, K, bits);
+  if (sp.splits > 1 && ws_bytes >= sp.ws_bytes && !(rows128 && tiles >= 96)) return HOT_GEMM_DMA_128_SPLITK;
+  if (tiles <= 256) return (rows128 && kpad >= 1024) ? HOT_GEMM_SLOT_128 : HOT_GEMM_DMA_128_S4;
+  auto rounds = [](int64_t t) { return (double)((t + 255) / 256); };
+  int best = bits == 4 ? HOT_GEMM_DMA_128_S3 : HOT_GEMM_DMA_128_S4;
+  double t_best = (bits == 4 ? 0.9 + 0.0037 * k : 0.5 + 0.0052 * k) * rounds(tiles);
+  if (big >= 256) {
+    const double t = rows128 ? (9.0 + (bits == 4 ? 0.0108 : 0.0122) * k) * rounds(big)
+                             : (10.0 + (bits == 4 ? 0.0131 : 0.0136) * k) * rounds(big);
+    if (t < t_best) { t_best = t; best = rows128 ? HOT_GEMM_SLOT_256 : HOT_GEMM_DMA_256_S4; }
+  }
+  if (rows128 && bits == 4 && mid <= 256) {
+    const double t = 14.3 + 0.0064 * k;
+    if (t < t_best) { t_best = t; best = HOT_GEMM_SLOT_160X256; }
+  }
+  return best;
 }
 
 template <int BITS, typename OutT>
@@ -726,6 +980,9 @@ static int launch_variant(int variant, GemmArgs& g, hipStream_t st) {
     case HOT_GEMM_DMA_256_S4: return launch_gemm_pipe<4, 4, BITS, 4, OutT>(g, st);
     case HOT_GEMM_DMA_128_SPLITK: return launch_gemm_pipe<2, 2, BITS, 3, OutT>(g, st);
     case HOT_GEMM_REG_128: return launch_gemm<2, 2, BITS, OutT>(g, st);
+    case HOT_GEMM_SLOT_256: return launch_gemm_slot<4, 4, 2, 2, BITS, 2, 128, OutT>(g, st);
+    case HOT_GEMM_SLOT_128: return launch_gemm_slot<2, 2, 2, 2, BITS, 4, 128, OutT>(g, st);
+    case HOT_GEMM_SLOT_160X256: return launch_gemm_slot<5, 2, 1, 4, BITS, 2, 128, OutT>(g, st);
     default: return fail(HOT_ERR_INVALID, "hot_gemm_i8: unknown kernel variant %d", variant);
   }
 }

@@ -222,8 +222,8 @@ HOT_API int hot_linear_backward_bias(const void* gy, const void* w, int dtype, c
  * Number of K ranges into which the GEMMs inside hot_linear_backward cut a product of
  * M x N outputs over K codes of `bits` bits (1 = one kernel; more = a kernel per range
  * writing int32 partial tiles to the workspace, then a reduce kernel).  Products with
- * few 128 x 128 output tiles and a long K are cut so that the whole chip takes part.
- * hot_gemm_i8 itself has no workspace and never splits.  No counterpart in the
+ * few (below 96) 128 x 128 output tiles and a long K are cut so that the whole chip takes
+ * part.  hot_gemm_i8 itself has no workspace and never splits.  No counterpart in the
  * reference (its CUTLASS GEMMs run without split-K, HLQ_backward_kernel.cu:236-250).
  */
 HOT_API int hot_gemm_splits(int64_t M, int64_t N, int64_t K, int bits);
@@ -243,7 +243,13 @@ enum hot_gemm_variant {
   HOT_GEMM_REG_128 = 4,        /* 128 x 128 tiles staged through registers (operands >= 4 GiB)  */
   HOT_GEMM_DMA_128_SPLITK = 5, /* 128 x 128 tiles, K cut into ranges + reduce kernel; needs a
                                   workspace of hot_gemm_workspace_bytes                         */
-  HOT_GEMM_VARIANTS = 6
+  /* Slot-scheduled kernels: the K loop laid out by hand, one MFMA per slot with the fragment reads,
+     the INT4 expansion and the DMA issue in its shadow; stages of 128 bytes per row (whole cache
+     lines), so they take rows (K codes rounded up to 128, times bits / 8) of a multiple of 128 bytes */
+  HOT_GEMM_SLOT_256 = 6,       /* 256 x 256 tiles, two stages                                   */
+  HOT_GEMM_SLOT_128 = 7,       /* 128 x 128 tiles, four stages, one workgroup per CU            */
+  HOT_GEMM_SLOT_160X256 = 8,   /* 160 x 256 tiles (four waves side by side), two stages         */
+  HOT_GEMM_VARIANTS = 9
 };
 /* The variant hot_gemm_i8 (workspace_bytes = 0) or a GEMM inside hot_linear_backward
  * (workspace_bytes = what the call can spare) runs for this product; lda, ldb in bytes. */

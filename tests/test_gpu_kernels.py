@@ -343,6 +343,13 @@ VARIANT_CASES = [
     ("GEMM_REG_128", 8, 515, 390, 1000), ("GEMM_REG_128", 4, 515, 390, 1000), ("GEMM_REG_128", 8, 77, 130, 90),
     ("GEMM_DMA_128_SPLITK", 8, 260, 200, 2500), ("GEMM_DMA_128_SPLITK", 4, 260, 200, 5000),
     ("GEMM_DMA_128_SPLITK", 8, 1000, 900, 2100),
+    # slot-scheduled kernels: rows of a multiple of 128 bytes (K rounded up to 128 codes, INT4: to 256)
+    ("GEMM_SLOT_256", 8, 700, 530, 600), ("GEMM_SLOT_256", 4, 700, 530, 1000), ("GEMM_SLOT_256", 8, 257, 255, 100),
+    ("GEMM_SLOT_256", 4, 300, 100, 3000), ("GEMM_SLOT_256", 8, 512, 512, 128),
+    ("GEMM_SLOT_128", 8, 515, 390, 1000), ("GEMM_SLOT_128", 4, 515, 390, 1000), ("GEMM_SLOT_128", 8, 130, 72, 100),
+    ("GEMM_SLOT_128", 4, 1, 1, 200), ("GEMM_SLOT_128", 8, 384, 256, 7092),
+    ("GEMM_SLOT_160X256", 8, 700, 530, 600), ("GEMM_SLOT_160X256", 4, 700, 530, 1000), ("GEMM_SLOT_160X256", 4, 161, 257, 2304),
+    ("GEMM_SLOT_160X256", 8, 159, 255, 128), ("GEMM_SLOT_160X256", 4, 1600, 768, 3072),
 ]
 
 
@@ -372,11 +379,14 @@ def test_gemm_every_variant_exact(gpu, name, bits, M, N, K):
 
 
 @pytest.mark.parametrize("bits,M,N,K,expect", [
-    (8, 4000, 4090, 2048, "GEMM_DMA_256_S4"),      # 16 x 16 large tiles, ragged on both edges
-    (4, 4000, 4090, 8192, "GEMM_DMA_256_S4"),
+    (8, 4000, 4090, 2048, "GEMM_SLOT_256"),        # 16 x 16 large tiles, ragged on both edges
+    (4, 4000, 4090, 8192, "GEMM_SLOT_256"),
+    (4, 4000, 4090, 8320, "GEMM_DMA_256_S4"),      # rows of 4160 bytes: not whole 128-byte lines
     (4, 5000, 6600, 192, "GEMM_DMA_128_S3"),       # short K: many small tiles, three workgroups per CU
     (8, 5000, 6600, 192, "GEMM_DMA_128_S4"),
-    (8, 384, 256, 4000, "GEMM_DMA_128_S4"),        # few tiles, no workspace: one deep-ring workgroup per tile
+    (8, 384, 256, 4000, "GEMM_SLOT_128"),          # few tiles, no workspace: one deep-ring workgroup per tile
+    (4, 384, 256, 4200, "GEMM_DMA_128_S4"),        # the same with rows of 2112 bytes
+    (4, 12608, 768, 3072, "GEMM_SLOT_160X256"),    # ViT-B fc1 g_x: one balanced round of 237 tiles
 ])
 def test_gemm_plan_and_result(gpu, bits, M, N, K, expect):
     """hot_gemm_i8 picks its kernel by the rule hot_gemm_plan reports; the test names the kernel it
@@ -397,12 +407,12 @@ def test_gemm_plan_and_result(gpu, bits, M, N, K, expect):
 
 
 @pytest.mark.parametrize("bits,M,N,K,expect", [
-    (4, 8192, 4096, 11008, "GEMM_DMA_256_S4"),     # Llama-7B gate/up: g_x
-    (8, 11008, 4096, 4096, "GEMM_DMA_256_S4"),     # Llama-7B gate/up: g_W at the paper rule (L' = 4096)
-    (4, 8192, 11008, 4096, "GEMM_DMA_128_S3"),     # Llama-7B down: g_x (packed INT4, K below the large tiles' break-even)
-    (8, 4096, 11008, 4096, "GEMM_DMA_256_S4"),     # Llama-7B down: g_W
-    (8, 4096, 4096, 4096, "GEMM_DMA_256_S4"),      # Llama-7B q/k/v/o: g_W
-    (4, 8192, 4096, 4096, "GEMM_DMA_256_S4"),      # Llama-7B q/k/v/o: g_x (exactly 256 large tiles)
+    (4, 8192, 4096, 11008, "GEMM_SLOT_256"),     # Llama-7B gate/up: g_x
+    (8, 11008, 4096, 4096, "GEMM_SLOT_256"),     # Llama-7B gate/up: g_W at the paper rule (L' = 4096)
+    (4, 8192, 11008, 4096, "GEMM_SLOT_256"),     # Llama-7B down: g_x
+    (8, 4096, 11008, 4096, "GEMM_SLOT_256"),     # Llama-7B down: g_W
+    (8, 4096, 4096, 4096, "GEMM_SLOT_256"),      # Llama-7B q/k/v/o: g_W
+    (4, 8192, 4096, 4096, "GEMM_SLOT_256"),      # Llama-7B q/k/v/o: g_x
 ])
 def test_gemm_llama_products_sampled_rows_and_columns(gpu, bits, M, N, K, expect):
     """The products of the Llama-7B shapes, on the kernel the library picks for them (named, so the
@@ -435,7 +445,8 @@ def test_gemm_splits_rule():
     """hot_gemm_splits: products with few output tiles and a long K are cut, others are not."""
     from hot_amd import _lib
     f = _lib.lib().hot_gemm_splits
-    assert f(3072, 768, 7092, 8) == 3          # ViT-B fc1 g_W: 144 tiles
+    assert f(3072, 768, 7092, 8) == 1          # ViT-B fc1 g_W: 144 tiles, one deep-ring workgroup each
+    assert f(768, 768, 7092, 8) == 7           # ViT-B proj g_W: 36 tiles, 112 stages in 7 ranges of 16
     assert f(12608, 768, 3072, 4) == 1         # ViT-B fc1 g_x: 594 tiles
     assert f(11008, 4096, 4096, 8) == 1
     assert f(256, 256, 128, 8) == 1            # short K

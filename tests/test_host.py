@@ -220,12 +220,16 @@ def test_library_argument_checks_need_no_gpu():
     assert lib.hot_hla_tokenwise(one, 0, 64, 8, 16, rows, 2, 8, 0, 0, 0, 0, one, 128, one, one, 1 << 30, None) == -1
     assert b"listed twice" in lib.hot_last_error()
     # the variant query and the named-variant entry point validate before they touch anything
-    assert lib.hot_gemm_plan(12608, 768, 3072, 4, 1536, 1536, 0) == _lib.GEMM_DMA_128_S3
-    assert lib.hot_gemm_plan(3072, 768, 7092, 8, 7168, 7168, 0) == _lib.GEMM_DMA_128_S4
-    assert lib.hot_gemm_plan(3072, 768, 7092, 8, 7168, 7168, 1 << 30) == _lib.GEMM_DMA_128_SPLITK
-    assert lib.hot_gemm_plan(8192, 4096, 11008, 4, 5504, 5504, 0) == _lib.GEMM_DMA_256_S4
+    assert lib.hot_gemm_plan(12608, 768, 3072, 4, 1536, 1536, 0) == _lib.GEMM_SLOT_160X256
+    assert lib.hot_gemm_plan(12608, 768, 2304, 4, 1152, 1152, 0) == _lib.GEMM_DMA_128_S3
+    assert lib.hot_gemm_plan(3072, 768, 7092, 8, 7168, 7168, 0) == _lib.GEMM_SLOT_128
+    assert lib.hot_gemm_plan(3072, 768, 7092, 8, 7168, 7168, 1 << 30) == _lib.GEMM_SLOT_128     # 144 tiles: unsplit
+    assert lib.hot_gemm_plan(768, 768, 7092, 8, 7168, 7168, 1 << 30) == _lib.GEMM_DMA_128_SPLITK # 36 tiles
+    assert lib.hot_gemm_plan(768, 768, 7092, 8, 7168, 7168, 0) == _lib.GEMM_SLOT_128
+    assert lib.hot_gemm_plan(8192, 4096, 11008, 4, 5504, 5504, 0) == _lib.GEMM_SLOT_256
+    assert lib.hot_gemm_plan(8192, 4096, 11136, 4, 5568, 5568, 0) == _lib.GEMM_DMA_256_S4     # rows of 43.5 lines
     assert lib.hot_gemm_plan(1 << 20, 128, 8192, 8, 8192, 8192, 0) == _lib.GEMM_REG_128     # A is 8 GiB
-    assert lib.hot_gemm_workspace_bytes(3072, 768, 7092, 8) == 144 * 3 * 128 * 128 * 4
+    assert lib.hot_gemm_workspace_bytes(3072, 768, 7092, 8) == 144 * 3 * 128 * 128 * 4      # what the split-K variant would take
     assert lib.hot_gemm_i8_variant(one, 128, one, 128, 8, 4, 4, 100, one, 0, one, 1.0, one, 0, 4, None, 99, None, 0, None) == -1
     assert b"variant" in lib.hot_last_error()
     assert lib.hot_gemm_i8_variant(one, 128, one, 128, 8, 4, 4, 100, one, 0, one, 1.0, one, 0, 4, None,
