@@ -17,9 +17,15 @@ Prints ONE JSON line.  Besides the contract fields it carries
                 (hot_linear_backward_kernels), against the chip's published peak
   cpu_baseline  the op-for-op CPU port of the reference's fake-quant path
                 (oracle/fakequant_port.py) on the same layer, on the host cores
+  ceilings      what this box reaches with a plain copy kernel and a loop of INT8 MFMAs
   kernels       per-kernel microseconds and achieved rates for this layer
-  llama_gate_up the same step at the Llama-7B gate/up shape (reported only)
-  quantiser_grid the same step over bits x rounding x step granularity x low-rank setting (reported only)
+  layers        the same step at every ViT-B and Llama-7B layer shape, bf16 and fp32
+  llama_gate_up per-kernel pass at the Llama-7B gate/up shape
+  hq_rowwise_sweep  the row-wise quantise kernel alone over the kernel-level sweep (launches replayed
+                from a HIP graph, so no host time is in the figures)
+  quantiser_grid the step over bits x rounding x step granularity x low-rank setting
+  measure_py    the reference's latency harness (cuda_measure/measure.py) on the drop-in op
+  vit_b16       whole-model backward with every layer swapped
 This run uses one GPU; --gpus above 1 is refused.
 """
 from __future__ import annotations
@@ -67,19 +73,35 @@ def make_layer(L, O, I, dtype, dev, nsets, seed=0):
     return w, sets
 
 
-# HBM bytes per launch of each kernel of the step at the bench workload, from two `rocprofv3 --pmc`
-# runs of this file (FETCH_SIZE, then WRITE_SIZE; KiB per dispatch), each scaled by what the same
-# counter reads for a 512 MiB device copy (FETCH_SIZE reads half the bytes, WRITE_SIZE all of them).
-# Summary and commands: profiles/hot_linear_backward_vit_b_fc1_bf16.hbm_traffic.txt
-MEASURED_TRAFFIC_BYTES = {
-    "gy_stats": (2 * 37911.5 + 19.7) * 1024,
-    "gy_hla_quant": (2 * 37947.0 + 21683.0) * 1024,      # the g_y launches (the trace averages 4 launches on x in)
-    "gy_hq_quant": (2 * 37869.4 + 18912.0) * 1024,
-    "w_stats": (2 * 2333.7 + 4.5) * 1024,
-    "w_quant": (2 * 2363.5 + 1152.0) * 1024,
-    "gemm_gx": (2 * 19683.1 + 18912.0) * 1024,
-    "gemm_gw": (2 * 23058.7 + 27648.0 + 2 * 13862.0 + 4608.0) * 1024,   # K-range kernel + reduce kernel
-}
+def profiled_traffic():
+    """HBM bytes per launch of the kernels of the step at the bench workload, as the committed counter
+    summary gives them (profiles/hot_linear_backward_vit_b_fc1_bf16.hbm_traffic.txt: lines
+    `traffic_bytes <kernel key> <bytes>` and `measured_at <commit>`), or (None, None) when the summary
+    is absent or carries no such lines.  The figures belong to the commit named there: kernels changed
+    since then are listed without traffic."""
+    path = os.path.join(ROOT, "profiles", "hot_linear_backward_vit_b_fc1_bf16.hbm_traffic.txt")
+    table, commit = {}, None
+    try:
+        for line in open(path):
+            f = line.split()
+            if len(f) == 3 and f[0] == "traffic_bytes":
+                table[f[1]] = float(f[2])
+            elif len(f) >= 2 and f[0] == "measured_at":
+                commit = f[1]
+    except OSError:
+        return None, None
+    return (table or None), commit
+
+
+GEMM_VARIANT_NAMES = {1: "gemm_i8_pipe_kernel<128x128, 3 stages>", 2: "gemm_i8_pipe_kernel<128x128, 4 stages>",
+                      3: "gemm_i8_pipe_kernel<256x256, 4 stages>", 4: "gemm_i8_kernel<128x128, register-staged>",
+                      5: "gemm_i8_pipe_kernel<128x128, split K>", 6: "gemm_i8_slot_kernel<256x256>",
+                      7: "gemm_i8_slot_kernel<128x128>", 8: "gemm_i8_slot_kernel<160x256>"}
+
+
+def gemm_kernel_name(M, N, K, bits, with_ws=False):
+    from hot_amd import ops
+    return GEMM_VARIANT_NAMES.get(ops.gemm_plan(M, N, K, bits, workspace_bytes=(1 << 40) if with_ws else 0), "gemm")
 
 
 def kernel_table(w, sets, bufs, opt, ws, iters, warm, traffic=None):
@@ -111,10 +133,9 @@ def kernel_table(w, sets, bufs, opt, ws, iters, warm, traffic=None):
         ("w_stats", "hot::colwise_kernel<.., PASS 0> (W)", us[4], "hbm", O * I * e),
         ("w_quant", "hot::colwise_kernel<.., PASS 1> (W: Hadamard-16 + INT%d, transposed)" % opt.w_bits, us[5], "hbm",
          O * I * e + O * I * opt.w_bits // 8),
-        ("gemm_gx", "hot::gemm_i8_pipe_kernel<.., %d, ..> (g_x)" % opt.gx_bits, us[6], "mfma", 2.0 * L * O * I),
-        ("gemm_gw", "hot::gemm_i8_pipe_kernel<.., 8, ..> (g_W)" + (" in %d K ranges + gemm_i8_reduce_kernel" % gw_splits
-                                                                     if gw_splits > 1 else ""),
-         us[7], "mfma", 2.0 * O * I * lp),
+        ("gemm_gx", "hot::%s INT%d (g_x)" % (gemm_kernel_name(L, I, O, opt.gx_bits), opt.gx_bits), us[6], "mfma", 2.0 * L * O * I),
+        ("gemm_gw", "hot::%s INT8 (g_W)" % gemm_kernel_name(O, I, lp, 8, with_ws=True)
+         + (" in %d K ranges + gemm_i8_reduce_kernel" % gw_splits if gw_splits > 1 else ""), us[7], "mfma", 2.0 * O * I * lp),
     ]
     launches = {"gemm_gw": 2 if gw_splits > 1 else 1, "gemm_gx": 2 if gx_splits > 1 else 1}
     rows = []
@@ -216,37 +237,128 @@ def cpu_baseline(reps=5):
                 host_cpus=os.cpu_count())
 
 
-def hq_rowwise_sweep(dev):
+def hq_rowwise_sweep(dev, reps=20):
     """Kernel-level extra: the fused block-Hadamard + per-token absmax step + quantise kernel alone
     (hot_hq_rowwise, bf16 input with per-channel scales drawn log-uniform in [0.1, 10]), GB/s of
-    algorithmic bytes (input read once + codes + steps written) against the 8 TB/s HBM peak."""
+    algorithmic bytes (input read once + codes + steps written) against the 8 TB/s HBM peak.  `reps`
+    launches are captured into a HIP graph once and replayed between two events, so the figures hold
+    no host-side launch time; two input tensors alternate inside the graph."""
     import torch
-    from hot_amd import ops
+    from hot_amd import _lib, ops
+    lib = _lib.lib()
     rows = []
     g = torch.Generator(device=dev).manual_seed(0)
+    side = torch.cuda.Stream()
     for M in (4096, 16384, 65536):
         for K in (768, 3072, 4096, 11008):
-            x = (torch.randn(M, K, generator=g, device=dev) *
-                 (10.0 ** (torch.rand(K, generator=g, device=dev) * 2 - 1))).to(torch.bfloat16)
+            xs = [(torch.randn(M, K, generator=g, device=dev) *
+                   (10.0 ** (torch.rand(K, generator=g, device=dev) * 2 - 1))).to(torch.bfloat16) for _ in range(2)]
+            scales = torch.empty(M, dtype=torch.float32, device=dev)
             for n in (16, 32, 64):
                 if K % n:
                     continue
                 for bits in (4, 8):
-                    for _ in range(3):
-                        ops.hq_rowwise(x, n=n, bits=bits, scale="row")
+                    codes = torch.empty((M, K * bits // 8), dtype=torch.int8, device=dev)
+
+                    def launch(i, stream):
+                        _lib.check(lib.hot_hq_rowwise(xs[i & 1].data_ptr(), _lib.BF16, M, K, n, bits, ops.ROUND_NEAREST, 0, 0,
+                                                      ops.SCALE_ROW, codes.data_ptr(), scales.data_ptr(), None, 0, stream))
                     torch.cuda.synchronize()
-                    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                    e0.record()
-                    for _ in range(10):
-                        ops.hq_rowwise(x, n=n, bits=bits, scale="row")
-                    e1.record()
-                    torch.cuda.synchronize()
-                    us = e0.elapsed_time(e1) * 100.0
+                    graph = torch.cuda.CUDAGraph()
+                    with torch.cuda.stream(side):
+                        launch(0, side.cuda_stream)
+                        side.synchronize()
+                        with torch.cuda.graph(graph, stream=side):
+                            for i in range(reps):
+                                launch(i, side.cuda_stream)
+                        graph.replay()
+                        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                        e0.record(side)
+                        graph.replay()
+                        e1.record(side)
+                        side.synchronize()
+                    us = e0.elapsed_time(e1) * 1e3 / reps
                     byt = M * K * 2 + M * K * bits // 8 + 4 * M
-                    rows.append([M, K, n, bits, round(us, 1), round(byt / us / 1e3), round(byt / us / 1e3 / HBM_PEAK_GBS, 3)])
-            del x
+                    rows.append([M, K, n, bits, round(us, 2), round(byt / us / 1e3), round(byt / us / 1e3 / HBM_PEAK_GBS, 3)])
+                    del graph
+            del xs
     return {"columns": ["M", "K", "hadamard_block", "bits", "us", "GB/s", "frac_of_8TB/s"], "rows": rows,
-            "note": "per-token steps, round-to-nearest; includes the Python wrapper (about 14 us floor)"}
+            "note": "per-token steps, round-to-nearest; %d launches replayed from a HIP graph between two events" % reps}
+
+
+def layer_table(dev, steps=30, warmup=8):
+    """The step at every layer shape of the ViT-B (batch 64 x 197 tokens, make_WHT rule: n 64, r 36) and
+    Llama-7B (8192 tokens, n 16 / 8 lowest sequencies) configurations, bf16 and fp32, per-tensor steps,
+    round-to-nearest, INT4 g_x / INT8 g_W; beside it the two plain matmuls (g_y @ W, g_y^T @ x) in the
+    same dtype through torch (hipBLASLt), and the forward-side buffer write."""
+    import torch
+    from hot_amd import ops
+    from hot_amd.hadamard_matmul import hla_rows, paper_rows
+    shapes = [("vit_qkv", 12608, 2304, 768), ("vit_proj", 12608, 768, 768), ("vit_fc1", 12608, 3072, 768),
+              ("vit_fc2", 12608, 768, 3072), ("llama_qkvo", 8192, 4096, 4096), ("llama_gate_up", 8192, 11008, 4096),
+              ("llama_down", 8192, 4096, 11008)]
+    rows = []
+    for name, L, O, I in shapes:
+        n, sel = hla_rows(L) if name.startswith("vit") else paper_rows(16, 8)
+        opt = ops.HotOptions(n_o=16, hla_n=int(n), hla_rows=tuple(int(v) for v in sel))
+        for dt, dname in ((torch.bfloat16, "bf16"), (torch.float32, "fp32")):
+            w, sets = make_layer(L, O, I, dt, dev, nsets=3 if name.startswith("vit") else 2, seed=3)
+            sec, bufs, ws = step_time(w, sets, opt, steps, warmup)
+            st = {"i": 0}
+
+            def mm():
+                x, gy = sets[st["i"] % len(sets)]
+                st["i"] += 1
+                torch.matmul(gy, w)
+                torch.matmul(gy.t(), x)
+
+            def fwd():
+                x, _ = sets[st["i"] % len(sets)]
+                st["i"] += 1
+                ops.abc_forward(x, opt)
+            rows.append([name, L, O, I, "n=%d r=%d" % (opt.hla_n, opt.hla_r), dname, round(sec * 1e6, 1),
+                         round(_events(mm, 10, 3), 1), round(_events(fwd, 10, 3), 1)])
+            del w, sets, bufs, ws
+            torch.cuda.empty_cache()
+    return {"columns": ["layer", "L", "O", "I", "hla", "dtype", "hot_backward_us", "two_matmuls_us", "buffer_write_us"],
+            "rows": rows, "note": "%d steps after %d warm-ups, inputs rotated" % (steps, warmup)}
+
+
+def measure_py(dev, trials=100):
+    """The reference's latency harness (cuda_measure/measure.py:35-80) on the drop-in op: L = 49 tokens,
+    O = 3072, I = 768, lognormal(1, 0.1) inputs (numpy seed 2023), `trials` trials, medians.  As there:
+    the plain pair of matmuls by wall clock with device synchronisation, the op by the sum of the stage
+    times it returns (per-token and per-tensor steps); the op's wall clock is reported beside it."""
+    import statistics
+    import numpy as np
+    import torch
+    from hot_amd import HLQ_backward
+    B, O, I = 49, 3072, 768
+    rng = np.random.RandomState(2023)
+    fp, tok, ten, tok_wall, ten_wall = [], [], [], [], []
+    for _ in range(trials):
+        X = torch.tensor(rng.lognormal(1.0, 0.1, B * I).reshape(B, I), dtype=torch.float32).to(dev)
+        Go = torch.tensor(rng.lognormal(1.0, 0.1, B * O).reshape(B, O), dtype=torch.float32).to(dev)
+        W = torch.tensor(rng.lognormal(1.0, 0.1, O * I).reshape(O, I), dtype=torch.float32).to(dev)
+        torch.cuda.synchronize()
+        t0 = time.time()
+        torch.matmul(Go, W)
+        torch.cuda.synchronize()
+        torch.matmul(Go.T, X)
+        torch.cuda.synchronize()
+        fp.append(time.time() - t0)
+        for per_token, acc, wall in ((True, tok, tok_wall), (False, ten, ten_wall)):
+            t0 = time.time()
+            _, _, tl = HLQ_backward.backward(Go, W, X, 0, 0, 16, per_token)
+            torch.cuda.synchronize()
+            wall.append(time.time() - t0)
+            acc.append(sum(tl))
+    med = lambda v: round(statistics.median(v) * 1e6, 1)
+    return {"shape": {"L": B, "O": O, "I": I}, "trials": trials, "unit": "us (medians)",
+            "fp_matmuls_wall": med(fp), "per_token_stage_sum": med(tok), "per_tensor_stage_sum": med(ten),
+            "per_token_wall": med(tok_wall), "per_tensor_wall": med(ten_wall),
+            "note": "stage sums are HIP-event times of the kernels run one after the other, as the op's time list "
+                    "reports them; wall clock adds the Python and launch overhead of one call"}
 
 
 def quantiser_grid(w, sets, steps=60, warmup=10):
@@ -403,8 +515,19 @@ def main():
                    "L": L, "O": O, "I": I, "input_sets_rotated": len(sets)},
     }
     if not a.no_extras:
-        table = kernel_table(w, sets, bufs, opt, ws, iters=20, warm=4, traffic=MEASURED_TRAFFIC_BYTES)
+        traffic, traffic_commit = profiled_traffic()
+        table = kernel_table(w, sets, bufs, opt, ws, iters=20, warm=4, traffic=traffic)
         out["kernels"] = table
+        out["traffic_source"] = ("profiles/hot_linear_backward_vit_b_fc1_bf16.hbm_traffic.txt, rocprofv3 FETCH_SIZE / WRITE_SIZE "
+                                 "at commit %s" % traffic_commit) if traffic else None
+        try:
+            copy_gbs, mfma_tops = ops.measure_ceilings(dev)
+            out["ceilings"] = {"copy_kernel_GBps": round(copy_gbs), "copy_frac_of_8TBps": round(copy_gbs / HBM_PEAK_GBS, 3),
+                               "mfma_int8_loop_TOPs": round(mfma_tops), "mfma_frac_of_5POPs": round(mfma_tops / INT8_PEAK_TOPS, 3),
+                               "note": "plain kernels of the library on this box: 512 MiB device copy (bytes read + written), "
+                                       "loop of independent v_mfma_i32_32x32x32_i8, one wave per SIMD"}
+        except Exception as e:
+            out["ceilings"] = {"error": repr(e)[:200]}
         # Roofline entry: the single launch with the longest duration inside the step, measured with
         # HIP events on the launch stream around every kernel group, the groups launched one after
         # the other (the timed steps above overlap independent kernels on two streams, which
@@ -443,6 +566,11 @@ def main():
                                 "kernels_serial": {r["key"]: [r["us"], r["frac"]] for r in ltable}}
         del lw, lsets, lbufs, lws
     if not a.no_extras and not a.table_only:
+        for key, fn in (("layers", lambda: layer_table(dev)), ("measure_py", lambda: measure_py(dev))):
+            try:
+                out[key] = fn()
+            except Exception as e:          # extras never cost the headline line
+                out[key] = {"error": repr(e)[:200]}
         try:
             out["hq_rowwise_sweep"] = hq_rowwise_sweep(dev)
         except Exception as e:

@@ -31,7 +31,7 @@ EXPORTS = (
     "hot_abc_forward", "hot_backward_workspace_bytes", "hot_linear_backward", "hot_linear_backward_kernels",
     "hot_gemm_splits", "hot_hla_workspace_bytes", "hot_linear_backward_bias",
     "hot_gemm_plan", "hot_gemm_workspace_bytes", "hot_gemm_i8_variant",
-    "hot_hla_tokenwise_static",
+    "hot_hla_tokenwise_static", "hot_measure_ceilings",
 )
 
 
@@ -100,6 +100,8 @@ def _declare(lib):
     lib.hot_hla_tokenwise_static.restype = i32
     lib.hot_hla_tokenwise_static.argtypes = [vp, i32, i64, i64, i32, C.POINTER(C.c_int32), i32, i32, i32, u64, u32,
                                              i32, vp, i64, vp, vp]
+    lib.hot_measure_ceilings.restype = i32
+    lib.hot_measure_ceilings.argtypes = [vp, sz, C.POINTER(C.c_float), C.POINTER(C.c_float), vp]
     lib.hot_linear_backward_bias.restype = i32
     lib.hot_linear_backward_bias.argtypes = [vp, vp, i32, vp, vp, i64, i64, i64, cfgp, vp, vp, vp, i32, vp, sz, vp]
 

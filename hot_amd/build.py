@@ -17,7 +17,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libhot_gfx950.so")
-SOURCES = ["hq_rowwise.hip", "colwise.hip", "hla_big.hip", "gemm_i8.hip", "backward.hip"]
+SOURCES = ["hq_rowwise.hip", "colwise.hip", "hla_big.hip", "gemm_i8.hip", "backward.hip", "ceilings.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -53,7 +53,7 @@ def build(verbose: bool = True, only=None) -> str:
     those and reuses the other object files of an earlier full build: a developer shortcut."""
     todo = [s for s in SOURCES if not only or s in only
             or not os.path.exists(os.path.join(CSRC, s.replace(".hip", ".o")))]
-    with ThreadPoolExecutor(max_workers=min(5, len(SOURCES))) as ex:
+    with ThreadPoolExecutor(max_workers=min(6, len(SOURCES))) as ex:
         list(ex.map(_compile, todo))
     objs = [os.path.join(CSRC, s.replace(".hip", ".o")) for s in SOURCES]
     cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]

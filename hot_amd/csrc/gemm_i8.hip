@@ -945,8 +945,15 @@ GemmSplit gemm_split_plan(int64_t M, int64_t N, int64_t K, int bits) {
 // split-K pair.  The slot-scheduled kernels stage 128 bytes of every row at a time and take rows of
 // a multiple of 128 bytes only.  The DMA kernels address operands with 32-bit offsets; larger
 // operands take the register-staged kernel.
+#ifdef HOT_EXPERIMENTS
+int g_force_variant[2] = {0, 0};   // [INT4, INT8]; 0 = the rule
+extern "C" __attribute__((visibility("default"))) void hot_experiment_force(int bits, int variant) { g_force_variant[bits == 8] = variant; }
+#endif
 int gemm_plan_impl(int64_t M, int64_t N, int64_t K, int bits, int64_t lda, int64_t ldb, size_t ws_bytes) {
   if (M <= 0 || N <= 0 || K <= 0 || (bits != 4 && bits != 8)) return HOT_GEMM_AUTO;
+#ifdef HOT_EXPERIMENTS
+  if (g_force_variant[bits == 8]) return g_force_variant[bits == 8];
+#endif
   if (M * lda >= (1ll << 32) || N * ldb >= (1ll << 32)) return HOT_GEMM_REG_128;
   const int64_t kpad = round_up(K, GEMM_KTILE);
   const bool rows128 = (kpad * bits / 8) % 128 == 0;

@@ -275,3 +275,12 @@ def linear_backward(gy: torch.Tensor, w: torch.Tensor, xq: torch.Tensor, sx: tor
     if timing:
         return gx, gw, [float(t) for t in times]
     return gx, gw
+
+
+def measure_ceilings(device=None):
+    """(copy GB/s, INT8 MFMA TOP/s) of this box from the library's two plain ceiling kernels."""
+    device = device or torch.device("cuda", torch.cuda.current_device())
+    buf = torch.empty(1 << 30, dtype=torch.uint8, device=device)
+    copy, mfma = C.c_float(0), C.c_float(0)
+    _lib.check(_lib.lib().hot_measure_ceilings(buf.data_ptr(), buf.numel(), C.byref(copy), C.byref(mfma), _stream()))
+    return float(copy.value), float(mfma.value)

@@ -284,6 +284,16 @@ HOT_API int hot_linear_backward_kernels(const void* gy, const void* w, int dtype
                                 void* workspace, size_t workspace_bytes, float* times8,
                                 void* hip_stream);
 
+/*
+ * What this box can do at most, from two plain kernels: a device-to-device copy (copy_gbs: bytes read
+ * + bytes written per second, in GB/s) and a loop of independent INT8 MFMAs, one wave per SIMD
+ * (mfma_tops, in TOP/s).  bench.py reports them beside the published peaks.  `scratch`: device
+ * memory, at least 64 MiB (the copy moves its first half onto its second).  Synchronises the stream.
+ * No counterpart in the reference.
+ */
+HOT_API int hot_measure_ceilings(void* scratch, size_t scratch_bytes, float* copy_gbs, float* mfma_tops,
+                         void* hip_stream);
+
 #ifdef __cplusplus
 }
 #endif
