@@ -13,10 +13,16 @@
 //             transform -> natural-order coefficient 64 j + k of the block; kept ones are measured
 //             (statistics pass) or quantised (quantise pass) into codes [L', C]
 //   transpose codes [L', C] -> [C, ld] (K-major for the GEMM), padding zeroed
+// Only the coefficients a kept row needs make the round trip: natural row i of a block is coefficient
+// k = i % 64 of run i / 64, so a k that no kept row has is never written by stage 1 nor read by stage 2
+// (the make_WHT selections keep no odd row: half the traffic).  The row table lives in the workspace
+// and is written by kernels whose arguments carry the rows by value, so the whole call is a sequence
+// of launches: no host-to-device copy, nothing read from host memory after the call returns, and a
+// stream under graph capture records it like any other call.
 // This is the exactness path for large blocks, not a tuned one: the input is read with scalar loads
 // and the coefficients make a round trip through HBM in fp32.
 #include <algorithm>
-#include <vector>
+#include <memory>
 
 #include "hot_device.h"
 #include "hot_host.h"
@@ -35,6 +41,9 @@ struct BigArgs {
   const int32_t* tab;  // per natural row of a block: slot | visit << 16, or -1 when dropped
   int64_t R, C, NB;    // NB = R / n blocks
   int32_t n, r, rpad, bits, rounding, mode;
+  int32_t nk;          // coefficients of a 64-run that some kept row needs
+  uint64_t kmask;      // bit k: coefficient k is one of them
+  uint8_t klist[64];   // the nk set bits of kmask in increasing order
   float* stat;         // [0] absmax, [1] step, [2] clip; the absmax slots from word 64
   float* colmax;       // per-channel absmax (ROW)
   double* partial;     // SAWB: 2 doubles per workgroup
@@ -73,9 +82,10 @@ __global__ void __launch_bounds__(BT) big_stage1_kernel(const BigArgs a) {
 #pragma unroll
   for (int i = 0; i < 64; ++i) v[i] = load_f32<T>(in + (int64_t)i * a.C);
   fwht<64>(v);
-  float* out = a.T + row0 * a.C + c;
+  float* out = a.T + (int64_t)blockIdx.y * a.nk * a.C + c;    // T [run][needed coefficient][channel]
 #pragma unroll
-  for (int i = 0; i < 64; ++i) out[(int64_t)i * a.C] = v[i];
+  for (int i = 0; i < 64; ++i)
+    if ((a.kmask >> i) & 1ull) { *out = v[i]; out += a.C; }
 }
 
 __device__ __forceinline__ float uniform_of(uint64_t e, uint64_t seed, uint32_t stream) {
@@ -87,7 +97,7 @@ __device__ __forceinline__ float uniform_of(uint64_t e, uint64_t seed, uint32_t 
   return r;
 }
 
-// blockIdx.y = block * 64 + k
+// blockIdx.y = block * nk + (index of k among the needed coefficients)
 template <int M, int PASS, int ROUND, bool SAWB>
 __global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
   __shared__ float s_max[BT / 64];
@@ -95,14 +105,15 @@ __global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int64_t c = (int64_t)blockIdx.x * BT + tid;
   const bool active = c < a.C;
-  const int64_t blk = blockIdx.y >> 6;
-  const int k = blockIdx.y & 63;
+  const int64_t blk = blockIdx.y / a.nk;
+  const int kc = (int)(blockIdx.y - blk * a.nk);
+  const int k = a.klist[kc];
   const int qmax = (1 << (a.bits - 1)) - 1;
   float v[M];
   if (active) {
-    const float* t = a.T + (blk * a.n + k) * a.C + c;
+    const float* t = a.T + ((blk * M) * a.nk + kc) * a.C + c;
 #pragma unroll
-    for (int j = 0; j < M; ++j) v[j] = t[(int64_t)j * 64 * a.C];
+    for (int j = 0; j < M; ++j) v[j] = t[(int64_t)j * a.nk * a.C];
   } else {
 #pragma unroll
     for (int j = 0; j < M; ++j) v[j] = 0.f;
@@ -170,10 +181,21 @@ __global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
   }
 }
 
-__global__ void big_clear_kernel(float* stat, float* colmax, int64_t C) {
+__global__ void big_clear_kernel(float* stat, float* colmax, int64_t C, int32_t* tab, int n) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < (int64_t)(STAT_BYTES / 4)) stat[i] = 0.f;
   if (i < C) colmax[i] = 0.f;
+  if (i < n) tab[i] = -1;
+}
+
+// A piece of the row table, carried in the kernel arguments (under the 4 KiB a launch may carry):
+// natural row row[i] of a block is the visit[i]-th kept row in natural order and goes to output
+// coefficient slot[i].
+constexpr int TAB_PIECE = 512;
+struct TabPiece { uint16_t row[TAB_PIECE], visit[TAB_PIECE], slot[TAB_PIECE]; int32_t count; };
+__global__ void big_table_kernel(int32_t* tab, const TabPiece p) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < p.count) tab[p.row[i]] = (int32_t)p.slot[i] | ((int32_t)p.visit[i] << 16);
 }
 
 // statistics -> steps (absmax modes are also read directly by the quantise pass)
@@ -287,20 +309,23 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
   if (!workspace || workspace_bytes < b.total) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, b.total, workspace_bytes);
   if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
   const int64_t gx = (C + BT - 1) / BT;
-  if (NB * 64 > 65535 || R / 64 > 65535 || (scale_mode == HOT_SCALE_SAWB && gx * NB * 64 > 65536))
+  if (R / 64 > 65535 || (scale_mode == HOT_SCALE_SAWB && gx * NB * 64 > 65536))
     return fail(HOT_ERR_UNSUPPORTED, "%s: %lld blocks of %d tokens x %lld channels exceed the grid of the large-block path", who, (long long)NB, n, (long long)C);
 
-  // slot and visit number of every natural row of a block (visit = rank among the kept rows)
-  thread_local std::vector<int32_t> tab;
-  tab.assign((size_t)n, -1);
-  std::vector<int32_t> sorted(rows, rows + r);
+  // visit number of every kept row (rank among the kept rows in natural order) and the coefficients
+  // of a 64-run that the selection needs at all
+  std::unique_ptr<int32_t[]> slot_of(new int32_t[(size_t)n]);
+  std::unique_ptr<int32_t[]> sorted(new int32_t[(size_t)r]);
+  for (int i = 0; i < n; ++i) slot_of[(size_t)i] = -1;
+  uint64_t kmask = 0;
   for (int k = 0; k < r; ++k) {
     if (rows[k] < 0 || rows[k] >= n) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d outside [0, %d)", who, k, rows[k], n);
-    if (tab[(size_t)rows[k]] != -1) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d listed twice", who, k, rows[k]);
-    tab[(size_t)rows[k]] = k;
+    if (slot_of[(size_t)rows[k]] != -1) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d listed twice", who, k, rows[k]);
+    slot_of[(size_t)rows[k]] = k;
+    sorted[(size_t)k] = rows[k];
+    kmask |= 1ull << (rows[k] & 63);
   }
-  std::sort(sorted.begin(), sorted.end());
-  for (int v = 0; v < r; ++v) tab[(size_t)sorted[(size_t)v]] |= v << 16;
+  std::sort(sorted.get(), sorted.get() + r);
 
   uint8_t* ws = (uint8_t*)workspace;
   BigArgs a;
@@ -308,11 +333,30 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
   a.R = R; a.C = C; a.NB = NB; a.n = n; a.r = r; a.rpad = (r + 7) & ~7; a.bits = bits; a.rounding = rounding;
   a.mode = scale_mode; a.stat = (float*)ws; a.colmax = (float*)(ws + b.off_colmax);
   a.partial = (double*)(ws + b.off_partial); a.scales_out = scales_out; a.seed = seed; a.stream = rng_stream;
+  a.kmask = kmask; a.nk = 0;
+  for (int k = 0; k < 64; ++k) {
+    a.klist[k] = 0;
+    if ((kmask >> k) & 1ull) a.klist[a.nk++] = (uint8_t)k;
+  }
+  if (NB * a.nk > 65535) return fail(HOT_ERR_UNSUPPORTED, "%s: %lld blocks of %d tokens exceed the grid of the large-block path", who, (long long)NB, n);
 
-  // the table travels through a staged copy: the call returns once the host buffer has been read
-  if (int rc = check_hip(hipMemcpyAsync(ws + b.off_tab, tab.data(), (size_t)n * 4, hipMemcpyHostToDevice, st), "hipMemcpyAsync(row table)")) return rc;
-  const int64_t nclr = C > (int64_t)(STAT_BYTES / 4) ? C : (int64_t)(STAT_BYTES / 4);
-  hipLaunchKernelGGL(big_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat, a.colmax, C);
+  // statistics and table cleared, then the table written piece by piece (rows in natural order, so
+  // the visit number of a piece's entry i is its position in the sorted list)
+  const int64_t nclr = std::max<int64_t>(std::max<int64_t>(C, n), (int64_t)(STAT_BYTES / 4));
+  hipLaunchKernelGGL(big_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat, a.colmax, C,
+                     (int32_t*)(ws + b.off_tab), n);
+  for (int v0 = 0; v0 < r; v0 += TAB_PIECE) {
+    TabPiece piece;
+    piece.count = std::min(TAB_PIECE, r - v0);
+    for (int i = 0; i < piece.count; ++i) {
+      const int32_t row = sorted[(size_t)(v0 + i)];
+      piece.row[i] = (uint16_t)row;
+      piece.visit[i] = (uint16_t)(v0 + i);
+      piece.slot[i] = (uint16_t)slot_of[(size_t)row];
+    }
+    hipLaunchKernelGGL(big_table_kernel, dim3(TAB_PIECE / 256), dim3(256), 0, st, (int32_t*)(ws + b.off_tab), piece);
+  }
+  if (int rc = check_launch("big_table_kernel")) return rc;
   const dim3 g1((unsigned)gx, (unsigned)(R / 64));
   switch (dtype) {
     case HOT_F32: hipLaunchKernelGGL(big_stage1_kernel<float>, g1, dim3(BT), 0, st, a); break;
@@ -321,9 +365,9 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
     default: return fail(HOT_ERR_INVALID, "%s: bad dtype %d", who, dtype);
   }
   if (int rc = check_launch("big_stage1_kernel")) return rc;
-  const dim3 g2((unsigned)gx, (unsigned)(NB * 64));
+  const dim3 g2((unsigned)gx, (unsigned)(NB * a.nk));
   if (int rc = dispatch_stage2(m, a, g2, 0, st)) return rc;
-  hipLaunchKernelGGL(big_finalize_kernel, dim3(1), dim3(256), 0, st, a, (int64_t)gx * NB * 64, kout);
+  hipLaunchKernelGGL(big_finalize_kernel, dim3(1), dim3(256), 0, st, a, (int64_t)gx * NB * a.nk, kout);
   if (after_stats) (void)hipEventRecord(after_stats, st);
   if (int rc = dispatch_stage2(m, a, g2, 1, st)) return rc;
   const dim3 gt((unsigned)((ld_out + 63) / 64), (unsigned)((C + 63) / 64));

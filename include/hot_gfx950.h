@@ -80,12 +80,11 @@ typedef struct hot_config {
   int32_t gx_scale, w_scale, gw_scale, act_scale;     /* hot_scale_mode           */
   uint64_t seed;    /* stochastic-rounding key                                    */
   const int32_t* hla_rows_big; /* host, hla_r entries: the rows of blocks above
-                                  HOT_MAX_HLA_N tokens (NULL otherwise).  Blocks of
-                                  128 tokens run in the same kernels as smaller
-                                  ones; from 256 on they take a two-level
-                                  transform through an fp32 workspace and a staged
-                                  host-to-device copy of the row table, which
-                                  cannot be graph-captured                       */
+                                  HOT_MAX_HLA_N tokens (NULL otherwise); read
+                                  during the call only.  Blocks of 128 tokens run
+                                  in the same kernels as smaller ones; from 256 on
+                                  they take a two-level transform through an fp32
+                                  workspace (launches only: capturable)          */
 } hot_config;
 
 HOT_API const char* hot_last_error(void);

@@ -467,6 +467,50 @@ def test_backward_in_hip_graph(gpu):
         assert torch.equal(again[0], eager[0]) and torch.equal(again[1], eager[1])
 
 
+def test_backward_large_block_in_hip_graph(gpu):
+    """Token blocks of 1024 (the make_WHT rule on 2048 tokens) take the two-level path, whose row table
+    is written by kernels that carry the rows in their arguments: the call records into a HIP graph like
+    any other, replays equal the eager result and the oracle, also after the host arrays that held the
+    rows during capture are gone and the workspace has been scribbled over."""
+    from hot_amd import ops
+    L, O, I = 2048, 128, 64
+    x, w, gy = make_case(L, O, I, seed=13, dtype=torch.float32)
+    ocfg = orc.HotConfig.python_rule(L)
+    assert ocfg.hla_n == 2048 and len(ocfg.hla_rows) == 528
+    n, rows = orc.hla_rows(1024)
+    ocfg.hla_n, ocfg.hla_rows = n, tuple(int(v) for v in rows)
+    opt = ops.HotOptions(n_o=16, hla_n=n, hla_rows=ocfg.hla_rows)
+    xd, wd, gyd = x.to(gpu), w.to(gpu), gy.to(gpu)
+    xq, sx = ops.abc_forward(xd, opt)
+    xq_ref, sx_ref = orc.abc_forward(x.numpy(), ocfg)
+    tr = orc.linear_backward(gy.numpy(), w.numpy(), xq_ref, sx_ref, ocfg)
+    need = 1 << 26
+    ws = torch.empty(need, dtype=torch.uint8, device=gpu)
+    eager = ops.linear_backward(gyd, wd, xq, sx, opt, workspace=ws)
+    torch.cuda.synchronize()
+    assert np.array_equal(eager[0].cpu().numpy(), tr.g_x) and np.array_equal(eager[1].cpu().numpy(), tr.g_w)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.linear_backward(gyd, wd, xq, sx, opt, workspace=ws)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    opt_cap = ops.HotOptions(n_o=16, hla_n=n, hla_rows=ocfg.hla_rows)       # its own C arrays, dropped below
+    with torch.cuda.graph(graph):
+        out = ops.linear_backward(gyd, wd, xq, sx, opt_cap, workspace=ws)
+    del opt_cap
+    import gc
+    gc.collect()
+    for _ in range(3):
+        ws.fill_(0x5A)                                   # the row table in the workspace is rebuilt by the replay
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(out[0].cpu().numpy(), tr.g_x) and np.array_equal(out[1].cpu().numpy(), tr.g_w)
+        again = ops.linear_backward(gyd, wd, xq, sx, opt, workspace=ws)
+        torch.cuda.synchronize()
+        assert torch.equal(again[0], eager[0]) and torch.equal(again[1], eager[1])
+
+
 def test_small_vit_with_hot_layers(gpu, fresh_args):
     """A whole (small) ViT with every Linear / Conv2d swapped: LQS calibration, then one HOT step whose
     parameter gradients point the same way as the full-precision ones."""
