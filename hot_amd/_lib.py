@@ -32,6 +32,8 @@ EXPORTS = (
     "hot_gemm_splits", "hot_hla_workspace_bytes", "hot_linear_backward_bias",
     "hot_gemm_plan", "hot_gemm_workspace_bytes", "hot_gemm_i8_variant",
     "hot_hla_tokenwise_static", "hot_measure_ceilings",
+    "hot_kpad_group", "hot_abc_batched_workspace_bytes", "hot_abc_forward_batched",
+    "hot_backward_batched_workspace_bytes", "hot_linear_backward_batched",
 )
 
 
@@ -100,6 +102,16 @@ def _declare(lib):
     lib.hot_hla_tokenwise_static.restype = i32
     lib.hot_hla_tokenwise_static.argtypes = [vp, i32, i64, i64, i32, C.POINTER(C.c_int32), i32, i32, i32, u64, u32,
                                              i32, vp, i64, vp, vp]
+    lib.hot_kpad_group.restype = i64
+    lib.hot_kpad_group.argtypes = [i64, cfgp]
+    lib.hot_abc_batched_workspace_bytes.restype = sz
+    lib.hot_abc_batched_workspace_bytes.argtypes = [i64, i64, i64, cfgp]
+    lib.hot_abc_forward_batched.restype = i32
+    lib.hot_abc_forward_batched.argtypes = [vp, i32, i64, i64, i64, cfgp, vp, vp, vp, sz, vp]
+    lib.hot_backward_batched_workspace_bytes.restype = sz
+    lib.hot_backward_batched_workspace_bytes.argtypes = [i64, i64, i64, i64, cfgp]
+    lib.hot_linear_backward_batched.restype = i32
+    lib.hot_linear_backward_batched.argtypes = [vp, vp, i32, vp, vp, i64, i64, i64, i64, cfgp, vp, vp, i32, vp, sz, vp]
     lib.hot_measure_ceilings.restype = i32
     lib.hot_measure_ceilings.argtypes = [vp, sz, C.POINTER(C.c_float), C.POINTER(C.c_float), vp]
     lib.hot_linear_backward_bias.restype = i32

@@ -452,6 +452,122 @@ int hot_linear_backward_bias(const void* gy, const void* w, int dtype, const voi
                       nullptr, (hipStream_t)hip_stream, gb);
 }
 
+// ---- 3-D activations: one set of steps per sample --------------------------------------------------
+// The reference vmaps its quantisers over the batch dimension of [B, T, C] tensors
+// (utils/quant_matmul.py:33-37,102-106,118-122), applies the token-wise transform inside each sample
+// (utils/hadamard_matmul.py:143-161, 3-D branch) and returns one weight gradient per sample, which
+// autograd sums (utils/quant_matmul.py:288-290,322-324).  Here the B samples are the rows [b T, (b+1) T)
+// of the flattened tensors; the codes of sample b occupy K range [b kg, (b+1) kg) of the g_W operands,
+// kg = hot_kpad_group(T') = T' rounded up to 128 codes, and the g_W product dequantises every sample's
+// integer sums with that sample's steps before adding them up in fp32, in sample order.
+
+struct BatchedLayout {
+  int64_t ld_g, ld_w, kg, ld_gp;
+  size_t off_colw, off_colg, off_hq, off_sg, off_sw, off_sgp, off_qg, off_qw, off_qgp, total;
+};
+
+static int64_t kpad_group(int64_t T, const hot_config* c) { return round_up((T / c->hla_n) * c->hla_r, 128); }
+
+static BatchedLayout batched_layout(int64_t B, int64_t T, int64_t O, int64_t I, const hot_config* c) {
+  BatchedLayout b;
+  const int64_t L = B * T;
+  b.ld_g = round_up(O, GEMM_KTILE) * c->gx_bits / 8;
+  b.ld_w = round_up(O, GEMM_KTILE) * c->w_bits / 8;
+  b.kg = kpad_group(T, c);
+  b.ld_gp = B * b.kg;
+  size_t o = 0;
+  b.off_colw = o; o += align256(colwise_workspace_bytes_impl(I));
+  b.off_colg = o; o += align256(colwise_group_workspace_bytes_impl(O, (int)B));
+  b.off_hq = o;   o += align256((size_t)B * 4 > STAT_SLOT_BYTES ? (size_t)B * 4 : STAT_SLOT_BYTES);
+  b.off_sg = o;   o += align256((size_t)L * 4);
+  b.off_sw = o;   o += 256;
+  b.off_sgp = o;  o += align256((size_t)B * (size_t)O * 4);
+  b.off_qg = o;   o += align256((size_t)L * b.ld_g);
+  b.off_qw = o;   o += align256((size_t)I * b.ld_w);
+  b.off_qgp = o;  o += align256((size_t)O * b.ld_gp);
+  b.total = o;
+  return b;
+}
+
+static int check_batched(const hot_config* cfg, int64_t B, int64_t T, const char* who) {
+  if (int e = check_cfg(cfg, who)) return e;
+  if (B < 1 || B > 65535 || T < 1) return fail(HOT_ERR_INVALID, "%s: bad batch %lld x %lld tokens", who, (long long)B, (long long)T);
+  if (cfg->hla_n > COL_MAX_N) return fail(HOT_ERR_UNSUPPORTED, "%s: token blocks up to %d inside a sample", who, COL_MAX_N);
+  if (T % cfg->hla_n) return fail(HOT_ERR_INVALID, "%s: T=%lld is not a multiple of hla_n=%d", who, (long long)T, cfg->hla_n);
+  return HOT_OK;
+}
+
+int64_t hot_kpad_group(int64_t T, const hot_config* cfg) {
+  if (!cfg || cfg->hla_n < 1 || T < 1) return 0;
+  return kpad_group(T, cfg);
+}
+
+size_t hot_abc_batched_workspace_bytes(int64_t B, int64_t T, int64_t I, const hot_config* cfg) {
+  (void)T; (void)cfg;
+  return colwise_group_workspace_bytes_impl(I > 0 ? I : 0, B > 0 ? (int)B : 1);
+}
+
+int hot_abc_forward_batched(const void* x, int dtype, int64_t B, int64_t T, int64_t I, const hot_config* cfg,
+                            void* xq_out, float* sx_out, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  const char* who = "hot_abc_forward_batched";
+  if (int e = check_batched(cfg, B, T, who)) return e;
+  if (I <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape I=%lld", who, (long long)I);
+  if (cfg->act_scale == HOT_SCALE_ROW) return fail(HOT_ERR_UNSUPPORTED, "%s: the activation buffer uses one step per sample", who);
+  const int64_t kg = kpad_group(T, cfg);
+  return colwise_quant_impl(x, dtype, B * T, I, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, cfg->act_bits, cfg->act_round, cfg->seed,
+                            HOT_STREAM_ACT, cfg->act_scale, xq_out, B * kg, 0, sx_out, workspace, workspace_bytes,
+                            (hipStream_t)hip_stream, who, nullptr, false, nullptr, nullptr, (int)B, kg);
+}
+
+size_t hot_backward_batched_workspace_bytes(int64_t B, int64_t T, int64_t O, int64_t I, const hot_config* cfg) {
+  if (check_batched(cfg, B, T, "hot_backward_batched_workspace_bytes") || O <= 0 || I <= 0) return 0;
+  return batched_layout(B, T, O, I, cfg).total;
+}
+
+int hot_linear_backward_batched(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t B,
+                                int64_t T, int64_t O, int64_t I, const hot_config* cfg, void* gx, void* gw, int out_dtype,
+                                void* workspace, size_t workspace_bytes, void* hip_stream) {
+  const char* who = "hot_linear_backward_batched";
+  if (int e = check_batched(cfg, B, T, who)) return e;
+  if (!gy || !w || !xq || !sx || !gx || !gw) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
+  if (O <= 0 || I <= 0 || O % 8 || I % 8) return fail(HOT_ERR_INVALID, "%s: O=%lld and I=%lld must be positive multiples of 8", who, (long long)O, (long long)I);
+  if (O % cfg->n_o) return fail(HOT_ERR_INVALID, "%s: O=%lld is not a multiple of n_o=%d", who, (long long)O, cfg->n_o);
+  if (cfg->gx_bits != cfg->w_bits) return fail(HOT_ERR_UNSUPPORTED, "%s: gx_bits (%d) and w_bits (%d) must match", who, cfg->gx_bits, cfg->w_bits);
+  if (cfg->gx_scale == HOT_SCALE_SAWB || cfg->gw_scale == HOT_SCALE_SAWB) return fail(HOT_ERR_UNSUPPORTED, "%s: SAWB applies to W and x only", who);
+  if (cfg->w_scale == HOT_SCALE_ROW) return fail(HOT_ERR_UNSUPPORTED, "%s: W uses one step per tensor", who);
+  const int64_t L = B * T;
+  if (L * O * 4 >= (1ll << 32) || O * I * 4 >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "%s: tensors exceed the 32-bit offsets of the loader", who);
+  const BatchedLayout b = batched_layout(B, T, O, I, cfg);
+  if (!workspace || workspace_bytes < b.total) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, b.total, workspace_bytes);
+  if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
+  hipStream_t st = (hipStream_t)hip_stream;
+  uint8_t* ws = (uint8_t*)workspace;
+  float* sg = (float*)(ws + b.off_sg);
+  float* sw = (float*)(ws + b.off_sw);
+  float* sgp = (float*)(ws + b.off_sgp);
+  // W: Hadamard along O + quantise, stored [I, O]
+  int rc = colwise_quant_impl(w, dtype, O, I, cfg->n_o, identity_rows(), cfg->n_o, cfg->w_bits, cfg->w_round, cfg->seed,
+                              HOT_STREAM_W, cfg->w_scale, ws + b.off_qw, b.ld_w, cfg->w_bits == 4, sw, ws + b.off_colw,
+                              colwise_workspace_bytes_impl(I), st, who);
+  if (rc) return rc;
+  // g_y: Hadamard along O, one step per sample (or per token) -> g_x operand; the GEMM reads a step per row
+  rc = hq_rowwise_impl(gy, dtype, L, O, cfg->n_o, cfg->gx_bits, cfg->gx_round, cfg->seed, HOT_STREAM_GX, cfg->gx_scale,
+                       ws + b.off_qg, b.ld_g, sg, ws + b.off_hq, b.off_sg - b.off_hq, st, false,
+                       cfg->gx_scale == HOT_SCALE_TENSOR ? T : 0, nullptr);
+  if (rc) return rc;
+  rc = gemm_i8_impl(ws + b.off_qg, b.ld_g, ws + b.off_qw, b.ld_w, cfg->gx_bits, L, I, O, sg, 1, sw, 1.0f / (float)cfg->n_o, gx,
+                    out_dtype, I, nullptr, st);
+  if (rc) return rc;
+  // g_y: HLA inside every sample, one step per sample (or per sample and channel), transposed -> g_W operand
+  rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, cfg->gw_bits, cfg->gw_round, cfg->seed,
+                          HOT_STREAM_GW, cfg->gw_scale, ws + b.off_qgp, b.ld_gp, 0, sgp, ws + b.off_colg,
+                          colwise_group_workspace_bytes_impl(O, (int)B), st, who, nullptr, false, nullptr, nullptr, (int)B, b.kg);
+  if (rc) return rc;
+  // g_W = sum over samples of (qGp_b . xq_b^T) sGp_b sx_b / hla_n
+  return gemm_i8_grouped_impl(ws + b.off_qgp, b.ld_gp, xq, b.ld_gp, O, I, (int)B, b.kg, sgp, cfg->gw_scale == HOT_SCALE_ROW, sx,
+                              1.0f / (float)cfg->hla_n, gw, out_dtype, I, st);
+}
+
 int hot_linear_backward_kernels(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,
                                 int64_t O, int64_t I, const hot_config* cfg, void* gx, void* gw, int out_dtype,
                                 void* workspace, size_t workspace_bytes, float* times8, void* hip_stream) {

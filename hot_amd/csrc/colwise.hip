@@ -53,6 +53,14 @@ struct ColArgs {
   uint32_t stream;
   int32_t r, rpad, bits, store4, rounding, mode, tb, stats_cleared;
   uint32_t gx, gy;     // logical grid: channel strips x runs of token blocks
+  // Sample groups (3-D activations: one step per sample).  The R rows are `groups` samples of NBs
+  // token blocks each; a workgroup's run of blocks never leaves its sample (`runs` runs per sample),
+  // the codes of a sample take Kpad bytes of every output row (the tail zeroed), and the statistics
+  // are kept per sample: gstat[g] (absmax, TENSOR), gstat[groups + 2 g] / [.. + 1] (step / clip,
+  // SAWB), colmax[g * C + c] (ROW).  groups == 1: the whole input is one group with Kpad = ld_out.
+  int32_t groups, runs;
+  int64_t NBs, Kpad;
+  float* gstat;
   hipEvent_t after_stats;  // host only: recorded between the statistics and the quantise pass
   int8_t slot[COL_MAX_N];  // output position of natural row i, -1 = dropped
 };
@@ -210,8 +218,11 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   const int chan = RSP ? (tid ^ ((tid & 4) ? 0xB : 0)) : tid;   // channel of this thread within the workgroup
   const int64_t c = cg0 + chan;
   const bool active = c < a.C;
-  const int64_t blk0 = (int64_t)by * a.tb;
-  int nblk = (int)((a.NB - blk0) < a.tb ? (a.NB - blk0) : a.tb);
+  const int sample = a.groups > 1 ? (int)(by / (unsigned)a.runs) : 0;
+  const int run = (int)by - sample * a.runs;
+  const int64_t blk_in = (int64_t)run * a.tb;                    // first block of the run within its sample
+  const int64_t blk0 = (int64_t)sample * a.NBs + blk_in;
+  int nblk = (int)((a.NBs - blk_in) < a.tb ? (a.NBs - blk_in) : a.tb);
   const int nsteps = (nblk * N + CW_ROWS - 1) / CW_ROWS;
   const int qmax = (1 << (a.bits - 1)) - 1;
   const int sb = a.tb * a.r;        // staged code bytes per channel
@@ -242,7 +253,20 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       __syncthreads();
     }
     // absmax modes read the statistic itself (no finalize kernel in between) and publish the step
-    if (a.mode == HOT_SCALE_ROW) {
+    if (a.groups > 1) {
+      if (a.mode == HOT_SCALE_ROW) {
+        const float sc = (active ? a.colmax[(int64_t)sample * a.C + c] : 0.f) / (float)qmax;
+        d = active ? sc + 1e-11f : 1.f;
+        if (active && run == 0) a.scales_out[(int64_t)sample * a.C + c] = sc;
+      } else if (a.mode == HOT_SCALE_TENSOR) {
+        const float sc = a.gstat[sample] / (float)qmax;
+        d = sc + 1e-11f;
+        if (bx == 0 && run == 0 && tid == 0) a.scales_out[sample] = sc;
+      } else {
+        d = a.gstat[a.groups + 2 * sample] + 1e-11f;
+        clip = a.gstat[a.groups + 2 * sample + 1];
+      }
+    } else if (a.mode == HOT_SCALE_ROW) {
       float cm = 0.f;
       if (active) {
 #pragma unroll
@@ -423,7 +447,10 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       __syncthreads();
     }
     if (a.mode == HOT_SCALE_ROW) {
-      if (active) atomic_max_nonneg(a.colmax + (by % COLMAX_COPIES) * a.C + c, cmax);
+      if (active) {
+        if (a.groups > 1) atomic_max_nonneg(a.colmax + (int64_t)sample * a.C + c, cmax);
+        else atomic_max_nonneg(a.colmax + (by % COLMAX_COPIES) * a.C + c, cmax);
+      }
       return;
     }
     if (a.mode == HOT_SCALE_TENSOR) {
@@ -433,7 +460,8 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       if (tid == 0) {
         float mm = s_max[0];
         for (int i = 1; i < CW / 64; ++i) mm = fmaxf(mm, s_max[i]);
-        stat_slot_update(a.slots, wg_id, mm);
+        if (a.groups > 1) atomic_max_nonneg(a.gstat + sample, mm);
+        else stat_slot_update(a.slots, wg_id, mm);
       }
       return;
     }
@@ -452,10 +480,10 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   } else {
     __syncthreads();
     // flush: each channel's staged run is one contiguous global segment
-    const bool last = blk0 + a.tb >= a.NB;
+    const bool last = blk_in + a.tb >= a.NBs;       // the run that ends its sample also zeroes the sample's tail
     const int out_sb = a.store4 ? sb / 2 : sb;
-    const int64_t seg0 = (int64_t)by * out_sb;      // byte offset in the output row
-    const int64_t seg_end = last ? a.ld_out : seg0 + out_sb;
+    const int64_t seg0 = (int64_t)sample * a.Kpad + (int64_t)run * out_sb;      // byte offset in the output row
+    const int64_t seg_end = last ? (int64_t)(sample + 1) * a.Kpad : seg0 + out_sb;
     const int ndw = (int)((seg_end - seg0) / 4);            // output dwords per channel
     const int sdw = out_sb / 4;                             // of which staged
     const int nch = (int)((a.C - cg0) < CW ? (a.C - cg0) : CW);
@@ -520,8 +548,11 @@ __global__ void __launch_bounds__(256) colwise_finalize_kernel(const ColArgs a, 
     }
     return;
   }
+  // SAWB: one block per sample group adds up the partial sums of the group's workgroups (nwg each,
+  // numbered run-major, so a group's workgroups are adjacent) in a fixed order
+  const int64_t g = blockIdx.x;
   double q = 0.0, b = 0.0;
-  for (int64_t i = tid; i < nwg; i += 256) { q += a.partial[2 * i]; b += a.partial[2 * i + 1]; }
+  for (int64_t i = tid; i < nwg; i += 256) { q += a.partial[2 * (g * nwg + i)]; b += a.partial[2 * (g * nwg + i) + 1]; }
   s_q[tid] = q; s_b[tid] = b;
   __syncthreads();
   for (int s = 128; s > 0; s >>= 1) {
@@ -529,21 +560,28 @@ __global__ void __launch_bounds__(256) colwise_finalize_kernel(const ColArgs a, 
     __syncthreads();
   }
   if (tid == 0) {
-    const double cnt = (double)a.Kout * (double)a.C;
+    const double cnt = (double)(a.Kout / a.groups) * (double)a.C;
     const float clip = (float)(12.1 * sqrt(s_q[0] / cnt) - 12.2 * (s_b[0] / cnt));
     const float s = clip / qmax;
-    a.stat[1] = s;
-    a.stat[2] = clip;
-    a.scales_out[0] = s;
+    if (a.groups > 1) {
+      a.gstat[a.groups + 2 * g] = s;
+      a.gstat[a.groups + 2 * g + 1] = clip;
+      a.scales_out[g] = s;
+    } else {
+      a.stat[1] = s;
+      a.stat[2] = clip;
+      a.scales_out[0] = s;
+    }
   }
 }
 
 // stat | slots are adjacent (COL_STAT_BYTES); row_absmax is another slot array
-__global__ void colwise_clear_kernel(float* stat, float* colmax, int64_t C, float* row_absmax) {
+__global__ void colwise_clear_kernel(float* stat, float* colmax, int64_t ncolmax, float* row_absmax, float* gstat, int64_t ngstat) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < (int64_t)(COL_STAT_BYTES / 4)) stat[i] = 0.f;
   if (row_absmax && i < (int64_t)(STAT_SLOT_BYTES / 4)) row_absmax[i] = 0.f;
-  if (colmax && i < C * COLMAX_COPIES) colmax[i] = 0.f;
+  if (colmax && i < ncolmax) colmax[i] = 0.f;
+  if (gstat && i < ngstat) gstat[i] = 0.f;
 }
 
 // ---- column sums ------------------------------------------------------------------
@@ -618,6 +656,14 @@ size_t colwise_workspace_bytes_impl(int64_t C) {
   return COL_STAT_BYTES + (size_t)round_up(C * 4 * COLMAX_COPIES, 256) + (size_t)(2 * sizeof(double)) * 65536;
 }
 
+// with sample groups: stat | per-sample per-channel max | per-sample statistics | partial sums
+static size_t group_colmax_bytes(int64_t C, int groups) { return (size_t)round_up(C * 4 * (int64_t)groups, 256); }
+static size_t group_gstat_bytes(int groups) { return (size_t)round_up((int64_t)groups * 3 * 4, 256); }
+size_t colwise_group_workspace_bytes_impl(int64_t C, int groups) {
+  if (groups <= 1) return colwise_workspace_bytes_impl(C);
+  return COL_STAT_BYTES + group_colmax_bytes(C, groups) + group_gstat_bytes(groups) + (size_t)(2 * sizeof(double)) * 65536;
+}
+
 template <typename T, int N, int PASS, int ROUND, bool SAWB, typename SEL, int RS = 0>
 static int launch_pass(const ColArgs& a, dim3 grid, size_t lds, hipStream_t st) {
   // one-time per instantiation; later calls only read the outcome
@@ -676,13 +722,19 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   const size_t in_bytes = (size_t)ring_depth<T>() * CW_ROWS * CW * sizeof(T);
   const size_t lds_stats = in_bytes, lds_quant = in_bytes + (size_t)CW * (tb * a.r + 4);
   if (lds_quant > 150 * 1024) return fail(HOT_ERR_UNSUPPORTED, "colwise: staging does not fit LDS");
-  const int64_t gx = (a.C + CW - 1) / CW, gy = (a.NB + tb - 1) / tb;
+  // runs of token blocks: per sample group (a run never leaves its sample)
+  const int64_t gx = (a.C + CW - 1) / CW, runs = (a.NBs + tb - 1) / tb, gy = runs * a.groups;
   if (gy > 65535 || gx * gy > 65536) return fail(HOT_ERR_UNSUPPORTED, "colwise: grid %lld x %lld too large", (long long)gx, (long long)gy);
+  a.runs = (int)runs;
   const dim3 grid((unsigned)gx, (unsigned)gy);
   if (!a.stats_cleared) {
-    const int64_t nclr = a.C * COLMAX_COPIES > (int64_t)(COL_STAT_BYTES / 4) ? a.C * COLMAX_COPIES : (int64_t)(COL_STAT_BYTES / 4);
+    const int64_t ncolmax = a.mode == HOT_SCALE_ROW ? (a.groups > 1 ? a.C * a.groups : a.C * COLMAX_COPIES) : 0;
+    const int64_t ngstat = a.groups > 1 ? 3 * (int64_t)a.groups : 0;
+    int64_t nclr = (int64_t)(COL_STAT_BYTES / 4);
+    if (ncolmax > nclr) nclr = ncolmax;
+    if (ngstat > nclr) nclr = ngstat;
     hipLaunchKernelGGL(colwise_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat,
-                       a.mode == HOT_SCALE_ROW ? a.colmax : (float*)nullptr, a.C, a.row_absmax);
+                       ncolmax ? a.colmax : (float*)nullptr, ncolmax, a.row_absmax, ngstat ? a.gstat : (float*)nullptr, ngstat);
   }
   int rc;
   if (a.mode == HOT_SCALE_SAWB) {
@@ -690,12 +742,13 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   } else {
     ColArgs a0 = a;
     a0.tb = part.tb0;
-    const dim3 grid0((unsigned)gx, (unsigned)((a.NB + a0.tb - 1) / a0.tb));
+    a0.runs = (int)((a.NBs + a0.tb - 1) / a0.tb);
+    const dim3 grid0((unsigned)gx, (unsigned)(a0.runs * a.groups));
     if (a.row_absmax) rc = launch_pass<T, N, 0, 0, false, SEL, 16>(a0, grid0, lds_stats, st);
     else rc = launch_pass<T, N, 0, 0, false, SEL>(a0, grid0, lds_stats, st);
   }
   if (rc) return rc;
-  if (a.mode == HOT_SCALE_SAWB) hipLaunchKernelGGL(colwise_finalize_kernel, dim3(1), dim3(256), 0, st, a, gx * gy);
+  if (a.mode == HOT_SCALE_SAWB) hipLaunchKernelGGL(colwise_finalize_kernel, dim3((unsigned)a.groups), dim3(256), 0, st, a, gx * runs);
   if (a.after_stats) (void)hipEventRecord(a.after_stats, st);
   if (a.rounding == HOT_ROUND_STOCH) {
     if (a.mode == HOT_SCALE_SAWB) rc = launch_pass<T, N, 1, 1, true, SEL>(a, grid, lds_quant, st);
@@ -776,9 +829,16 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
                        int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
                        void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,
                        size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out,
-                       bool stats_cleared, hipEvent_t after_stats, float* colsum_partial) {
+                       bool stats_cleared, hipEvent_t after_stats, float* colsum_partial, int groups, int64_t kpad_group) {
   if (!in || !codes_out || !scales_out || !rows) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
   if (R <= 0 || C <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape R=%lld C=%lld", who, (long long)R, (long long)C);
+  if (groups < 1) return fail(HOT_ERR_INVALID, "%s: %d sample groups", who, groups);
+  if (groups > 1) {
+    if (n > COL_MAX_N || store4 || row16_absmax_out || colsum_partial || stats_cleared)
+      return fail(HOT_ERR_UNSUPPORTED, "%s: per-sample steps take token blocks up to %d, INT8 storage, and neither the fused row statistic nor the column sums", who, COL_MAX_N);
+    if (n < 1 || R % ((int64_t)n * groups)) return fail(HOT_ERR_INVALID, "%s: R=%lld is not %d samples of whole blocks of %d", who, (long long)R, groups, n);
+    if (kpad_group < (R / n / groups) * r || (kpad_group & 15)) return fail(HOT_ERR_INVALID, "%s: %lld code bytes per sample must be a multiple of 16 and hold the sample's codes", who, (long long)kpad_group);
+  }
   if (n > COL_MAX_N) {
     // blocks one thread cannot hold: the two-level path
     if (store4 || row16_absmax_out) return fail(HOT_ERR_UNSUPPORTED, "%s: blocks above %d tokens have no packed-INT4 store and no fused row statistic", who, COL_MAX_N);
@@ -821,10 +881,10 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
     if (a.slot[rows[k]] != -1) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d listed twice", who, k, rows[k]);
     a.slot[rows[k]] = (int8_t)k;
   }
-  const int64_t row_bytes = store4 ? a.Kout / 2 : a.Kout;
+  const int64_t row_bytes = groups > 1 ? kpad_group * groups : (store4 ? a.Kout / 2 : a.Kout);
   if (store4 && (r & 1)) return fail(HOT_ERR_UNSUPPORTED, "%s: packed INT4 output needs an even r", who);
   if (ld_out < row_bytes || (ld_out & 15)) return fail(HOT_ERR_INVALID, "%s: ld_out=%lld must be a multiple of 16 and >= %lld", who, (long long)ld_out, (long long)row_bytes);
-  if (!workspace || workspace_bytes < colwise_workspace_bytes_impl(C)) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed", who, colwise_workspace_bytes_impl(C));
+  if (!workspace || workspace_bytes < colwise_group_workspace_bytes_impl(C, groups)) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed", who, colwise_group_workspace_bytes_impl(C, groups));
   if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
   a.store4 = store4;
   a.stats_cleared = stats_cleared ? 1 : 0;
@@ -834,6 +894,12 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   a.slots = (float*)(ws + 256);
   a.colmax = (float*)(ws + COL_STAT_BYTES);
   a.partial = (double*)(ws + COL_STAT_BYTES + round_up(C * 4 * COLMAX_COPIES, 256));
+  a.gstat = nullptr;
+  a.groups = groups; a.runs = 1; a.NBs = a.NB / groups; a.Kpad = groups > 1 ? kpad_group : ld_out;
+  if (groups > 1) {
+    a.gstat = (float*)(ws + COL_STAT_BYTES + group_colmax_bytes(C, groups));
+    a.partial = (double*)(ws + COL_STAT_BYTES + group_colmax_bytes(C, groups) + group_gstat_bytes(groups));
+  }
   a.scales_out = scales_out;
   // the fused row-wise statistic exists for block 16 and absmax steps, and needs whole 16-blocks of channels
   a.colsum = colsum_partial;

@@ -51,6 +51,12 @@ struct GemmArgs {
   int32_t vec16;     // out and its row pitch are 16-byte aligned (staged epilogue)
   int32_t splits;    // K is cut into this many ranges, one workgroup each (1 = no split)
   v4i* partials;     // [tile][range][wave][fragment quad][lane]: raw accumulators of the ranges
+  // K groups (3-D activations: a group is a sample with steps of its own): every group_stages
+  // stages the integer accumulators are dequantised with the group's steps and added, in group order,
+  // to fp32 accumulators: out = (sum over groups of (float(acc_g) * sa_g[row or 0]) * sb_g) * post_scale
+  int32_t group_stages;     // stages (of the kernel's stage width) per group; 0 = one group, integer all the way
+  const float* gscale_a;    // [groups] or, with a_per_row, [groups][M]
+  const float* gscale_b;    // [groups]
 };
 
 // Workgroup -> tile.  Hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with
@@ -620,7 +626,9 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
 // robin to the four waves; when that is not a multiple of four the spare DMA slots fetch into a
 // spare KiB, so that every wave issues the same number of loads and one vmcnt serves all.
 // ---------------------------------------------------------------------------
-template <int WM, int WN, int GM, int GN, int BITS, int S, int RB, typename OutT>
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+template <int WM, int WN, int GM, int GN, int BITS, int S, int RB, typename OutT, bool GROUPED = false>
 __global__ void __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(1, (WM * WN <= 8 ? 2 : 1))))
 gemm_i8_slot_kernel(const GemmArgs g) {
   static_assert(GM * GN == 4, "four waves");
@@ -688,7 +696,13 @@ gemm_i8_slot_kernel(const GemmArgs g) {
   const uint32_t ring0 = lds_offset(ring);
   const int KT = g.ktiles * (G_BK * BITS / 8) / RB;               // stages of RB bytes per row
   auto dma_one = [&](int stage_off, int kt, int i) {
-    const uint8_t* base = ((is_b >> i) & 1u ? g.B : g.A) + (int64_t)kt * RB;
+    // (wave-uniform by construction; said explicitly, since the instruction takes it in scalar registers)
+    const uint64_t b64 = (uint64_t)(uintptr_t)(((is_b >> i) & 1u ? g.B : g.A) + (int64_t)kt * RB);
+    // (the builtin returns a signed int: both halves go through uint32_t, or a low half with its top
+    // bit set would sign-extend over the high half)
+    const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b64 >> 32));
+    const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b64);
+    const uint8_t* base = reinterpret_cast<const uint8_t*>(((uint64_t)b_hi << 32) | (uint64_t)b_lo);
     const bool spare = SPARE && ldst[i] == (uint32_t)(S * STAGE_BYTES);
     dma16(ring0 + (spare ? 0u : (uint32_t)stage_off) + ldst[i], goff[i], base);
   };
@@ -740,6 +754,50 @@ gemm_i8_slot_kernel(const GemmArgs g) {
     for (int e = e0; e < e1 && e < 4 * NR; ++e) fr[p][e >> 2][e & 3] &= (int)0xF0F0F0F0;
   };
   constexpr int EPS_ = BITS == 4 ? (4 * NR + H - 1) / H : 0;     // expansion items per slot of a half round
+
+  // K groups: fp32 accumulators, the steps of the current group (loaded a group ahead), a stage counter
+  v16f facc[GROUPED ? WM : 1][GROUPED ? WN : 1];
+  float gsa[GROUPED ? WM : 1], gsb = 0.f;
+  int gstage = 0, gidx = 0;
+  auto load_group_scales = [&](int gi) {
+    if constexpr (GROUPED) {
+#pragma unroll
+      for (int i = 0; i < WM; ++i) {
+        const int64_t row = row0 + wm * WM * 32 + i * 32 + (lane & 31);
+        gsa[i] = g.a_per_row ? g.gscale_a[(int64_t)gi * g.M + (row < g.M ? row : g.M - 1)] : g.gscale_a[gi];
+      }
+      gsb = g.gscale_b[gi];
+    }
+  };
+  if constexpr (GROUPED) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j) facc[i][j] = (v16f)(0.f);
+    load_group_scales(0);
+  }
+  // end of a stage: when it closes a group, dequantise the group's sums into the fp32 accumulators
+  auto stage_done = [&](int kt) {
+    if constexpr (GROUPED) {
+      if (++gstage == g.group_stages) {
+        gstage = 0;
+#pragma unroll
+        for (int i = 0; i < WM; ++i)
+#pragma unroll
+          for (int j = 0; j < WN; ++j) {
+            // the product is rounded before it is added (no fused multiply-add): the sum over the
+            // groups is the fp32 sum of the per-group results
+#pragma clang fp contract(off)
+            v16i a = acc[i][j];
+            if constexpr (BITS == 4) a = a >> 8;
+            facc[i][j] += (__builtin_convertvector(a, v16f) * gsa[i]) * gsb;
+            acc[i][j] = a - a;
+          }
+        ++gidx;
+        if (kt + 1 < KT) load_group_scales(gidx);
+      }
+    }
+  };
 
   // prologue: S tiles in flight, tile 0 landed and visible, its first round in registers
   static_for<S>([&](auto k) {
@@ -800,15 +858,45 @@ gemm_i8_slot_kernel(const GemmArgs g) {
   auto rotation = [&](auto steady, int kt0) {
     static_for<S>([&](auto k) {
       constexpr int K = decltype(k)::value;
-      if (decltype(steady)::value || kt0 + K < KT)
+      if (decltype(steady)::value || kt0 + K < KT) {
         ktile(steady, std::integral_constant<int, K * STAGE_BYTES>{}, std::integral_constant<int, ((K + 1) % S) * STAGE_BYTES>{},
               kt0 + K);
+        stage_done(kt0 + K);
+      }
     });
   };
   int kt0 = 0;
   for (; kt0 + 2 * S - 1 < KT; kt0 += S) rotation(std::true_type{}, kt0);   // every tile inside has a tile kt + S
   for (; kt0 < KT; kt0 += S) rotation(std::false_type{}, kt0);
 
+  if constexpr (GROUPED) {
+    // the sums are dequantised already: scale once more and store, four adjacent outputs per lane
+    OutT* out = reinterpret_cast<OutT*>(g.out);
+    const int half = lane >> 5;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+      const int64_t row = row0 + wm * WM * 32 + i * 32 + (lane & 31);
+      if (row >= g.M) continue;
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int64_t col = col0 + wn * WN * 32 + j * 32 + 8 * q + 4 * half;
+          if (col >= g.N) continue;
+          if (g.vec_out && col + 3 < g.N) {
+            typename Quad<OutT>::type v;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) quad_set<OutT>(v, t, facc[i][j][4 * q + t] * g.post_scale);
+            *reinterpret_cast<typename Quad<OutT>::type*>(out + row * g.ldo + col) = v;
+          } else {
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+              if (col + t < g.N) store_scalar<OutT>(out + row * g.ldo + col + t, facc[i][j][4 * q + t] * g.post_scale);
+          }
+        }
+    }
+    return;
+  }
   if constexpr (!EARLY_SCALES) {
     load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
     sb = g.scale_b[0];
@@ -872,7 +960,7 @@ static int launch_gemm_pipe(GemmArgs& g, hipStream_t st) {
   return check_launch("gemm_i8_pipe_kernel");
 }
 
-template <int WM, int WN, int GM, int GN, int BITS, int S, int RB, typename OutT>
+template <int WM, int WN, int GM, int GN, int BITS, int S, int RB, typename OutT, bool GROUPED = false>
 static int launch_gemm_slot(GemmArgs& g, hipStream_t st) {
   constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN;
   g.tiles_m = (int)((g.M + BM - 1) / BM);
@@ -882,7 +970,7 @@ static int launch_gemm_slot(GemmArgs& g, hipStream_t st) {
   if (total > (1 << 30)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: too many tiles");
   if (g.M * g.lda >= (1ll << 32) || g.N * g.ldb >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: operand larger than 4 GiB");
   if (((int64_t)g.ktiles * (G_BK * BITS / 8)) % RB) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: this kernel takes rows of a multiple of %d bytes", RB);
-  hipLaunchKernelGGL((gemm_i8_slot_kernel<WM, WN, GM, GN, BITS, S, RB, OutT>), dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
+  hipLaunchKernelGGL((gemm_i8_slot_kernel<WM, WN, GM, GN, BITS, S, RB, OutT, GROUPED>), dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
   return check_launch("gemm_i8_slot_kernel");
 }
 
@@ -945,15 +1033,8 @@ GemmSplit gemm_split_plan(int64_t M, int64_t N, int64_t K, int bits) {
 // split-K pair.  The slot-scheduled kernels stage 128 bytes of every row at a time and take rows of
 // a multiple of 128 bytes only.  The DMA kernels address operands with 32-bit offsets; larger
 // operands take the register-staged kernel.
-#ifdef HOT_EXPERIMENTS
-int g_force_variant[2] = {0, 0};   // [INT4, INT8]; 0 = the rule
-extern "C" __attribute__((visibility("default"))) void hot_experiment_force(int bits, int variant) { g_force_variant[bits == 8] = variant; }
-#endif
 int gemm_plan_impl(int64_t M, int64_t N, int64_t K, int bits, int64_t lda, int64_t ldb, size_t ws_bytes) {
   if (M <= 0 || N <= 0 || K <= 0 || (bits != 4 && bits != 8)) return HOT_GEMM_AUTO;
-#ifdef HOT_EXPERIMENTS
-  if (g_force_variant[bits == 8]) return g_force_variant[bits == 8];
-#endif
   if (M * lda >= (1ll << 32) || N * ldb >= (1ll << 32)) return HOT_GEMM_REG_128;
   const int64_t kpad = round_up(K, GEMM_KTILE);
   const bool rows128 = (kpad * bits / 8) % 128 == 0;
@@ -1034,6 +1115,7 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
   g.vec_out = ((ldo & 3) == 0 && ((uintptr_t)out & 15) == 0) ? 1 : 0;
   g.vec16 = (((uintptr_t)out & 15) == 0 && ((ldo * (out_dtype == HOT_F32 ? 4 : 2)) & 15) == 0) ? 1 : 0;
   g.splits = 1; g.partials = nullptr;
+  g.group_stages = 0; g.gscale_a = nullptr; g.gscale_b = nullptr;
   if (variant == HOT_GEMM_DMA_128_SPLITK) {
     const GemmSplit plan = gemm_split_plan(M, N, K, bits);
     if (plan.splits < 2) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: the split-K kernel needs a product of fewer than 256 tiles of 128 x 128 and a long K");
@@ -1043,6 +1125,39 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
     g.partials = (v4i*)split_ws;
   }
   return bits == 4 ? dispatch_out<4>(out_dtype, variant, g, st) : dispatch_out<8>(out_dtype, variant, g, st);
+}
+
+// INT8 product whose K dimension is `groups` samples of group_k codes each (a multiple of 128), every
+// sample with steps of its own: out = (sum_g (float(acc_g) * sa[g][row or 0]) * sb[g]) * post_scale,
+// the groups added in order in fp32.  128 x 128 tiles, slot-scheduled, one workgroup per tile.
+int gemm_i8_grouped_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t M, int64_t N, int groups,
+                         int64_t group_k, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
+                         void* out, int out_dtype, int64_t ldo, hipStream_t st) {
+  const char* who = "hot_gemm_i8_grouped";
+  if (!A || !B || !scale_a || !scale_b || !out) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
+  if (M < 0 || N < 0 || groups < 1 || group_k <= 0 || (group_k % 128)) return fail(HOT_ERR_INVALID, "%s: bad shape %lld x %lld, %d groups of %lld codes (a multiple of 128)", who, (long long)M, (long long)N, groups, (long long)group_k);
+  const int64_t K = (int64_t)groups * group_k;
+  if (lda < K || ldb < K || (lda & 15) || (ldb & 15)) return fail(HOT_ERR_INVALID, "%s: row pitches (%lld, %lld) must be multiples of 16 and >= %lld bytes", who, (long long)lda, (long long)ldb, (long long)K);
+  if (((uintptr_t)A & 15) || ((uintptr_t)B & 15)) return fail(HOT_ERR_INVALID, "%s: operands must be 16-byte aligned", who);
+  if (ldo < N) return fail(HOT_ERR_INVALID, "%s: ldo=%lld < N", who, (long long)ldo);
+  if (group_k > (int64_t)(0x7FFFFFFF / (127 * 127))) return fail(HOT_ERR_UNSUPPORTED, "%s: group too long for int32 accumulation", who);
+  if (M * lda >= (1ll << 32) || N * ldb >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "%s: operand larger than 4 GiB", who);
+  if (M == 0 || N == 0) return HOT_OK;
+  GemmArgs g;
+  g.A = (const uint8_t*)A; g.B = (const uint8_t*)B; g.lda = lda; g.ldb = ldb; g.M = M; g.N = N;
+  g.ktiles = (int)(K / G_BK);
+  g.scale_a = scale_a; g.scale_b = scale_b; g.post_scale = post_scale; g.a_per_row = a_per_row;
+  g.out = out; g.ldo = ldo; g.acc_out = nullptr;
+  g.vec_out = ((ldo & 3) == 0 && ((uintptr_t)out & 15) == 0) ? 1 : 0;
+  g.vec16 = 0;
+  g.splits = 1; g.partials = nullptr;
+  g.group_stages = (int)(group_k / 128); g.gscale_a = scale_a; g.gscale_b = scale_b;
+  switch (out_dtype) {
+    case HOT_F32: return launch_gemm_slot<2, 2, 2, 2, 8, 4, 128, float, true>(g, st);
+    case HOT_BF16: return launch_gemm_slot<2, 2, 2, 2, 8, 4, 128, bf16_t, true>(g, st);
+    case HOT_F16: return launch_gemm_slot<2, 2, 2, 2, 8, 4, 128, f16_t, true>(g, st);
+    default: return fail(HOT_ERR_INVALID, "%s: bad out dtype %d", who, out_dtype);
+  }
 }
 
 }  // namespace hot

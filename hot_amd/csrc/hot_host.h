@@ -33,13 +33,21 @@ constexpr size_t STAT_SLOT_BYTES = (size_t)STAT_SLOTS * STAT_SLOT_STRIDE * 4;   
 int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, int rounding,
                     uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_codes,
                     float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st,
-                    bool absmax_ready = false);
+                    bool absmax_ready = false, int64_t group_rows = 0, float* group_steps = nullptr);
+// group_rows > 0 (per-tensor steps only): every run of group_rows rows is a sample with a step of its
+// own; scales_out then holds M entries (the step of each row's sample, the form the GEMM epilogue
+// reads), group_steps (may be null) the M / group_rows steps, and the workspace 4 bytes per sample.
 
 int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r,
                        int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
                        void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,
                        size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out = nullptr,
-                       bool stats_cleared = false, hipEvent_t after_stats = nullptr, float* colsum_partial = nullptr);
+                       bool stats_cleared = false, hipEvent_t after_stats = nullptr, float* colsum_partial = nullptr,
+                       int groups = 1, int64_t kpad_group = 0);
+// With groups > 1 the R rows are `groups` samples of equal length, each quantised with steps of its own
+// (scales_out: [groups], or [groups][C] with per-channel steps); the codes of sample g take the bytes
+// [g * kpad_group, (g + 1) * kpad_group) of every output row, zero-filled behind the sample's codes.
+size_t colwise_group_workspace_bytes_impl(int64_t C, int groups);
 // Column sums of the input of a colwise_quant_impl call (the bias gradient when the input is g_y):
 // with colsum_partial the call also writes colsum_strips_impl(...) rows of C partial sums (fp32; elem_bytes
 // = size of an input element, on which the partition of the passes depends; one
@@ -66,6 +74,10 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
                  size_t split_ws_bytes = 0, int variant = HOT_GEMM_AUTO);
 // The hot_gemm_variant that gemm_i8_impl picks for a product when `ws_bytes` of workspace come with it.
 int gemm_plan_impl(int64_t M, int64_t N, int64_t K, int bits, int64_t lda, int64_t ldb, size_t ws_bytes);
+
+int gemm_i8_grouped_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t M, int64_t N, int groups,
+                         int64_t group_k, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
+                         void* out, int out_dtype, int64_t ldo, hipStream_t st);
 
 // Split-K plan of gemm_i8_impl for a problem: `splits` K ranges (1 = none) and the bytes of workspace
 // that hold their partial accumulators (16-byte aligned; contents need no initialisation).

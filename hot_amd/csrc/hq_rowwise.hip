@@ -211,6 +211,59 @@ __global__ void hq_tensor_kernel(const T* __restrict__ in, int64_t nchunks, int6
   }
 }
 
+// ---- one scale per group of rows (3-D activations: a group is a sample) -------------------------
+// grid (blocks per group, groups); a block walks its group's chunks with a stride of the group's blocks
+
+template <typename T, int N>
+__global__ void hq_group_absmax_kernel(const T* __restrict__ in, int64_t chunks_per_group, float* __restrict__ gmax, int nrt) {
+  __shared__ float s_red[16];
+  const int lane = threadIdx.x & 63;
+  const int64_t g = blockIdx.y;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  float mx = 0.f;
+  for (int64_t ch = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ch < chunks_per_group; ch += stride) {
+    float x[EPL];
+    load_chunk<T>(in + (g * chunks_per_group + ch) * EPL, x);
+    fwht_lanes<N>(x, lane, nrt);
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) mx = fmaxf(mx, fabsf(x[j]));
+  }
+  mx = wave_max(mx);
+  if (lane == 0) s_red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float m = s_red[0];
+    for (int i = 1; i < (int)(blockDim.x >> 6); ++i) m = fmaxf(m, s_red[i]);
+    atomic_max_nonneg(gmax + g, m);
+  }
+}
+
+// scales_out [M]: the step of every row (= of its group), the form the GEMM epilogue reads;
+// group_steps [groups] (may be null): the steps themselves
+template <typename T, int N, int BITS, int ROUND>
+__global__ void hq_group_quant_kernel(const T* __restrict__ in, int64_t chunks_per_group, int64_t nch_row, int64_t ld,
+                                      const float* __restrict__ gmax, int8_t* __restrict__ codes,
+                                      float* __restrict__ scales_out, float* __restrict__ group_steps, uint64_t seed,
+                                      uint32_t stream, int nrt) {
+  const int lane = threadIdx.x & 63;
+  const int64_t g = blockIdx.y;
+  constexpr float QMAXF = (float)((1 << (BITS - 1)) - 1);
+  const float s = gmax[g] / QMAXF;
+  const float d = s + 1e-11f;
+  const float rcp = 1.0f / d;
+  if (group_steps && blockIdx.x == 0 && threadIdx.x == 0) group_steps[g] = s;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t c0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; c0 < chunks_per_group; c0 += stride) {
+    const int64_t ch = g * chunks_per_group + c0;
+    float x[EPL];
+    load_chunk<T>(in + ch * EPL, x);
+    fwht_lanes<N>(x, lane, nrt);
+    const int64_t row = ch / nch_row, col = ch - row * nch_row;
+    if (col == 0) scales_out[row] = s;
+    quant_store_chunk<BITS, ROUND>(x, d, rcp, (uint64_t)ch * EPL, seed, stream, codes + row * ld + col * (EPL * BITS / 8));
+  }
+}
+
 // zero the bytes [row_bytes, ld) of every row (K padding for the GEMM)
 __global__ void zero_pad_kernel(int8_t* codes, int64_t M, int64_t row_bytes, int64_t ld) {
   const int64_t padw = (ld - row_bytes) / 4;
@@ -270,13 +323,33 @@ static int launch_tensor(const void* in, int64_t M, int64_t K, void* codes, int6
 }
 
 template <typename T, int N, int BITS, int ROUND>
+static int launch_groups(const void* in, int64_t M, int64_t K, void* codes, int64_t ld, float* scales, float* gmax,
+                         float* group_steps, int64_t group_rows, uint64_t seed, uint32_t stream_id, hipStream_t st, int nrt) {
+  const int64_t groups = M / group_rows, cpg = group_rows * (K / EPL);
+  int64_t bx = (cpg + 255) / 256;
+  const int64_t cap = (256 * 16 + groups - 1) / groups;    // about 16 workgroups per CU in all
+  if (bx > cap) bx = cap;
+  if (bx < 1) bx = 1;
+  if (groups > 65535) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: more than 65535 sample groups");
+  const dim3 grid((unsigned)bx, (unsigned)groups);
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, st, (uint32_t*)gmax, 0u, (int)groups);
+  hipLaunchKernelGGL((hq_group_absmax_kernel<T, N>), grid, dim3(256), 0, st, (const T*)in, cpg, gmax, nrt);
+  hipLaunchKernelGGL((hq_group_quant_kernel<T, N, BITS, ROUND>), grid, dim3(256), 0, st, (const T*)in, cpg, K / EPL, ld, gmax,
+                     (int8_t*)codes, scales, group_steps, seed, stream_id, nrt);
+  return check_launch("hq_group_quant_kernel");
+}
+
+template <typename T, int N, int BITS, int ROUND>
 static int dispatch_mode(int scale_mode, const void* in, int64_t M, int64_t K, void* codes, int64_t ld, float* scales,
-                         float* absmax, uint64_t seed, uint32_t stream_id, hipStream_t st, bool absmax_ready, int nrt) {
+                         float* absmax, uint64_t seed, uint32_t stream_id, hipStream_t st, bool absmax_ready, int nrt,
+                         int64_t group_rows, float* group_steps) {
   const int64_t row_bytes = K * BITS / 8;
   if (ld > row_bytes) {
     const int64_t n = M * ((ld - row_bytes) / 4);
     hipLaunchKernelGGL(zero_pad_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (int8_t*)codes, M, row_bytes, ld);
   }
+  if (scale_mode == HOT_SCALE_TENSOR && group_rows > 0)
+    return launch_groups<T, N, BITS, ROUND>(in, M, K, codes, ld, scales, absmax, group_steps, group_rows, seed, stream_id, st, nrt);
   if (scale_mode == HOT_SCALE_ROW) return launch_row<T, N, BITS, ROUND>(in, M, K, codes, ld, scales, seed, stream_id, st, nrt);
   return launch_tensor<T, N, BITS, ROUND>(in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt);
 }
@@ -284,33 +357,34 @@ static int dispatch_mode(int scale_mode, const void* in, int64_t M, int64_t K, v
 template <typename T, int N>
 static int dispatch_bits(int bits, int rounding, int scale_mode, const void* in, int64_t M, int64_t K,
                          void* codes, int64_t ld, float* scales, float* absmax, uint64_t seed, uint32_t stream_id,
-                         hipStream_t st, bool absmax_ready, int nrt) {
+                         hipStream_t st, bool absmax_ready, int nrt, int64_t group_rows, float* group_steps) {
   if (bits == 4) {
     return rounding == HOT_ROUND_NEAREST
-               ? dispatch_mode<T, N, 4, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt)
-               : dispatch_mode<T, N, 4, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt);
+               ? dispatch_mode<T, N, 4, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt, group_rows, group_steps)
+               : dispatch_mode<T, N, 4, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt, group_rows, group_steps);
   }
   return rounding == HOT_ROUND_NEAREST
-             ? dispatch_mode<T, N, 8, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt)
-             : dispatch_mode<T, N, 8, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt);
+             ? dispatch_mode<T, N, 8, 0>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt, group_rows, group_steps)
+             : dispatch_mode<T, N, 8, 1>(scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, nrt, group_rows, group_steps);
 }
 
 template <typename T>
 static int dispatch_n(int n, int bits, int rounding, int scale_mode, const void* in, int64_t M, int64_t K,
                       void* codes, int64_t ld, float* scales, float* absmax, uint64_t seed, uint32_t stream_id,
-                      hipStream_t st, bool absmax_ready) {
+                      hipStream_t st, bool absmax_ready, int64_t group_rows, float* group_steps) {
   switch (n) {
     case 1: case 2: case 4: case 8:
-      return dispatch_bits<T, 8>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n);
-    case 16: return dispatch_bits<T, 16>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n);
-    case 32: return dispatch_bits<T, 32>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n);
-    default: return dispatch_bits<T, 64>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n);
+      return dispatch_bits<T, 8>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n, group_rows, group_steps);
+    case 16: return dispatch_bits<T, 16>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n, group_rows, group_steps);
+    case 32: return dispatch_bits<T, 32>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n, group_rows, group_steps);
+    default: return dispatch_bits<T, 64>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n, group_rows, group_steps);
   }
 }
 
 int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, int rounding,
                     uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_codes,
-                    float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st, bool absmax_ready) {
+                    float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st, bool absmax_ready,
+                    int64_t group_rows, float* group_steps) {
   if (M != 0 && (!in || !codes_out || !scales_out)) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: null pointer");
   if (M < 0 || K <= 0) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: bad shape M=%lld K=%lld", (long long)M, (long long)K);
   if (n < 1 || n > 64 || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: Hadamard block %d (a power of two up to 64)", n);
@@ -322,15 +396,18 @@ int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int 
   if (M >= (1ll << 31)) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: M too large");
   if (ld_codes < K * bits / 8 || (ld_codes & 7)) return fail(HOT_ERR_INVALID, "hot_hq_rowwise: code pitch %lld must be a multiple of 8 and >= %lld", (long long)ld_codes, (long long)(K * bits / 8));
   float* absmax = nullptr;
+  if (group_rows < 0 || (group_rows > 0 && (M % group_rows || scale_mode != HOT_SCALE_TENSOR)))
+    return fail(HOT_ERR_INVALID, "hot_hq_rowwise: %lld rows are not whole groups of %lld rows with one step each", (long long)M, (long long)group_rows);
   if (scale_mode == HOT_SCALE_TENSOR) {
-    if (!workspace || workspace_bytes < STAT_SLOT_BYTES) return fail(HOT_ERR_WORKSPACE, "hot_hq_rowwise: per-tensor scale needs a %zu-byte workspace", STAT_SLOT_BYTES);
+    const size_t need = group_rows > 0 ? (size_t)(M / group_rows) * 4 : STAT_SLOT_BYTES;
+    if (!workspace || workspace_bytes < need) return fail(HOT_ERR_WORKSPACE, "hot_hq_rowwise: per-tensor scale needs a %zu-byte workspace", need);
     absmax = (float*)workspace;
   }
   if (M == 0) return HOT_OK;
   switch (dtype) {
-    case HOT_F32: return dispatch_n<float>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st, absmax_ready);
-    case HOT_BF16: return dispatch_n<bf16_t>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st, absmax_ready);
-    case HOT_F16: return dispatch_n<f16_t>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st, absmax_ready);
+    case HOT_F32: return dispatch_n<float>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st, absmax_ready, group_rows, group_steps);
+    case HOT_BF16: return dispatch_n<bf16_t>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st, absmax_ready, group_rows, group_steps);
+    case HOT_F16: return dispatch_n<f16_t>(n, bits, rounding, scale_mode, in, M, K, codes_out, ld_codes, scales_out, absmax, seed, rng_stream, st, absmax_ready, group_rows, group_steps);
     default: return fail(HOT_ERR_INVALID, "hot_hq_rowwise: bad dtype %d", dtype);
   }
 }

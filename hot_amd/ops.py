@@ -277,6 +277,56 @@ def linear_backward(gy: torch.Tensor, w: torch.Tensor, xq: torch.Tensor, sx: tor
     return gx, gw
 
 
+def kpad_group(T: int, opt: HotOptions) -> int:
+    """Code bytes every sample takes in the K dimension of the batched g_W operands."""
+    return int(_lib.lib().hot_kpad_group(int(T), C.byref(opt.to_c())))
+
+
+def abc_forward_batched(x: torch.Tensor, opt: HotOptions):
+    """Activation buffer of a 3-D input [B, T, I] with one step per sample (hot_abc_forward_batched):
+    (xq int8 [I, B * kpad_group(T)], sx fp32 [B])."""
+    if not x.is_cuda or x.dim() != 3 or not x.is_contiguous():
+        raise RuntimeError("X must be a contiguous CUDA tensor [B, T, I]!")
+    B, T, I = x.shape
+    cfg = opt.to_c()
+    kg = kpad_group(T, opt)
+    xq = torch.empty((I, B * kg), dtype=torch.int8, device=x.device)
+    sx = torch.empty((B,), dtype=torch.float32, device=x.device)
+    ws = _ws(_lib.lib().hot_abc_batched_workspace_bytes(B, T, I, C.byref(cfg)), x.device)
+    _lib.check(_lib.lib().hot_abc_forward_batched(x.data_ptr(), _dt(x), B, T, I, C.byref(cfg), xq.data_ptr(), sx.data_ptr(),
+                                                  ws.data_ptr(), ws.numel(), _stream()))
+    return xq, sx
+
+
+def linear_backward_batched(gy: torch.Tensor, w: torch.Tensor, xq: torch.Tensor, sx: torch.Tensor, opt: HotOptions,
+                            out_dtype=None, workspace: Optional[torch.Tensor] = None):
+    """g_x [B, T, I] and g_W [O, I] (summed over the samples) for g_y [B, T, O] with one set of steps per
+    sample (hot_linear_backward_batched)."""
+    if not gy.is_cuda or gy.dim() != 3 or not gy.is_contiguous():
+        raise RuntimeError("Go must be a contiguous CUDA tensor [B, T, O]!")
+    _need_gpu_2d(w, "Wt")
+    B, T, O = gy.shape
+    if w.shape[0] != O or w.dtype != gy.dtype:
+        raise RuntimeError("W must be [O, I] with O = Go.shape[2], in the dtype of Go")
+    I = w.shape[1]
+    out_dtype = out_dtype or gy.dtype
+    cfg = opt.to_c()
+    kg = kpad_group(T, opt)
+    if tuple(xq.shape) != (I, B * kg) or xq.dtype != torch.int8 or sx.numel() != B:
+        raise RuntimeError("xq / sx must be the buffers written by abc_forward_batched")
+    need = _lib.lib().hot_backward_batched_workspace_bytes(B, T, O, I, C.byref(cfg))
+    if need == 0:
+        raise HotError("bad configuration: %s" % _lib.lib().hot_last_error().decode())
+    if workspace is None or workspace.numel() < need:
+        workspace = _ws(need, gy.device)
+    gx = torch.empty((B, T, I), dtype=out_dtype, device=gy.device)
+    gw = torch.empty((O, I), dtype=out_dtype, device=gy.device)
+    _lib.check(_lib.lib().hot_linear_backward_batched(gy.data_ptr(), w.data_ptr(), _dt(gy), xq.data_ptr(), sx.data_ptr(), B, T,
+                                                      O, I, C.byref(cfg), gx.data_ptr(), gw.data_ptr(), _DTYPES[out_dtype],
+                                                      workspace.data_ptr(), workspace.numel(), _stream()))
+    return gx, gw
+
+
 def measure_ceilings(device=None):
     """(copy GB/s, INT8 MFMA TOP/s) of this box from the library's two plain ceiling kernels."""
     device = device or torch.device("cuda", torch.cuda.current_device())

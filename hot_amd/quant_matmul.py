@@ -134,7 +134,7 @@ def _check_padding(w: Tensor, opt: ops.HotOptions) -> None:
 
 
 def _pad8(t: Tensor) -> Tensor:
-    """`t` (2-D) contiguous, its last dimension padded with zeros to a multiple of 8."""
+    """`t` contiguous, its last dimension padded with zeros to a multiple of 8."""
     extra = (-t.shape[-1]) % 8
     return F.pad(t, (0, extra)).contiguous() if extra else t.contiguous()
 
@@ -175,13 +175,20 @@ class FLinearQ(Function):
             return
         # the kernels move 16-byte vectors: feature counts that are not multiples of 8 are padded with
         # zero channels, which change neither a Hadamard block of the real channels nor any absmax
+        ctx.batched = False
         if x.dim() == 3 and args.batched_mode == "per_sample":
+            # the reference's treatment of 3-D activations: every sample has steps of its own
             tokens = x.shape[1]
             opt = options_for(tokens, name, w.shape[0])
             _check_padding(w, opt)
-            bufs = [ops.abc_forward(_pad8(x[b]), opt) for b in range(x.shape[0])]
-            xq = torch.stack([b[0] for b in bufs])
-            sx = torch.cat([b[1] for b in bufs])
+            if opt.hla_n <= 128:
+                # one call per layer: the library keeps the samples apart
+                ctx.batched = True
+                xq, sx = ops.abc_forward_batched(_pad8(x), opt)
+            else:
+                bufs = [ops.abc_forward(_pad8(x[b]), opt) for b in range(x.shape[0])]
+                xq = torch.stack([b[0] for b in bufs])
+                sx = torch.cat([b[1] for b in bufs])
         else:
             x2 = x.reshape(-1, x.shape[-1])
             opt = options_for(x2.shape[0], name, w.shape[0])
@@ -207,7 +214,10 @@ class FLinearQ(Function):
         wc = _pad8(_pad8(w).t()).t().contiguous() if (O % 8 or I % 8) else w.contiguous()   # [O8, I8]
         if go.dtype != wc.dtype:
             go = go.to(wc.dtype)
-        if go.dim() == 3 and args.batched_mode == "per_sample":
+        if go.dim() == 3 and args.batched_mode == "per_sample" and ctx.batched:
+            gx, grad_w = ops.linear_backward_batched(_pad8(go), wc, xq, sx, opt)
+            grad_input = gx[..., :I]
+        elif go.dim() == 3 and args.batched_mode == "per_sample":
             gxs, gw = [], None
             for b in range(go.shape[0]):
                 gx_b, gw_b = ops.linear_backward(_pad8(go[b]), wc, xq[b], sx[b:b + 1], opt)

@@ -218,6 +218,33 @@ HOT_API int hot_linear_backward_bias(const void* gy, const void* w, int dtype, c
                              void* workspace, size_t workspace_bytes, void* hip_stream);
 
 /*
+ * 3-D activations [B, T, C]: the reference vmaps its quantisers over the batch dimension, so every
+ * sample has steps of its own, applies the token-wise transform inside each sample and sums the
+ * per-sample weight gradients (utils/quant_matmul.py:33-37,102-106,118-122,288-290,322-324;
+ * utils/hadamard_matmul.py:143-161).  These two entry points take the B samples as the rows
+ * [b T, (b + 1) T) of the flattened tensors and do one call per layer:
+ *   hot_abc_forward_batched      xq [I, B * kg] int8, kg = hot_kpad_group(T, cfg) (the codes of sample b
+ *                                in bytes [b kg, (b + 1) kg) of every row, zero behind its T' codes),
+ *                                sx [B]; cfg->hla_n must divide T and be at most 128
+ *   hot_linear_backward_batched  g_x [B T, I], g_W [O, I] = sum over samples, each sample's integer
+ *                                sums dequantised with its own steps and added in fp32 in sample order
+ * Per-tensor steps become per-sample steps, per-token steps stay per token, per-channel steps of the g_W
+ * operand become per sample and channel.  Stochastic rounding numbers the elements as the flattened
+ * calls do.  Everything runs on `hip_stream` in order.
+ */
+HOT_API int64_t hot_kpad_group(int64_t T, const hot_config* cfg);
+HOT_API size_t hot_abc_batched_workspace_bytes(int64_t B, int64_t T, int64_t I, const hot_config* cfg);
+HOT_API int hot_abc_forward_batched(const void* x, int dtype, int64_t B, int64_t T, int64_t I,
+                            const hot_config* cfg, void* xq_out, float* sx_out, void* workspace,
+                            size_t workspace_bytes, void* hip_stream);
+HOT_API size_t hot_backward_batched_workspace_bytes(int64_t B, int64_t T, int64_t O, int64_t I,
+                                            const hot_config* cfg);
+HOT_API int hot_linear_backward_batched(const void* gy, const void* w, int dtype, const void* xq,
+                                const float* sx, int64_t B, int64_t T, int64_t O, int64_t I,
+                                const hot_config* cfg, void* gx, void* gw, int out_dtype,
+                                void* workspace, size_t workspace_bytes, void* hip_stream);
+
+/*
  * Number of K ranges into which the GEMMs inside hot_linear_backward cut a product of
  * M x N outputs over K codes of `bits` bits (1 = one kernel; more = a kernel per range
  * writing int32 partial tiles to the workspace, then a reduce kernel).  Products with

@@ -475,3 +475,69 @@ def stoch_round_mantissa(x: np.ndarray) -> np.ndarray:
     flip = (prob <= rnd).astype(np.int64)
     sign = np.where(x < 0, -1, 1)
     return sign * (np.floor(np.abs(x)).astype(np.int64) + flip)
+
+
+# --------------------------------------------------------------------------
+# 3-D activations [B, T, C]: one set of steps per sample
+# --------------------------------------------------------------------------
+
+
+def abc_forward_batched(x: np.ndarray, cfg: HotConfig):
+    """FLinearQ.setup_context on a 3-D input (quant_matmul.py:178-212 with the vmapped quantisers
+    :33-37,51-55,102-106,118-122 and the 3-D branch of lowering_matmul_back, hadamard_matmul.py:143-161):
+    per sample, x_b <- P x_b then quantise with a step of its own.  Stochastic rounding numbers the
+    elements as the flattened [B T, I] call does.  Returns (xq int8 [B, T', I], sx fp32 [B])."""
+    x = np.asarray(x, dtype=F32)
+    B, T, I = x.shape
+    rows = np.asarray(cfg.hla_rows)
+    nbs = T // cfg.hla_n
+    idx_all = colwise_rng_index(I, B * nbs, rows)                       # [I, B nbs r]
+    per = nbs * len(rows)
+    xq, sx = [], []
+    for b in range(B):
+        xp = fwht_blocks_first(x[b], cfg.hla_n, rows)
+        q, s = quant(xp, cfg.act_bits, cfg.act_scale, cfg.act_round, cfg.seed, STREAM_ACT,
+                     index=idx_all[:, b * per:(b + 1) * per].T)
+        xq.append(q)
+        sx.append(s[0])
+    return np.stack(xq), np.asarray(sx, dtype=F32)
+
+
+def linear_backward_batched(g_y: np.ndarray, w: np.ndarray, xq: np.ndarray, sx: np.ndarray, cfg: HotConfig):
+    """FLinearQ.backward on 3-D tensors (quant_matmul.py:215-348): the g_y quantisers run per sample
+    (per-tensor steps become per-sample steps; per-row steps stay per token for g_y H and become per
+    sample and channel for (P g_y)^T), W has one step, grad_input is computed per sample and the
+    per-sample weight gradients ((acc_b s_gw,b) s_x,b) are added up in fp32 in sample order
+    (autograd's sum over the batch dimension of the returned [B, O, I] tensor), then divided by n.
+    Returns (g_x [B, T, I], g_w [O, I], list of per-sample traces)."""
+    g_y = np.asarray(g_y, dtype=F32)
+    w = np.asarray(w, dtype=F32)
+    B, T, O = g_y.shape
+    I = w.shape[1]
+    rows = np.asarray(cfg.hla_rows)
+    nbs = T // cfg.hla_n
+    per = nbs * len(rows)
+    Wh = fwht_blocks_first(w, cfg.n_o)
+    qW, sW = quant(Wh, cfg.w_bits, cfg.w_scale, cfg.w_round, cfg.seed, STREAM_W,
+                   index=colwise_rng_index(Wh.shape[1], Wh.shape[0] // cfg.n_o, np.arange(cfg.n_o)).T)
+    gw_idx = colwise_rng_index(O, B * nbs, rows)                         # [O, B nbs r]
+    g_x = np.empty((B, T, I), dtype=F32)
+    g_w = np.zeros((O, I), dtype=F32)
+    traces = []
+    for b in range(B):
+        tr = BackwardTrace()
+        G = fwht_blocks_last(g_y[b], cfg.n_o)
+        gx_idx = (np.arange(b * T, (b + 1) * T, dtype=np.int64)[:, None] * O + np.arange(O, dtype=np.int64)[None, :])
+        tr.qG, tr.sG = quant(G, cfg.gx_bits, cfg.gx_scale, cfg.gx_round, cfg.seed, STREAM_GX, index=gx_idx)
+        tr.acc_x = int_gemm_nt(tr.qG, qW.T)
+        sg = tr.sG.reshape(-1, 1) if cfg.gx_scale == SCALE_ROW else tr.sG.reshape(1, 1)
+        g_x[b] = (((tr.acc_x.astype(F32) * sg).astype(F32) * sW[0]).astype(F32) / F32(cfg.n_o)).astype(F32)
+        GpT = np.ascontiguousarray(fwht_blocks_first(g_y[b], cfg.hla_n, rows).T)           # [O, T']
+        tr.qGp, tr.sGp = quant(GpT, cfg.gw_bits, cfg.gw_scale, cfg.gw_round, cfg.seed, STREAM_GW,
+                               index=gw_idx[:, b * per:(b + 1) * per])
+        tr.acc_w = int_gemm_nt(tr.qGp, np.asarray(xq[b]).T)
+        sgw = tr.sGp.reshape(-1, 1) if cfg.gw_scale == SCALE_ROW else tr.sGp.reshape(1, 1)
+        g_w = (g_w + ((tr.acc_w.astype(F32) * sgw).astype(F32) * F32(sx[b])).astype(F32)).astype(F32)
+        traces.append(tr)
+    g_w = (g_w / F32(cfg.hla_n)).astype(F32)
+    return g_x, g_w, traces

@@ -322,13 +322,51 @@ def test_hq_linear_3d_input(gpu, fresh_args, mode):
             gxs.append(tr.g_x)
             gw = gw + tr.g_w
         assert np.array_equal(x.grad.cpu().numpy(), np.stack(gxs))
-        assert rel(lin.weight.grad.cpu().numpy(), gw) < 1e-6
+        assert np.array_equal(lin.weight.grad.cpu().numpy(), gw)      # fp32 sum over the samples, in sample order
     else:
         ocfg, _ = both_configs(B * L)
         xq_ref, sx_ref = orc.abc_forward(x.detach().reshape(B * L, I).cpu().numpy(), ocfg)
         tr = orc.linear_backward(gy.reshape(B * L, O).cpu().numpy(), wn, xq_ref, sx_ref, ocfg)
         assert np.array_equal(x.grad.cpu().numpy().reshape(B * L, I), tr.g_x)
         assert np.array_equal(lin.weight.grad.cpu().numpy(), tr.g_w)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,T,O,I,variant", [
+    (5, 197, 208, 72, dict()),                                                    # ViT tokens: no block divides 197
+    (3, 64, 192, 160, dict(gx_scale=orc.SCALE_ROW, gw_scale=orc.SCALE_ROW)),      # n = 64, r = 36 inside every sample
+    (4, 196, 96, 264, dict(gx_round=orc.ROUND_STOCH, gw_round=orc.ROUND_STOCH, act_round=orc.ROUND_STOCH, seed=21)),
+    (2, 200, 128, 96, dict(w_scale=orc.SCALE_SAWB, act_scale=orc.SCALE_SAWB)),
+    (7, 48, 64, 40, dict(gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW, gw_round=orc.ROUND_STOCH,
+                         gw_scale=orc.SCALE_ROW, gx_bits=8, w_bits=8, seed=5)),
+    (130, 197, 128, 64, dict()),                                                  # more samples than a ViT batch
+])
+def test_backward_batched_matches_oracle(gpu, dtype, B, T, O, I, variant):
+    """3-D activations through the batched entry points (one call per layer, one set of steps per
+    sample): activation buffer, g_x and the summed g_W equal the per-sample oracle bit for bit."""
+    from hot_amd import ops
+    g = torch.Generator().manual_seed(B * T + O)
+    mag = 10.0 ** (torch.rand(B, 1, 1, generator=g) * 3 - 3)                       # samples of very different size
+    x = (torch.randn(B, T, I, generator=g) * (mag * 100)).to(dtype)
+    w = ((torch.rand(O, I, generator=g) * 2 - 1) / I ** 0.5).to(dtype)
+    gy = (torch.randn(B, T, O, generator=g) * mag).to(dtype)
+    ocfg = orc.HotConfig.python_rule(T, **variant)
+    opt = ops.HotOptions(n_o=ocfg.n_o, hla_n=ocfg.hla_n, hla_rows=ocfg.hla_rows, gx_bits=ocfg.gx_bits, w_bits=ocfg.w_bits,
+                         gw_bits=ocfg.gw_bits, act_bits=ocfg.act_bits, gx_round=ocfg.gx_round, w_round=ocfg.w_round,
+                         gw_round=ocfg.gw_round, act_round=ocfg.act_round, gx_scale=ocfg.gx_scale, w_scale=ocfg.w_scale,
+                         gw_scale=ocfg.gw_scale, act_scale=ocfg.act_scale, seed=ocfg.seed)
+    xq, sx = ops.abc_forward_batched(x.to(gpu), opt)
+    gx, gw = ops.linear_backward_batched(gy.to(gpu), w.to(gpu), xq, sx, opt)
+    xq_ref, sx_ref = orc.abc_forward_batched(x.float().numpy(), ocfg)
+    gx_ref, gw_ref, _ = orc.linear_backward_batched(gy.float().numpy(), w.float().numpy(), xq_ref, sx_ref, ocfg)
+    kg = ops.kpad_group(T, opt)
+    tp = xq_ref.shape[1]
+    got = xq.cpu().numpy().reshape(I, B, kg)
+    assert kg % 128 == 0 and kg >= tp
+    assert np.array_equal(got[:, :, :tp], xq_ref.transpose(2, 0, 1)) and not got[:, :, tp:].any()
+    assert np.array_equal(sx.cpu().numpy(), sx_ref)
+    assert torch.equal(gx.cpu(), torch.from_numpy(gx_ref).to(dtype))
+    assert torch.equal(gw.cpu(), torch.from_numpy(gw_ref).to(dtype))
 
 
 def test_hq_conv2d_matches_oracle(gpu, fresh_args):

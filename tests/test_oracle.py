@@ -370,3 +370,42 @@ def test_oracle_matches_its_frozen_snapshots(name):
     assert set(frozen.files) == set(fresh)
     for k in frozen.files:
         assert np.array_equal(frozen[k], np.asarray(fresh[k])), k
+
+
+# ------------------------------------------------------------------ 3-D activations (per-sample steps)
+
+def test_batched_oracle_reduces_to_the_2d_path():
+    """One sample: the batched functions are the 2-D ones, stochastic rounding included (the element
+    numbering coincides).  Several samples under round-to-nearest: every sample is an independent 2-D
+    problem with steps of its own, g_x stacks and g_W adds (n is a power of two, so dividing each
+    sample's gradient by n or the sum gives the same fp32 numbers)."""
+    rng = np.random.default_rng(3)
+    B, T, O, I = 3, 32, 48, 24
+    x = rng.standard_normal((B, T, I)).astype(np.float32)
+    w = rng.standard_normal((O, I)).astype(np.float32) * 0.1
+    gy = (rng.standard_normal((B, T, O)) * np.array([1e-3, 5e-2, 2.0])[:, None, None]).astype(np.float32)
+    n, rows = orc.hla_rows(T)
+    assert n == 32
+    for kw in (dict(), dict(gx_scale=orc.SCALE_ROW, gw_scale=orc.SCALE_ROW), dict(act_scale=orc.SCALE_SAWB, w_scale=orc.SCALE_SAWB)):
+        cfg = orc.HotConfig(hla_n=n, hla_rows=tuple(int(v) for v in rows), **kw)
+        xq, sx = orc.abc_forward_batched(x, cfg)
+        gx, gw, traces = orc.linear_backward_batched(gy, w, xq, sx, cfg)
+        acc = np.zeros((O, I), dtype=np.float32)
+        for b in range(B):
+            xq_b, sx_b = orc.abc_forward(x[b], cfg)
+            assert np.array_equal(xq[b], xq_b) and sx[b] == sx_b[0]
+            tr = orc.linear_backward(gy[b], w, xq_b, sx_b, cfg)
+            assert np.array_equal(gx[b], tr.g_x)
+            assert np.array_equal(traces[b].qG, tr.qG) and np.array_equal(traces[b].qGp, tr.qGp)
+            acc = (acc + tr.g_w).astype(np.float32)
+        assert np.array_equal(gw, acc)
+        # the three samples differ by orders of magnitude: shared steps would crush the small ones
+        assert len({float(s) for s in sx}) == B and traces[0].sG.max() < traces[2].sG.min()
+    cfg = orc.HotConfig(hla_n=n, hla_rows=tuple(int(v) for v in rows), gx_round=orc.ROUND_STOCH, gw_round=orc.ROUND_STOCH,
+                        act_round=orc.ROUND_STOCH, seed=77)
+    xq1, sx1 = orc.abc_forward_batched(x[:1], cfg)
+    xq2, sx2 = orc.abc_forward(x[0], cfg)
+    assert np.array_equal(xq1[0], xq2) and sx1[0] == sx2[0]
+    gx1, gw1, _ = orc.linear_backward_batched(gy[:1], w, xq1, sx1, cfg)
+    tr = orc.linear_backward(gy[0], w, xq2, sx2, cfg)
+    assert np.array_equal(gx1[0], tr.g_x) and np.array_equal(gw1, tr.g_w)
