@@ -429,20 +429,17 @@ def vit_b16_backward(dev, batch=128, steps=3):
         hot, hot_all = backward_ms(model)
         picks = list(args.layer_quant_dict.values())
         # the reference's own treatment of 3-D activations: every sample a problem of its own (197
-        # tokens: no low-rank projection, one step per sample), here one library call per sample
+        # tokens: no block divides them, so no low-rank projection; one step per sample), one
+        # library call per layer
         args.batched_mode = "per_sample"
-        saved_steps, steps = steps, 1
-        try:
-            per_sample, _ = backward_ms(model)
-        finally:
-            steps = saved_steps
+        per_sample, _ = backward_ms(model)
     finally:
         for k, v in saved.items():
             setattr(args, k, v)
         args.layer_quant_dict.clear()
     return {"model": "ViT-B/16, batch %d, bf16, flattened tokens" % batch, "backward_ms_plain_bf16": round(plain, 2),
             "backward_ms_hot": round(hot, 2), "forward_backward_ms_plain_bf16": round(plain_all, 2),
-            "forward_backward_ms_hot": round(hot_all, 2), "backward_ms_hot_per_sample_calls": round(per_sample, 1),
+            "forward_backward_ms_hot": round(hot_all, 2), "backward_ms_hot_per_sample_steps": round(per_sample, 2),
             "hot_layers": len(picks) // 2,
             "per_token_quantiser_layers": sum(1 for i, v in enumerate(picks) if i % 2 == 0 and v == "norm_quantizer")}
 

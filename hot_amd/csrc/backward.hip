@@ -463,7 +463,7 @@ int hot_linear_backward_bias(const void* gy, const void* w, int dtype, const voi
 
 struct BatchedLayout {
   int64_t ld_g, ld_w, kg, ld_gp;
-  size_t off_colw, off_colg, off_hq, off_sg, off_sw, off_sgp, off_qg, off_qw, off_qgp, total;
+  size_t off_colw, off_colg, off_hq, off_sg, off_sw, off_sgp, off_qg, off_qw, off_qgp, off_part, part_bytes, total;
 };
 
 static int64_t kpad_group(int64_t T, const hot_config* c) { return round_up((T / c->hla_n) * c->hla_r, 128); }
@@ -485,6 +485,8 @@ static BatchedLayout batched_layout(int64_t B, int64_t T, int64_t O, int64_t I, 
   b.off_qg = o;   o += align256((size_t)L * b.ld_g);
   b.off_qw = o;   o += align256((size_t)I * b.ld_w);
   b.off_qgp = o;  o += align256((size_t)O * b.ld_gp);
+  b.part_bytes = gemm_grouped_workspace_bytes_impl(O, I, (int)B, b.kg);
+  b.off_part = o; o += align256(b.part_bytes);
   b.total = o;
   return b;
 }
@@ -517,6 +519,11 @@ int hot_abc_forward_batched(const void* x, int dtype, int64_t B, int64_t T, int6
   return colwise_quant_impl(x, dtype, B * T, I, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, cfg->act_bits, cfg->act_round, cfg->seed,
                             HOT_STREAM_ACT, cfg->act_scale, xq_out, B * kg, 0, sx_out, workspace, workspace_bytes,
                             (hipStream_t)hip_stream, who, nullptr, false, nullptr, nullptr, (int)B, kg);
+}
+
+int hot_backward_batched_ranges(int64_t B, int64_t T, int64_t O, int64_t I, const hot_config* cfg) {
+  if (check_batched(cfg, B, T, "hot_backward_batched_ranges") || O <= 0 || I <= 0) return 0;
+  return gemm_grouped_splits_impl(O, I, (int)B, kpad_group(T, cfg));
 }
 
 size_t hot_backward_batched_workspace_bytes(int64_t B, int64_t T, int64_t O, int64_t I, const hot_config* cfg) {
@@ -565,7 +572,7 @@ int hot_linear_backward_batched(const void* gy, const void* w, int dtype, const 
   if (rc) return rc;
   // g_W = sum over samples of (qGp_b . xq_b^T) sGp_b sx_b / hla_n
   return gemm_i8_grouped_impl(ws + b.off_qgp, b.ld_gp, xq, b.ld_gp, O, I, (int)B, b.kg, sgp, cfg->gw_scale == HOT_SCALE_ROW, sx,
-                              1.0f / (float)cfg->hla_n, gw, out_dtype, I, st);
+                              1.0f / (float)cfg->hla_n, gw, out_dtype, I, ws + b.off_part, b.part_bytes, st);
 }
 
 int hot_linear_backward_kernels(const void* gy, const void* w, int dtype, const void* xq, const float* sx, int64_t L,

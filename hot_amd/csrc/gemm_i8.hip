@@ -51,12 +51,19 @@ struct GemmArgs {
   int32_t vec16;     // out and its row pitch are 16-byte aligned (staged epilogue)
   int32_t splits;    // K is cut into this many ranges, one workgroup each (1 = no split)
   v4i* partials;     // [tile][range][wave][fragment quad][lane]: raw accumulators of the ranges
-  // K groups (3-D activations: a group is a sample with steps of its own): every group_stages
-  // stages the integer accumulators are dequantised with the group's steps and added, in group order,
-  // to fp32 accumulators: out = (sum over groups of (float(acc_g) * sa_g[row or 0]) * sb_g) * post_scale
-  int32_t group_stages;     // stages (of the kernel's stage width) per group; 0 = one group, integer all the way
+  // K groups (gemm_i8_grouped_kernel; 3-D activations: a group is a sample with steps of its own).
+  // The integer sums of every group are dequantised with the group's steps and added, in group
+  // order, to fp32 accumulators:
+  //   out = (sum over groups of (float(acc_g) * sa_g[row or 0]) * sb_g) * post_scale.
+  // With gsplits > 1 the groups are cut into gsplits contiguous ranges, one workgroup each; every
+  // range leaves its fp32 sum in gpart and a second kernel adds the ranges in order.
+  int32_t groups;
+  int32_t group_stages;     // 128-byte stages per group
+  int32_t gsplits, gper;    // ranges and groups per range
   const float* gscale_a;    // [groups] or, with a_per_row, [groups][M]
   const float* gscale_b;    // [groups]
+  float* gpart;             // [gsplits][M][ldp] fp32
+  int64_t ldp;
 };
 
 // Workgroup -> tile.  Hardware deals consecutive workgroup ids round-robin to the 8 XCDs, each with
@@ -628,7 +635,7 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
 // ---------------------------------------------------------------------------
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-template <int WM, int WN, int GM, int GN, int BITS, int S, int RB, typename OutT, bool GROUPED = false>
+template <int WM, int WN, int GM, int GN, int BITS, int S, int RB, typename OutT>
 __global__ void __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(1, (WM * WN <= 8 ? 2 : 1))))
 gemm_i8_slot_kernel(const GemmArgs g) {
   static_assert(GM * GN == 4, "four waves");
@@ -755,50 +762,6 @@ gemm_i8_slot_kernel(const GemmArgs g) {
   };
   constexpr int EPS_ = BITS == 4 ? (4 * NR + H - 1) / H : 0;     // expansion items per slot of a half round
 
-  // K groups: fp32 accumulators, the steps of the current group (loaded a group ahead), a stage counter
-  v16f facc[GROUPED ? WM : 1][GROUPED ? WN : 1];
-  float gsa[GROUPED ? WM : 1], gsb = 0.f;
-  int gstage = 0, gidx = 0;
-  auto load_group_scales = [&](int gi) {
-    if constexpr (GROUPED) {
-#pragma unroll
-      for (int i = 0; i < WM; ++i) {
-        const int64_t row = row0 + wm * WM * 32 + i * 32 + (lane & 31);
-        gsa[i] = g.a_per_row ? g.gscale_a[(int64_t)gi * g.M + (row < g.M ? row : g.M - 1)] : g.gscale_a[gi];
-      }
-      gsb = g.gscale_b[gi];
-    }
-  };
-  if constexpr (GROUPED) {
-#pragma unroll
-    for (int i = 0; i < WM; ++i)
-#pragma unroll
-      for (int j = 0; j < WN; ++j) facc[i][j] = (v16f)(0.f);
-    load_group_scales(0);
-  }
-  // end of a stage: when it closes a group, dequantise the group's sums into the fp32 accumulators
-  auto stage_done = [&](int kt) {
-    if constexpr (GROUPED) {
-      if (++gstage == g.group_stages) {
-        gstage = 0;
-#pragma unroll
-        for (int i = 0; i < WM; ++i)
-#pragma unroll
-          for (int j = 0; j < WN; ++j) {
-            // the product is rounded before it is added (no fused multiply-add): the sum over the
-            // groups is the fp32 sum of the per-group results
-#pragma clang fp contract(off)
-            v16i a = acc[i][j];
-            if constexpr (BITS == 4) a = a >> 8;
-            facc[i][j] += (__builtin_convertvector(a, v16f) * gsa[i]) * gsb;
-            acc[i][j] = a - a;
-          }
-        ++gidx;
-        if (kt + 1 < KT) load_group_scales(gidx);
-      }
-    }
-  };
-
   // prologue: S tiles in flight, tile 0 landed and visible, its first round in registers
   static_for<S>([&](auto k) {
     if (k.value < KT) {
@@ -858,45 +821,15 @@ gemm_i8_slot_kernel(const GemmArgs g) {
   auto rotation = [&](auto steady, int kt0) {
     static_for<S>([&](auto k) {
       constexpr int K = decltype(k)::value;
-      if (decltype(steady)::value || kt0 + K < KT) {
+      if (decltype(steady)::value || kt0 + K < KT)
         ktile(steady, std::integral_constant<int, K * STAGE_BYTES>{}, std::integral_constant<int, ((K + 1) % S) * STAGE_BYTES>{},
               kt0 + K);
-        stage_done(kt0 + K);
-      }
     });
   };
   int kt0 = 0;
   for (; kt0 + 2 * S - 1 < KT; kt0 += S) rotation(std::true_type{}, kt0);   // every tile inside has a tile kt + S
   for (; kt0 < KT; kt0 += S) rotation(std::false_type{}, kt0);
 
-  if constexpr (GROUPED) {
-    // the sums are dequantised already: scale once more and store, four adjacent outputs per lane
-    OutT* out = reinterpret_cast<OutT*>(g.out);
-    const int half = lane >> 5;
-#pragma unroll
-    for (int i = 0; i < WM; ++i) {
-      const int64_t row = row0 + wm * WM * 32 + i * 32 + (lane & 31);
-      if (row >= g.M) continue;
-#pragma unroll
-      for (int j = 0; j < WN; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          const int64_t col = col0 + wn * WN * 32 + j * 32 + 8 * q + 4 * half;
-          if (col >= g.N) continue;
-          if (g.vec_out && col + 3 < g.N) {
-            typename Quad<OutT>::type v;
-#pragma unroll
-            for (int t = 0; t < 4; ++t) quad_set<OutT>(v, t, facc[i][j][4 * q + t] * g.post_scale);
-            *reinterpret_cast<typename Quad<OutT>::type*>(out + row * g.ldo + col) = v;
-          } else {
-#pragma unroll
-            for (int t = 0; t < 4; ++t)
-              if (col + t < g.N) store_scalar<OutT>(out + row * g.ldo + col + t, facc[i][j][4 * q + t] * g.post_scale);
-          }
-        }
-    }
-    return;
-  }
   if constexpr (!EARLY_SCALES) {
     load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
     sb = g.scale_b[0];
@@ -909,6 +842,277 @@ gemm_i8_slot_kernel(const GemmArgs g) {
     return;
   }
   gemm_epilogue<WM, WN, BITS, OutT>(acc, g, row0 + wm * WM * 32, col0 + wn * WN * 32, lane, sa_row, sb);
+}
+
+// ---------------------------------------------------------------------------
+// K groups with steps of their own (3-D activations: the K range of sample b holds the codes of
+// sample b, and the reference dequantises every sample's product with that sample's steps before
+// the sum over the batch, utils/quant_matmul.py:322-324 and the batch sum of autograd).
+// INT8 operands, 128 x 128 tiles, the data path of the slot-scheduled kernel with 128-byte stage
+// rows.  When a group ends, its integer sums are moved aside and, while the next group accumulates,
+// converted, scaled twice (rounded after each product, as the reference's two multiplications are)
+// and added to the fp32 accumulators, a few elements per MFMA slot, so the conversion rides in the
+// shadow of the matrix pipe.  The first MFMA of a group takes a zero C operand, which replaces
+// clearing the accumulators.  The ring stage is a run-time offset (a group may be any number of
+// stages long).
+// ---------------------------------------------------------------------------
+template <typename OutT>
+__global__ void __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(1, 1)))
+gemm_i8_grouped_kernel(const GemmArgs g) {
+  constexpr int WM = 2, WN = 2, GN = 2, S = 4, RB = 128;
+  constexpr int BM = 128, BN = 128;
+  constexpr int SPR = RB / 16, RPC = 1024 / RB, RPS = RB / 32;
+  constexpr int ROWS = BM + BN, CHUNKS = ROWS / RPC, LPW = CHUNKS / 4;
+  constexpr int STAGE_BYTES = ROWS * RB;
+  constexpr int NF = WM * WN, NM = NF, NR = WM + WN;
+  constexpr int DPS = (LPW + NM - 1) / NM;
+  __shared__ __attribute__((aligned(1024))) uint8_t ring[S * STAGE_BYTES];
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = wave / GN, wn = wave % GN;
+  const int tiles_total = g.tiles_m * g.tiles_n;
+  int tm, tn, split = 0;
+  {
+    const int u = xcd_chunk_position(tiles_total * g.gsplits, (int)blockIdx.x);
+    split = u / tiles_total;
+    grouped_tile(g, u - split * tiles_total, tm, tn);
+  }
+  const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
+  const int g_lo = split * g.gper;
+  const int g_hi = g_lo + g.gper < g.groups ? g_lo + g.gper : g.groups;
+  const int gs = g.group_stages;
+  const int KT = (g_hi - g_lo) * gs;                       // stages of this range
+  const int64_t kbase = (int64_t)g_lo * gs * RB;           // byte offset of the range in every operand row
+
+  uint32_t goff[LPW], ldst[LPW];
+  uint32_t is_b = 0;
+#pragma unroll
+  for (int i = 0; i < LPW; ++i) {
+    const int c = 4 * i + wave;
+    ldst[i] = (uint32_t)c * 1024u;
+    const int r = c * RPC + lane / SPR;
+    const int slot = (lane % SPR) ^ ((r >> 1) & 7);
+    if (c * RPC < BM) {
+      int64_t gr = row0 + r;
+      if (gr >= g.M) gr = g.M - 1;
+      goff[i] = (uint32_t)(gr * g.lda + slot * 16);
+    } else {
+      int64_t gr = col0 + (r - BM);
+      if (gr >= g.N) gr = g.N - 1;
+      goff[i] = (uint32_t)(gr * g.ldb + slot * 16);
+      is_b |= 1u << i;
+    }
+  }
+  is_b = (uint32_t)__builtin_amdgcn_readfirstlane((int)is_b);
+  const uint32_t ring0 = lds_offset(ring);
+  const uint8_t* const a_base = g.A + kbase;
+  const uint8_t* const b_base = g.B + kbase;
+  auto dma_one = [&](uint32_t stage_off, int kt, int i) {
+    const uint64_t b64 = (uint64_t)(uintptr_t)(((is_b >> i) & 1u ? b_base : a_base) + (int64_t)kt * RB);
+    const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b64 >> 32));
+    const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b64);
+    dma16(ring0 + stage_off + ldst[i], goff[i], reinterpret_cast<const uint8_t*>(((uint64_t)b_hi << 32) | (uint64_t)b_lo));
+  };
+
+  // acc: integer sums of the group in progress; held: the finished sums of the group before it,
+  // on their way into facc, the fp32 result
+  v16i acc[WM][WN], held[WM][WN];
+  v16f facc[WM][WN];
+#pragma unroll
+  for (int i = 0; i < WM; ++i)
+#pragma unroll
+    for (int j = 0; j < WN; ++j) {
+      facc[i][j] = (v16f)(0.f);
+#pragma unroll
+      for (int e = 0; e < 16; ++e) { acc[i][j][e] = 0; held[i][j][e] = 0; }
+    }
+  // steps of the group being accumulated (c*) and of the held group (p*): all zero before the
+  // first group, so that folding "the group before the first" adds nothing
+  float csa[WM], psa[WM], csb = 0.f, psb = 0.f;
+#pragma unroll
+  for (int i = 0; i < WM; ++i) { csa[i] = 0.f; psa[i] = 0.f; }
+  auto next_group_scales = [&](int gi) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+      const int64_t row = row0 + wm * WM * 32 + i * 32 + (lane & 31);
+      psa[i] = csa[i];
+      csa[i] = g.a_per_row ? g.gscale_a[(int64_t)gi * g.M + (row < g.M ? row : g.M - 1)] : g.gscale_a[gi];
+    }
+    psb = csb;
+    csb = g.gscale_b[gi];
+  };
+
+  v4i fr[2][NR];
+  const int frow = lane & 31, fhalf = lane >> 5;
+  const int sw = (frow >> 1) & 7;
+  const int offA = (wm * 32 * WM + frow) * RB, offB = (BM + wn * 32 * WN + frow) * RB;
+  auto frag_off = [&](int t) { return t == 0 ? offA : (t <= WN ? offB + (t - 1) * 32 * RB : offA + (t - WN) * 32 * RB); };
+  auto read_frag = [&](const uint8_t* stage, int d, int t) {
+    const int so = ((2 * d + fhalf) ^ sw) * 16;
+    fr[d & 1][t] = *reinterpret_cast<const v4i*>(stage + frag_off(t) + so);
+  };
+  auto a_of = [](int i) { return i == 0 ? 0 : WN + i; };
+  auto b_of = [](int j) { return 1 + j; };
+
+  // prologue: up to S tiles in flight, tile 0 landed and visible, its first round in registers
+#pragma unroll
+  for (int k = 0; k < S; ++k)
+    if (k < KT) {
+#pragma unroll
+      for (int i = 0; i < LPW; ++i) dma_one((uint32_t)(k * STAGE_BYTES), k, i);
+    }
+  wait_dma_upto<S - 1, LPW>((KT < S ? KT : S) - 1);
+  __builtin_amdgcn_s_barrier();
+#pragma unroll
+  for (int t = 0; t < NR; ++t) read_frag(ring, 0, t);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // One stage (16 slots: 4 rounds of 4 MFMAs).  FIRST: the stage opens a group: in round 0 the
+  // slot of fragment f moves the finished sums of f aside (acc -> held) and restarts f with a zero
+  // C operand.  The 64 held sums are folded into facc in QT "fold slots" (the slots of rounds 1-3
+  // of the opening stage and, for groups of two stages or more, all slots of the second stage);
+  // this stage owns the fold slots from Q0 on.  QT = 0: no folding in this stage.
+  auto stage = [&](auto firstc, auto q0c, auto qtc, int kt) {
+    constexpr bool FIRST = decltype(firstc)::value;
+    constexpr int Q0 = decltype(q0c)::value, QT = decltype(qtc)::value;
+    const uint32_t cur_off = (uint32_t)(kt & (S - 1)) * STAGE_BYTES;
+    const uint8_t* cur = ring + cur_off;
+    const uint8_t* nxt = ring + (uint32_t)((kt + 1) & (S - 1)) * STAGE_BYTES;
+    const bool more = kt + 1 < KT, refill = kt + S < KT;
+    static_for<RPS>([&](auto rc) {
+      constexpr int r = decltype(rc)::value, p = r & 1;
+      constexpr bool LAST = r == RPS - 1;
+      if constexpr (LAST) {
+        if (more) {
+          wait_dma_upto<S - 2, LPW, true>((kt + S - 1 < KT - 1 ? kt + S - 1 : KT - 1) - (kt + 1));
+          __builtin_amdgcn_s_barrier();
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      static_for<NM>([&](auto mc) {
+        constexpr int m = decltype(mc)::value;
+        if constexpr (LAST) {
+#pragma unroll
+          for (int i = m * DPS; i < (m + 1) * DPS && i < LPW; ++i)
+            if (refill) dma_one(cur_off, kt + S, i);
+        }
+        if constexpr (!LAST) read_frag(cur, r + 1, m);
+        else if (more) read_frag(nxt, 0, m);
+        constexpr int q = FIRST ? Q0 + (r - 1) * NM + m : Q0 + r * NM + m;      // fold slot of this slot
+        if constexpr (QT > 0 && (!FIRST || r >= 1) && q < QT) {
+          // the product is rounded before it is added (no fused multiply-add): the sum over the
+          // groups is the fp32 sum of the per-group results
+#pragma clang fp contract(off)
+          constexpr int E0 = q * 16 * NF / QT, E1 = (q + 1) * 16 * NF / QT;
+#pragma unroll
+          for (int e = E0; e < E1; ++e) {
+            const int f = e / 16, k = e % 16, i = f / WN, j = f % WN;
+            facc[i][j][k] += ((float)held[i][j][k] * psa[i]) * psb;
+          }
+        }
+        const int i = m / WN, j = m % WN;
+        if constexpr (FIRST && r == 0) {
+          const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+          held[i][j] = acc[i][j];
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[p][b_of(j)], fr[p][a_of(i)], zero, 0, 0, 0);
+        } else {
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[p][b_of(j)], fr[p][a_of(i)], acc[i][j], 0, 0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      });
+    });
+  };
+  using I0 = std::integral_constant<int, 0>;
+  constexpr int Q1 = (RPS - 1) * NM, Q2 = Q1 + RPS * NM;     // fold slots of the opening stage, and of two stages
+  int kt = 0;
+  for (int gi = g_lo; gi < g_hi; ++gi) {
+    next_group_scales(gi);
+    if (gs == 1) {
+      stage(std::true_type{}, I0{}, std::integral_constant<int, Q1>{}, kt++);
+    } else {
+      stage(std::true_type{}, I0{}, std::integral_constant<int, Q2>{}, kt++);
+      stage(std::false_type{}, std::integral_constant<int, Q1>{}, std::integral_constant<int, Q2>{}, kt++);
+      for (int s2 = 2; s2 < gs; ++s2) stage(std::false_type{}, I0{}, I0{}, kt++);
+    }
+  }
+  // the last group's sums
+  {
+#pragma clang fp contract(off)
+#pragma unroll
+    for (int i = 0; i < WM; ++i)
+#pragma unroll
+      for (int j = 0; j < WN; ++j) facc[i][j] += (__builtin_convertvector(acc[i][j], v16f) * csa[i]) * csb;
+  }
+
+  const int half = lane >> 5;
+  if (g.gsplits > 1) {
+    // this range's sum, unscaled; gemm_i8_grouped_reduce_kernel adds the ranges in order
+    float* part = g.gpart + (int64_t)split * g.M * g.ldp;
+#pragma unroll
+    for (int i = 0; i < WM; ++i) {
+      const int64_t row = row0 + wm * WM * 32 + i * 32 + (lane & 31);
+      if (row >= g.M) continue;
+#pragma unroll
+      for (int j = 0; j < WN; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int64_t col = col0 + wn * WN * 32 + j * 32 + 8 * q + 4 * half;
+          if (col >= g.ldp) continue;          // ldp is N rounded up to 4: whole quads
+          typedef float f4 __attribute__((ext_vector_type(4)));
+          const f4 v = {facc[i][j][4 * q], facc[i][j][4 * q + 1], facc[i][j][4 * q + 2], facc[i][j][4 * q + 3]};
+          *reinterpret_cast<f4*>(part + row * g.ldp + col) = v;
+        }
+    }
+    return;
+  }
+  OutT* out = reinterpret_cast<OutT*>(g.out);
+#pragma unroll
+  for (int i = 0; i < WM; ++i) {
+    const int64_t row = row0 + wm * WM * 32 + i * 32 + (lane & 31);
+    if (row >= g.M) continue;
+#pragma unroll
+    for (int j = 0; j < WN; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int64_t col = col0 + wn * WN * 32 + j * 32 + 8 * q + 4 * half;
+        if (col >= g.N) continue;
+        if (g.vec_out && col + 3 < g.N) {
+          typename Quad<OutT>::type v;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) quad_set<OutT>(v, t, facc[i][j][4 * q + t] * g.post_scale);
+          *reinterpret_cast<typename Quad<OutT>::type*>(out + row * g.ldo + col) = v;
+        } else {
+#pragma unroll
+          for (int t = 0; t < 4; ++t)
+            if (col + t < g.N) store_scalar<OutT>(out + row * g.ldo + col + t, facc[i][j][4 * q + t] * g.post_scale);
+        }
+      }
+  }
+}
+
+// out = (part[0] + part[1] + ... in this order) * post_scale, one thread per four adjacent outputs
+template <typename OutT>
+__global__ void __launch_bounds__(256) gemm_i8_grouped_reduce_kernel(const GemmArgs g) {
+  typedef float f4 __attribute__((ext_vector_type(4)));
+  const int64_t quads_row = g.ldp / 4;
+  const int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (id >= g.M * quads_row) return;
+  const int64_t row = id / quads_row, col = (id - row * quads_row) * 4;
+  const float* p = g.gpart + row * g.ldp + col;
+  f4 s = *reinterpret_cast<const f4*>(p);
+  for (int k = 1; k < g.gsplits; ++k) s += *reinterpret_cast<const f4*>(p + (int64_t)k * g.M * g.ldp);
+  OutT* out = reinterpret_cast<OutT*>(g.out);
+  if (g.vec_out && col + 3 < g.N) {
+    typename Quad<OutT>::type v;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) quad_set<OutT>(v, t, s[t] * g.post_scale);
+    *reinterpret_cast<typename Quad<OutT>::type*>(out + row * g.ldo + col) = v;
+  } else {
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+      if (col + t < g.N) store_scalar<OutT>(out + row * g.ldo + col + t, s[t] * g.post_scale);
+  }
 }
 
 // Second kernel of a split-K product: one single-wave workgroup per 32 x 32 accumulator fragment,
@@ -960,7 +1164,7 @@ static int launch_gemm_pipe(GemmArgs& g, hipStream_t st) {
   return check_launch("gemm_i8_pipe_kernel");
 }
 
-template <int WM, int WN, int GM, int GN, int BITS, int S, int RB, typename OutT, bool GROUPED = false>
+template <int WM, int WN, int GM, int GN, int BITS, int S, int RB, typename OutT>
 static int launch_gemm_slot(GemmArgs& g, hipStream_t st) {
   constexpr int BM = 32 * WM * GM, BN = 32 * WN * GN;
   g.tiles_m = (int)((g.M + BM - 1) / BM);
@@ -970,7 +1174,7 @@ static int launch_gemm_slot(GemmArgs& g, hipStream_t st) {
   if (total > (1 << 30)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: too many tiles");
   if (g.M * g.lda >= (1ll << 32) || g.N * g.ldb >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: operand larger than 4 GiB");
   if (((int64_t)g.ktiles * (G_BK * BITS / 8)) % RB) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: this kernel takes rows of a multiple of %d bytes", RB);
-  hipLaunchKernelGGL((gemm_i8_slot_kernel<WM, WN, GM, GN, BITS, S, RB, OutT, GROUPED>), dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
+  hipLaunchKernelGGL((gemm_i8_slot_kernel<WM, WN, GM, GN, BITS, S, RB, OutT>), dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
   return check_launch("gemm_i8_slot_kernel");
 }
 
@@ -1115,7 +1319,7 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
   g.vec_out = ((ldo & 3) == 0 && ((uintptr_t)out & 15) == 0) ? 1 : 0;
   g.vec16 = (((uintptr_t)out & 15) == 0 && ((ldo * (out_dtype == HOT_F32 ? 4 : 2)) & 15) == 0) ? 1 : 0;
   g.splits = 1; g.partials = nullptr;
-  g.group_stages = 0; g.gscale_a = nullptr; g.gscale_b = nullptr;
+  g.groups = 0; g.group_stages = 0; g.gsplits = 1; g.gper = 0; g.gscale_a = nullptr; g.gscale_b = nullptr; g.gpart = nullptr; g.ldp = 0;
   if (variant == HOT_GEMM_DMA_128_SPLITK) {
     const GemmSplit plan = gemm_split_plan(M, N, K, bits);
     if (plan.splits < 2) return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: the split-K kernel needs a product of fewer than 256 tiles of 128 x 128 and a long K");
@@ -1130,9 +1334,36 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
 // INT8 product whose K dimension is `groups` samples of group_k codes each (a multiple of 128), every
 // sample with steps of its own: out = (sum_g (float(acc_g) * sa[g][row or 0]) * sb[g]) * post_scale,
 // the groups added in order in fp32.  128 x 128 tiles, slot-scheduled, one workgroup per tile.
+// Ranges of groups a grouped product is cut into (a function of the shape alone, so that the order
+// of the fp32 sum is reproducible: ranges of ceil(groups / ranges) consecutive groups, each summed in
+// group order, the range sums added in range order).  One workgroup per tile and range occupies a
+// CU; few tiles with many groups leave most of the 256 CUs idle unless the groups are shared out,
+// and every range costs a round trip of the fp32 result.
+int gemm_grouped_splits_impl(int64_t M, int64_t N, int groups, int64_t group_k) {
+  if (M <= 0 || N <= 0 || groups <= 1 || group_k <= 0) return 1;
+  const int64_t tiles = ((M + 127) / 128) * ((N + 127) / 128);
+  const double t_group = 0.55 * (double)group_k / 256.0;            // us per group and tile
+  const double t_part = (double)M * (double)N * 8.0 / 3.0e6;        // us per range: partial written and read
+  int best = 1;
+  double t_best = (double)((tiles + 255) / 256) * groups * t_group;
+  const int smax = groups < 32 ? groups : 32;
+  for (int sp = 2; sp <= smax; ++sp) {
+    const int per = (groups + sp - 1) / sp;
+    if ((sp - 1) * per >= groups) continue;                         // not a partition into sp non-empty ranges
+    const double t = (double)((tiles * sp + 255) / 256) * per * t_group + sp * t_part + 3.0;
+    if (t < t_best * 0.97) { t_best = t; best = sp; }
+  }
+  return best;
+}
+
+size_t gemm_grouped_workspace_bytes_impl(int64_t M, int64_t N, int groups, int64_t group_k) {
+  const int sp = gemm_grouped_splits_impl(M, N, groups, group_k);
+  return sp > 1 ? (size_t)sp * (size_t)M * (size_t)round_up(N, 4) * 4 : 0;
+}
+
 int gemm_i8_grouped_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t M, int64_t N, int groups,
                          int64_t group_k, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
-                         void* out, int out_dtype, int64_t ldo, hipStream_t st) {
+                         void* out, int out_dtype, int64_t ldo, void* workspace, size_t workspace_bytes, hipStream_t st) {
   const char* who = "hot_gemm_i8_grouped";
   if (!A || !B || !scale_a || !scale_b || !out) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
   if (M < 0 || N < 0 || groups < 1 || group_k <= 0 || (group_k % 128)) return fail(HOT_ERR_INVALID, "%s: bad shape %lld x %lld, %d groups of %lld codes (a multiple of 128)", who, (long long)M, (long long)N, groups, (long long)group_k);
@@ -1151,13 +1382,39 @@ int gemm_i8_grouped_impl(const void* A, int64_t lda, const void* B, int64_t ldb,
   g.vec_out = ((ldo & 3) == 0 && ((uintptr_t)out & 15) == 0) ? 1 : 0;
   g.vec16 = 0;
   g.splits = 1; g.partials = nullptr;
-  g.group_stages = (int)(group_k / 128); g.gscale_a = scale_a; g.gscale_b = scale_b;
+  g.groups = groups; g.group_stages = (int)(group_k / 128); g.gscale_a = scale_a; g.gscale_b = scale_b;
+  g.gsplits = gemm_grouped_splits_impl(M, N, groups, group_k);
+  g.gper = (groups + g.gsplits - 1) / g.gsplits;
+  g.gpart = nullptr; g.ldp = round_up(N, 4);
+  if (g.gsplits > 1) {
+    const size_t need = gemm_grouped_workspace_bytes_impl(M, N, groups, group_k);
+    if (!workspace || workspace_bytes < need) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+    if ((uintptr_t)workspace & 15) return fail(HOT_ERR_INVALID, "%s: workspace must be 16-byte aligned", who);
+    g.gpart = (float*)workspace;
+  }
+  g.tiles_m = (int)((M + 127) / 128);
+  g.tiles_n = (int)((N + 127) / 128);
+  g.group_m = pick_group_m(g.tiles_m, g.tiles_n, 1);
+  const int64_t total = (int64_t)g.tiles_m * g.tiles_n * g.gsplits;
+  if (total > (1 << 30)) return fail(HOT_ERR_UNSUPPORTED, "%s: too many tiles", who);
+  const int64_t quads = M * (g.ldp / 4);
+  const dim3 rgrid((unsigned)((quads + 255) / 256));
   switch (out_dtype) {
-    case HOT_F32: return launch_gemm_slot<2, 2, 2, 2, 8, 4, 128, float, true>(g, st);
-    case HOT_BF16: return launch_gemm_slot<2, 2, 2, 2, 8, 4, 128, bf16_t, true>(g, st);
-    case HOT_F16: return launch_gemm_slot<2, 2, 2, 2, 8, 4, 128, f16_t, true>(g, st);
+    case HOT_F32:
+      hipLaunchKernelGGL(gemm_i8_grouped_kernel<float>, dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
+      if (g.gsplits > 1) hipLaunchKernelGGL(gemm_i8_grouped_reduce_kernel<float>, rgrid, dim3(256), 0, st, g);
+      break;
+    case HOT_BF16:
+      hipLaunchKernelGGL(gemm_i8_grouped_kernel<bf16_t>, dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
+      if (g.gsplits > 1) hipLaunchKernelGGL(gemm_i8_grouped_reduce_kernel<bf16_t>, rgrid, dim3(256), 0, st, g);
+      break;
+    case HOT_F16:
+      hipLaunchKernelGGL(gemm_i8_grouped_kernel<f16_t>, dim3((unsigned)total), dim3(G_THREADS), 0, st, g);
+      if (g.gsplits > 1) hipLaunchKernelGGL(gemm_i8_grouped_reduce_kernel<f16_t>, rgrid, dim3(256), 0, st, g);
+      break;
     default: return fail(HOT_ERR_INVALID, "%s: bad out dtype %d", who, out_dtype);
   }
+  return check_launch("gemm_i8_grouped_kernel");
 }
 
 }  // namespace hot

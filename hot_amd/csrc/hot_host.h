@@ -75,9 +75,15 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
 // The hot_gemm_variant that gemm_i8_impl picks for a product when `ws_bytes` of workspace come with it.
 int gemm_plan_impl(int64_t M, int64_t N, int64_t K, int bits, int64_t lda, int64_t ldb, size_t ws_bytes);
 
+// K groups with steps of their own: out = (sum over groups g, in the order below, of
+// (float(A_g . B_g^T) * scale_a[g or g M + row]) * scale_b[g]) * post_scale.  The groups are cut into
+// gemm_grouped_splits_impl(...) ranges of ceil(groups / ranges) consecutive groups; a range is summed in
+// group order, the range sums are added in range order.  More than one range needs a workspace.
 int gemm_i8_grouped_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t M, int64_t N, int groups,
                          int64_t group_k, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
-                         void* out, int out_dtype, int64_t ldo, hipStream_t st);
+                         void* out, int out_dtype, int64_t ldo, void* workspace, size_t workspace_bytes, hipStream_t st);
+int gemm_grouped_splits_impl(int64_t M, int64_t N, int groups, int64_t group_k);
+size_t gemm_grouped_workspace_bytes_impl(int64_t M, int64_t N, int groups, int64_t group_k);
 
 // Split-K plan of gemm_i8_impl for a problem: `splits` K ranges (1 = none) and the bytes of workspace
 // that hold their partial accumulators (16-byte aligned; contents need no initialisation).

@@ -282,6 +282,12 @@ def kpad_group(T: int, opt: HotOptions) -> int:
     return int(_lib.lib().hot_kpad_group(int(T), C.byref(opt.to_c())))
 
 
+def backward_batched_ranges(B: int, T: int, O: int, I: int, opt: HotOptions) -> int:
+    """Ranges of consecutive samples in which linear_backward_batched adds up the weight gradient
+    (hot_backward_batched_ranges): each range in sample order, then the range sums in order."""
+    return int(_lib.lib().hot_backward_batched_ranges(int(B), int(T), int(O), int(I), C.byref(opt.to_c())))
+
+
 def abc_forward_batched(x: torch.Tensor, opt: HotOptions):
     """Activation buffer of a 3-D input [B, T, I] with one step per sample (hot_abc_forward_batched):
     (xq int8 [I, B * kpad_group(T)], sx fp32 [B])."""

@@ -227,7 +227,12 @@ HOT_API int hot_linear_backward_bias(const void* gy, const void* w, int dtype, c
  *                                in bytes [b kg, (b + 1) kg) of every row, zero behind its T' codes),
  *                                sx [B]; cfg->hla_n must divide T and be at most 128
  *   hot_linear_backward_batched  g_x [B T, I], g_W [O, I] = sum over samples, each sample's integer
- *                                sums dequantised with its own steps and added in fp32 in sample order
+ *                                sums dequantised with its own steps and added in fp32
+ *   hot_backward_batched_ranges  the order of that fp32 sum: the samples are cut into this many ranges
+ *                                of ceil(B / ranges) consecutive samples (a function of the shape
+ *                                alone); a range is summed in sample order, the range sums are added
+ *                                in range order.  (The reference leaves the order to torch's sum over
+ *                                the batch dimension.)  0 = bad arguments.
  * Per-tensor steps become per-sample steps, per-token steps stay per token, per-channel steps of the g_W
  * operand become per sample and channel.  Stochastic rounding numbers the elements as the flattened
  * calls do.  Everything runs on `hip_stream` in order.
@@ -239,6 +244,7 @@ HOT_API int hot_abc_forward_batched(const void* x, int dtype, int64_t B, int64_t
                             size_t workspace_bytes, void* hip_stream);
 HOT_API size_t hot_backward_batched_workspace_bytes(int64_t B, int64_t T, int64_t O, int64_t I,
                                             const hot_config* cfg);
+HOT_API int hot_backward_batched_ranges(int64_t B, int64_t T, int64_t O, int64_t I, const hot_config* cfg);
 HOT_API int hot_linear_backward_batched(const void* gy, const void* w, int dtype, const void* xq,
                                 const float* sx, int64_t B, int64_t T, int64_t O, int64_t I,
                                 const hot_config* cfg, void* gx, void* gw, int out_dtype,

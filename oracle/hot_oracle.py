@@ -503,12 +503,16 @@ def abc_forward_batched(x: np.ndarray, cfg: HotConfig):
     return np.stack(xq), np.asarray(sx, dtype=F32)
 
 
-def linear_backward_batched(g_y: np.ndarray, w: np.ndarray, xq: np.ndarray, sx: np.ndarray, cfg: HotConfig):
+def linear_backward_batched(g_y: np.ndarray, w: np.ndarray, xq: np.ndarray, sx: np.ndarray, cfg: HotConfig,
+                            gw_ranges: int = 1):
     """FLinearQ.backward on 3-D tensors (quant_matmul.py:215-348): the g_y quantisers run per sample
     (per-tensor steps become per-sample steps; per-row steps stay per token for g_y H and become per
     sample and channel for (P g_y)^T), W has one step, grad_input is computed per sample and the
-    per-sample weight gradients ((acc_b s_gw,b) s_x,b) are added up in fp32 in sample order
-    (autograd's sum over the batch dimension of the returned [B, O, I] tensor), then divided by n.
+    per-sample weight gradients ((acc_b s_gw,b) s_x,b) are added up in fp32 (autograd's sum over
+    the batch dimension of the returned [B, O, I] tensor, whose order torch leaves open), then
+    divided by n.  The order here: the samples form gw_ranges ranges of ceil(B / gw_ranges)
+    consecutive samples; each range is summed in sample order starting from zero, and the range
+    sums are added in range order (gw_ranges = 1: plain sample order).
     Returns (g_x [B, T, I], g_w [O, I], list of per-sample traces)."""
     g_y = np.asarray(g_y, dtype=F32)
     w = np.asarray(w, dtype=F32)
@@ -522,9 +526,14 @@ def linear_backward_batched(g_y: np.ndarray, w: np.ndarray, xq: np.ndarray, sx: 
                    index=colwise_rng_index(Wh.shape[1], Wh.shape[0] // cfg.n_o, np.arange(cfg.n_o)).T)
     gw_idx = colwise_rng_index(O, B * nbs, rows)                         # [O, B nbs r]
     g_x = np.empty((B, T, I), dtype=F32)
+    per_range = -(-B // max(1, int(gw_ranges)))
+    range_sums = []
     g_w = np.zeros((O, I), dtype=F32)
     traces = []
     for b in range(B):
+        if b % per_range == 0 and b > 0:
+            range_sums.append(g_w)
+            g_w = np.zeros((O, I), dtype=F32)
         tr = BackwardTrace()
         G = fwht_blocks_last(g_y[b], cfg.n_o)
         gx_idx = (np.arange(b * T, (b + 1) * T, dtype=np.int64)[:, None] * O + np.arange(O, dtype=np.int64)[None, :])
@@ -539,5 +548,9 @@ def linear_backward_batched(g_y: np.ndarray, w: np.ndarray, xq: np.ndarray, sx: 
         sgw = tr.sGp.reshape(-1, 1) if cfg.gw_scale == SCALE_ROW else tr.sGp.reshape(1, 1)
         g_w = (g_w + ((tr.acc_w.astype(F32) * sgw).astype(F32) * F32(sx[b])).astype(F32)).astype(F32)
         traces.append(tr)
+    range_sums.append(g_w)
+    g_w = range_sums[0]
+    for part in range_sums[1:]:
+        g_w = (g_w + part).astype(F32)
     g_w = (g_w / F32(cfg.hla_n)).astype(F32)
     return g_x, g_w, traces

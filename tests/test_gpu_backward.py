@@ -48,6 +48,22 @@ def both_configs(L, rule="python", **kw):
     return ocfg, opt
 
 
+def sum_in_ranges(parts, ranges):
+    """fp32 sum of per-sample gradients in the order of the batched entry point: `ranges` ranges of
+    ceil(B / ranges) consecutive samples, each from zero in sample order, then the range sums in order."""
+    per = -(-len(parts) // ranges)
+    sums = []
+    for lo in range(0, len(parts), per):
+        acc = np.zeros_like(parts[0])
+        for p in parts[lo:lo + per]:
+            acc = (acc + p).astype(np.float32)
+        sums.append(acc)
+    total = sums[0]
+    for s in sums[1:]:
+        total = (total + s).astype(np.float32)
+    return total
+
+
 def run_both(x, w, gy, ocfg, opt, gpu):
     from hot_amd import ops
     xq, sx = ops.abc_forward(x.to(gpu), opt)
@@ -314,15 +330,17 @@ def test_hq_linear_3d_input(gpu, fresh_args, mode):
     lin(x).backward(gy)
     wn = lin.weight.detach().cpu().numpy()
     if mode == "per_sample":
-        ocfg, _ = both_configs(L)
-        gxs, gw = [], 0
+        from hot_amd import ops
+        ocfg, opt = both_configs(L)
+        gxs, gws = [], []
         for b in range(B):
             xq_ref, sx_ref = orc.abc_forward(x[b].detach().cpu().numpy(), ocfg)
             tr = orc.linear_backward(gy[b].cpu().numpy(), wn, xq_ref, sx_ref, ocfg)
             gxs.append(tr.g_x)
-            gw = gw + tr.g_w
+            gws.append(tr.g_w)
         assert np.array_equal(x.grad.cpu().numpy(), np.stack(gxs))
-        assert np.array_equal(lin.weight.grad.cpu().numpy(), gw)      # fp32 sum over the samples, in sample order
+        # fp32 sum over the samples, in the order the library states
+        assert np.array_equal(lin.weight.grad.cpu().numpy(), sum_in_ranges(gws, ops.backward_batched_ranges(B, L, O, I, opt)))
     else:
         ocfg, _ = both_configs(B * L)
         xq_ref, sx_ref = orc.abc_forward(x.detach().reshape(B * L, I).cpu().numpy(), ocfg)
@@ -358,7 +376,9 @@ def test_backward_batched_matches_oracle(gpu, dtype, B, T, O, I, variant):
     xq, sx = ops.abc_forward_batched(x.to(gpu), opt)
     gx, gw = ops.linear_backward_batched(gy.to(gpu), w.to(gpu), xq, sx, opt)
     xq_ref, sx_ref = orc.abc_forward_batched(x.float().numpy(), ocfg)
-    gx_ref, gw_ref, _ = orc.linear_backward_batched(gy.float().numpy(), w.float().numpy(), xq_ref, sx_ref, ocfg)
+    ranges = ops.backward_batched_ranges(B, T, O, I, opt)
+    assert 1 <= ranges <= B
+    gx_ref, gw_ref, _ = orc.linear_backward_batched(gy.float().numpy(), w.float().numpy(), xq_ref, sx_ref, ocfg, gw_ranges=ranges)
     kg = ops.kpad_group(T, opt)
     tp = xq_ref.shape[1]
     got = xq.cpu().numpy().reshape(I, B, kg)

@@ -401,6 +401,24 @@ def test_batched_oracle_reduces_to_the_2d_path():
         assert np.array_equal(gw, acc)
         # the three samples differ by orders of magnitude: shared steps would crush the small ones
         assert len({float(s) for s in sx}) == B and traces[0].sG.max() < traces[2].sG.min()
+    # the order of the sum over samples: ranges of ceil(B / ranges) samples, then the range sums
+    B5 = 5
+    x5 = rng.standard_normal((B5, T, I)).astype(np.float32)
+    gy5 = (rng.standard_normal((B5, T, O)) * (10.0 ** rng.uniform(-3, 1, (B5, 1, 1)))).astype(np.float32)
+    cfg = orc.HotConfig(hla_n=n, hla_rows=tuple(int(v) for v in rows))
+    xq5, sx5 = orc.abc_forward_batched(x5, cfg)
+    per_sample = [orc.linear_backward(gy5[b], w, *orc.abc_forward(x5[b], cfg), cfg).g_w for b in range(B5)]
+    f32 = np.float32
+    seq = per_sample[0]
+    for p in per_sample[1:]:
+        seq = (seq + p).astype(f32)
+    two = (((per_sample[0] + per_sample[1]).astype(f32) + per_sample[2]).astype(f32)
+           + (per_sample[3] + per_sample[4]).astype(f32)).astype(f32)
+    assert np.array_equal(orc.linear_backward_batched(gy5, w, xq5, sx5, cfg)[1], seq)
+    assert np.array_equal(orc.linear_backward_batched(gy5, w, xq5, sx5, cfg, gw_ranges=2)[1], two)
+    assert not np.array_equal(seq, two)                 # the order is visible in the last bits
+    assert np.array_equal(orc.linear_backward_batched(gy5, w, xq5, sx5, cfg, gw_ranges=5)[1], seq)   # one sample per range
+
     cfg = orc.HotConfig(hla_n=n, hla_rows=tuple(int(v) for v in rows), gx_round=orc.ROUND_STOCH, gw_round=orc.ROUND_STOCH,
                         act_round=orc.ROUND_STOCH, seed=77)
     xq1, sx1 = orc.abc_forward_batched(x[:1], cfg)
