@@ -702,9 +702,14 @@ gemm_i8_slot_kernel(const GemmArgs g) {
   is_b = __builtin_amdgcn_readfirstlane(is_b);
   const uint32_t ring0 = lds_offset(ring);
   const int KT = g.ktiles * (G_BK * BITS / 8) / RB;               // stages of RB bytes per row
+  // (copies in registers: selecting between the two kernel arguments by a run-time bit would reload
+  // the pointer from the argument segment at every DMA instruction, and wait for it)
+  const uint8_t* a_base = g.A;
+  const uint8_t* b_base = g.B;
+  asm volatile("" : "+s"(a_base), "+s"(b_base));
   auto dma_one = [&](int stage_off, int kt, int i) {
     // (wave-uniform by construction; said explicitly, since the instruction takes it in scalar registers)
-    const uint64_t b64 = (uint64_t)(uintptr_t)(((is_b >> i) & 1u ? g.B : g.A) + (int64_t)kt * RB);
+    const uint64_t b64 = (uint64_t)(uintptr_t)(((is_b >> i) & 1u ? b_base : a_base) + (int64_t)kt * RB);
     // (the builtin returns a signed int: both halves go through uint32_t, or a low half with its top
     // bit set would sign-extend over the high half)
     const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b64 >> 32));
