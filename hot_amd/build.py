@@ -17,7 +17,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libhot_gfx950.so")
-SOURCES = ["hq_rowwise.hip", "colwise.hip", "hla_big.hip", "gemm_i8.hip", "backward.hip", "ceilings.hip"]
+SOURCES = ["hq_rowwise.hip", "colwise.hip", "hla_big.hip", "gemm_i8.hip", "backward.hip", "ceilings.hip", "hla_expand.hip"]
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -452,6 +452,83 @@ int hot_linear_backward_bias(const void* gy, const void* w, int dtype, const voi
                       nullptr, (hipStream_t)hip_stream, gb);
 }
 
+// ---- g_x through a low-rank projection along the tokens ---------------------------------------------
+// transform_scheme "low_rank" and "gilr_gwh" (utils/quant_matmul.py:229-233, 263-266, 288-290, 334-337):
+// g_x = P^T ( q(P g_y) . q(W) ) s_g s_w / n, W untransformed.  The token-wise kernels store q(P g_y)
+// untransposed ([L', O], K along the channels), W goes through the column-wise kernel with blocks of
+// one row (quantise + transpose), the product lands in fp32 in the workspace and the expansion pass
+// takes it back to L tokens.  Kept for completeness of the reference's scheme list: four kernels on
+// one stream, not tuned.  The g_W side of those schemes is the g_W side of "gih_gwlr" / "hadamard".
+
+struct LowrankLayout {
+  int64_t lp, ld_g, ld_w;
+  size_t off_colg, off_colw, off_sg, off_sw, off_qg, off_qw, off_t, total;
+};
+
+static LowrankLayout lowrank_layout(int64_t L, int64_t O, int64_t I, const hot_config* c) {
+  LowrankLayout b;
+  b.lp = (L / c->hla_n) * c->hla_r;
+  b.ld_g = round_up(O, GEMM_KTILE) * c->gx_bits / 8;
+  b.ld_w = round_up(O, GEMM_KTILE) * c->w_bits / 8;
+  size_t o = 0;
+  b.off_colg = o; o += align256(colwise_workspace_bytes_impl(O));
+  b.off_colw = o; o += align256(colwise_workspace_bytes_impl(I));
+  b.off_sg = o;   o += 256;
+  b.off_sw = o;   o += 256;
+  b.off_qg = o;   o += align256((size_t)b.lp * b.ld_g);
+  b.off_qw = o;   o += align256((size_t)I * b.ld_w);
+  b.off_t = o;    o += align256((size_t)b.lp * (size_t)I * 4);
+  b.total = o;
+  return b;
+}
+
+static int check_lowrank(const hot_config* cfg, int64_t L, int64_t O, int64_t I, const char* who) {
+  if (int e = check_cfg(cfg, who)) return e;
+  if (L <= 0 || O <= 0 || I <= 0 || O % 8 || I % 8) return fail(HOT_ERR_INVALID, "%s: L=%lld, O=%lld and I=%lld must be positive, O and I multiples of 8", who, (long long)L, (long long)O, (long long)I);
+  if (cfg->hla_n > 64) return fail(HOT_ERR_UNSUPPORTED, "%s: token blocks up to 64 (the expansion pass holds a block per thread)", who);
+  if (L % cfg->hla_n) return fail(HOT_ERR_INVALID, "%s: L=%lld is not a multiple of hla_n=%d", who, (long long)L, cfg->hla_n);
+  if (cfg->gx_bits != cfg->w_bits) return fail(HOT_ERR_UNSUPPORTED, "%s: gx_bits (%d) and w_bits (%d) must match", who, cfg->gx_bits, cfg->w_bits);
+  if (cfg->gx_scale != HOT_SCALE_TENSOR) return fail(HOT_ERR_UNSUPPORTED, "%s: the projected g_y takes one step for the tensor (a step per coefficient row or per channel has no place in the product's epilogue)", who);
+  if (cfg->w_scale == HOT_SCALE_ROW) return fail(HOT_ERR_UNSUPPORTED, "%s: W uses one step per tensor", who);
+  return HOT_OK;
+}
+
+size_t hot_gx_lowrank_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_config* cfg) {
+  if (check_lowrank(cfg, L, O, I, "hot_gx_lowrank_workspace_bytes")) return 0;
+  return lowrank_layout(L, O, I, cfg).total;
+}
+
+int hot_gx_lowrank(const void* gy, const void* w, int dtype, int64_t L, int64_t O, int64_t I, const hot_config* cfg,
+                   void* gx, int out_dtype, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  const char* who = "hot_gx_lowrank";
+  if (int e = check_lowrank(cfg, L, O, I, who)) return e;
+  if (!gy || !w || !gx) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
+  if (L * O * 4 >= (1ll << 32) || O * I * 4 >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "%s: tensors exceed the 32-bit offsets of the loader", who);
+  const LowrankLayout b = lowrank_layout(L, O, I, cfg);
+  if (!workspace || workspace_bytes < b.total) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, b.total, workspace_bytes);
+  if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
+  hipStream_t st = (hipStream_t)hip_stream;
+  uint8_t* ws = (uint8_t*)workspace;
+  float* sg = (float*)(ws + b.off_sg);
+  float* sw = (float*)(ws + b.off_sw);
+  const int bits = cfg->gx_bits;
+  // q(P g_y), untransposed [L', O]; the K padding of every row is cleared apart
+  int rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, bits, cfg->gx_round, cfg->seed,
+                              HOT_STREAM_GX, HOT_SCALE_TENSOR, ws + b.off_qg, b.ld_g, bits == 4, sg, ws + b.off_colg,
+                              colwise_workspace_bytes_impl(O), st, who, nullptr, false, nullptr, nullptr, 1, 0, true);
+  if (rc) return rc;
+  zero_pad_impl(ws + b.off_qg, b.lp, O * bits / 8, b.ld_g, st);
+  // q(W), stored [I, O]: blocks of one row, nothing transformed
+  rc = colwise_quant_impl(w, dtype, O, I, 1, identity_rows(), 1, cfg->w_bits, cfg->w_round, cfg->seed, HOT_STREAM_W,
+                          cfg->w_scale, ws + b.off_qw, b.ld_w, cfg->w_bits == 4, sw, ws + b.off_colw,
+                          colwise_workspace_bytes_impl(I), st, who);
+  if (rc) return rc;
+  float* t = (float*)(ws + b.off_t);
+  rc = gemm_i8_impl(ws + b.off_qg, b.ld_g, ws + b.off_qw, b.ld_w, bits, b.lp, I, O, sg, 0, sw, 1.0f, t, HOT_F32, I, nullptr, st);
+  if (rc) return rc;
+  return hla_expand_impl(t, L / cfg->hla_n, I, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, 1.0f / (float)cfg->hla_n, gx, out_dtype, st);
+}
+
 // ---- 3-D activations: one set of steps per sample --------------------------------------------------
 // The reference vmaps its quantisers over the batch dimension of [B, T, C] tensors
 // (utils/quant_matmul.py:33-37,102-106,118-122), applies the token-wise transform inside each sample

@@ -61,6 +61,9 @@ struct ColArgs {
   int32_t groups, runs;
   int64_t NBs, Kpad;
   float* gstat;
+  // rowmajor: the codes are stored untransposed, [NB r, C] with ld_out bytes per coefficient row
+  // (the A operand of a product whose K runs along the channels), instead of [C, NB r]
+  int32_t rowmajor;
   hipEvent_t after_stats;  // host only: recorded between the statistics and the quantise pass
   int8_t slot[COL_MAX_N];  // output position of natural row i, -1 = dropped
 };
@@ -479,6 +482,23 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     }
   } else {
     __syncthreads();
+    if (a.rowmajor) {
+      // untransposed store: coefficient row (blk0 + b) r + k takes one code of every channel; a
+      // wave writes 64 adjacent bytes (INT8) or, two channels to a byte, 32 (packed INT4: the even
+      // channel in bits 3:0)
+      const int krun = nblk * a.r;
+      int8_t* orow = a.out + blk0 * a.r * a.ld_out;
+      for (int k = 0; k < krun; ++k, orow += a.ld_out) {
+        const int code = stage[tid * pitch + k];
+        if (a.store4) {
+          const int hi = __shfl_xor(code, 1, 64);
+          if (active && !(tid & 1)) orow[c >> 1] = (int8_t)((code & 0xF) | ((hi & 0xF) << 4));
+        } else if (active) {
+          orow[c] = (int8_t)code;
+        }
+      }
+      return;
+    }
     // flush: each channel's staged run is one contiguous global segment
     const bool last = blk_in + a.tb >= a.NBs;       // the run that ends its sample also zeroes the sample's tail
     const int out_sb = a.store4 ? sb / 2 : sb;
@@ -829,8 +849,11 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
                        int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
                        void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,
                        size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out,
-                       bool stats_cleared, hipEvent_t after_stats, float* colsum_partial, int groups, int64_t kpad_group) {
+                       bool stats_cleared, hipEvent_t after_stats, float* colsum_partial, int groups, int64_t kpad_group,
+                       bool rowmajor) {
   if (!in || !codes_out || !scales_out || !rows) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
+  if (rowmajor && (groups > 1 || n > COL_MAX_N || scale_mode == HOT_SCALE_ROW || row16_absmax_out || colsum_partial))
+    return fail(HOT_ERR_UNSUPPORTED, "%s: the untransposed store takes token blocks up to %d, one step for the tensor, and no fused statistics", who, COL_MAX_N);
   if (R <= 0 || C <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape R=%lld C=%lld", who, (long long)R, (long long)C);
   if (groups < 1) return fail(HOT_ERR_INVALID, "%s: %d sample groups", who, groups);
   if (groups > 1) {
@@ -881,8 +904,10 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
     if (a.slot[rows[k]] != -1) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d listed twice", who, k, rows[k]);
     a.slot[rows[k]] = (int8_t)k;
   }
-  const int64_t row_bytes = groups > 1 ? kpad_group * groups : (store4 ? a.Kout / 2 : a.Kout);
-  if (store4 && (r & 1)) return fail(HOT_ERR_UNSUPPORTED, "%s: packed INT4 output needs an even r", who);
+  const int64_t row_bytes = rowmajor ? (store4 ? C / 2 : C) : groups > 1 ? kpad_group * groups : (store4 ? a.Kout / 2 : a.Kout);
+  // packed INT4 pairs codes along K: a channel's codes must come in whole bytes (pairs along the channels
+  // when the store is untransposed: C is a multiple of 8)
+  if (store4 && !rowmajor && (a.Kout & 1)) return fail(HOT_ERR_UNSUPPORTED, "%s: packed INT4 output needs an even number of codes per channel", who);
   if (ld_out < row_bytes || (ld_out & 15)) return fail(HOT_ERR_INVALID, "%s: ld_out=%lld must be a multiple of 16 and >= %lld", who, (long long)ld_out, (long long)row_bytes);
   if (!workspace || workspace_bytes < colwise_group_workspace_bytes_impl(C, groups)) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed", who, colwise_group_workspace_bytes_impl(C, groups));
   if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
@@ -895,6 +920,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   a.colmax = (float*)(ws + COL_STAT_BYTES);
   a.partial = (double*)(ws + COL_STAT_BYTES + round_up(C * 4 * COLMAX_COPIES, 256));
   a.gstat = nullptr;
+  a.rowmajor = rowmajor ? 1 : 0;
   a.groups = groups; a.runs = 1; a.NBs = a.NB / groups; a.Kpad = groups > 1 ? kpad_group : ld_out;
   if (groups > 1) {
     a.gstat = (float*)(ws + COL_STAT_BYTES + group_colmax_bytes(C, groups));

@@ -1,0 +1,88 @@
+// Expansion pass of the schemes that project g_y to low rank along the tokens for the g_x product
+// (utils/quant_matmul.py:334-337, transform_scheme "low_rank" / "gilr_gwh":
+// grad_input = lowering_matmul_back(h.mT, grad_input) / n): the [L', I] product goes back to [L, I]
+// through P^T, block by block.  H_n is symmetric, so P^T c = H_n z with z = the r coefficients at
+// their natural rows and zeros elsewhere: the same canonical butterflies as every other transform
+// here (adding an exact zero changes no bit), then one exact scaling by 1 / n.
+//
+// A thread owns one channel; its column of the block lives in LDS ([n][256] floats, the thread's
+// own bank column, so no thread ever touches another's values and no barrier is needed).  Kept for
+// completeness of the reference's scheme list, not tuned: memory-bound work done at LDS speed.
+#include <hip/hip_runtime.h>
+
+#include <mutex>
+
+#include "hot_device.h"
+#include "hot_host.h"
+
+namespace hot {
+
+constexpr int EXP_MAX_N = 64;
+constexpr int EXP_THREADS = 256;
+
+struct ExpandArgs {
+  const float* t;      // [nb r, C]
+  void* out;           // [nb n, C]
+  int64_t nb, C;
+  int32_t n, r;
+  float post;
+  int8_t row[EXP_MAX_N];   // natural row of the k-th coefficient
+};
+
+template <typename OutT>
+__global__ void __launch_bounds__(EXP_THREADS) hla_expand_kernel(const ExpandArgs a) {
+  extern __shared__ float col[];                      // [n][EXP_THREADS]
+  const int tid = threadIdx.x;
+  const int64_t c = (int64_t)blockIdx.x * EXP_THREADS + tid;
+  const int64_t blk = blockIdx.y;
+  if (c >= a.C) return;                               // no barriers below: a thread may leave alone
+  for (int i = 0; i < a.n; ++i) col[i * EXP_THREADS + tid] = 0.f;
+  const float* src = a.t + blk * a.r * a.C + c;
+  for (int k = 0; k < a.r; ++k) col[a.row[k] * EXP_THREADS + tid] = src[(int64_t)k * a.C];
+  for (int h = 1; h < a.n; h <<= 1)
+    for (int i = 0; i < a.n; ++i)
+      if ((i & h) == 0) {
+        const float x = col[i * EXP_THREADS + tid], y = col[(i + h) * EXP_THREADS + tid];
+        col[i * EXP_THREADS + tid] = x + y;
+        col[(i + h) * EXP_THREADS + tid] = x - y;
+      }
+  OutT* dst = reinterpret_cast<OutT*>(a.out) + blk * a.n * a.C + c;
+  for (int i = 0; i < a.n; ++i) store_scalar<OutT>(dst + (int64_t)i * a.C, col[i * EXP_THREADS + tid] * a.post);
+}
+
+int hla_expand_impl(const float* t, int64_t nb, int64_t C, int n, const int32_t* rows, int r, float post,
+                    void* out, int out_dtype, hipStream_t st) {
+  const char* who = "hla_expand";
+  if (!t || !out || !rows) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
+  if (nb <= 0 || C <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape %lld blocks x %lld channels", who, (long long)nb, (long long)C);
+  if (n < 1 || n > EXP_MAX_N || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block %d (a power of two up to %d)", who, n, EXP_MAX_N);
+  if (r < 1 || r > n) return fail(HOT_ERR_INVALID, "%s: r=%d outside [1, %d]", who, r, n);
+  if (nb > 65535) return fail(HOT_ERR_UNSUPPORTED, "%s: more than 65535 token blocks", who);
+  ExpandArgs a;
+  a.t = t; a.out = out; a.nb = nb; a.C = C; a.n = n; a.r = r; a.post = post;
+  bool seen[EXP_MAX_N] = {};
+  for (int k = 0; k < r; ++k) {
+    if (rows[k] < 0 || rows[k] >= n || seen[rows[k]]) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d out of range or listed twice", who, k, rows[k]);
+    seen[rows[k]] = true;
+    a.row[k] = (int8_t)rows[k];
+  }
+  const dim3 grid((unsigned)((C + EXP_THREADS - 1) / EXP_THREADS), (unsigned)nb);
+  const size_t lds = (size_t)n * EXP_THREADS * sizeof(float);          // 64 KiB at n = 64
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&hla_expand_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    if (attr_err == hipSuccess) attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&hla_expand_kernel<bf16_t>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    if (attr_err == hipSuccess) attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&hla_expand_kernel<f16_t>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+  });
+  if (attr_err != hipSuccess) return check_hip(attr_err, "hipFuncSetAttribute(hla_expand_kernel)");
+  switch (out_dtype) {
+    case HOT_F32: hipLaunchKernelGGL(hla_expand_kernel<float>, grid, dim3(EXP_THREADS), lds, st, a); break;
+    case HOT_BF16: hipLaunchKernelGGL(hla_expand_kernel<bf16_t>, grid, dim3(EXP_THREADS), lds, st, a); break;
+    case HOT_F16: hipLaunchKernelGGL(hla_expand_kernel<f16_t>, grid, dim3(EXP_THREADS), lds, st, a); break;
+    default: return fail(HOT_ERR_INVALID, "%s: bad out dtype %d", who, out_dtype);
+  }
+  return check_launch("hla_expand_kernel");
+}
+
+}  // namespace hot

@@ -43,7 +43,14 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
                        void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,
                        size_t workspace_bytes, hipStream_t st, const char* who, float* row16_absmax_out = nullptr,
                        bool stats_cleared = false, hipEvent_t after_stats = nullptr, float* colsum_partial = nullptr,
-                       int groups = 1, int64_t kpad_group = 0);
+                       int groups = 1, int64_t kpad_group = 0, bool rowmajor = false);
+// rowmajor: codes stored untransposed, [NB r, C] with ld_out bytes per coefficient row (bytes past the C
+// channels of a row are left alone: zero_pad_impl clears them), one step for the tensor.
+void zero_pad_impl(void* codes, int64_t rows, int64_t row_bytes, int64_t ld, hipStream_t st);
+// out[NB n, C] = (P^T t) * post for t [NB r, C] fp32: the kept coefficients go back to their natural rows of
+// every block and the block is transformed again (H is symmetric); n up to 64.
+int hla_expand_impl(const float* t, int64_t nb, int64_t C, int n, const int32_t* rows, int r, float post,
+                    void* out, int out_dtype, hipStream_t st);
 // With groups > 1 the R rows are `groups` samples of equal length, each quantised with steps of its own
 // (scales_out: [groups], or [groups][C] with per-channel steps); the codes of sample g take the bytes
 // [g * kpad_group, (g + 1) * kpad_group) of every output row, zero-filled behind the sample's codes.

@@ -278,6 +278,12 @@ __global__ void fill_u32_kernel(uint32_t* p, uint32_t v, int n) {
   if (i < n) p[i] = v;
 }
 
+void zero_pad_impl(void* codes, int64_t rows, int64_t row_bytes, int64_t ld, hipStream_t st) {
+  if (ld <= row_bytes || rows <= 0) return;
+  const int64_t n = rows * ((ld - row_bytes) / 4);
+  hipLaunchKernelGGL(zero_pad_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (int8_t*)codes, rows, row_bytes, ld);
+}
+
 // ---- host dispatch -----------------------------------------------------------
 
 template <typename T, int N, int BITS, int ROUND>

@@ -18,6 +18,8 @@ from __future__ import annotations
 
 from typing import Optional, Tuple
 
+from dataclasses import replace
+
 import numpy as np
 import torch
 import torch.nn as nn
@@ -54,7 +56,9 @@ def token_rule(tokens: int):
     """(n, rows) of the token-wise transform for a token count: the low-rank projection under
     args.hla_rule, or, with the reference's scheme "hadamard", the whole block Hadamard of make_hadamard
     along the tokens (utils/quant_matmul.py:182-183,294-295,353-355: every coefficient, natural order)."""
-    if args.transform_scheme == "hadamard":
+    if args.transform_scheme in ("hadamard", "gilr_gwh"):
+        # "gilr_gwh": the g_W product and the activation buffer use the whole block Hadamard
+        # (utils/quant_matmul.py:186-187,298-299); its g_x product the projection of gx_token_rule
         n = int(biggest_power2_factor_max16(int(tokens)))
         return n, np.arange(n)
     if args.hla_rule == "paper":
@@ -64,6 +68,24 @@ def token_rule(tokens: int):
     n, rows = hla_rows(tokens, args.vectorPercentile)
     if n > args.hla_max_block:
         n, rows = hla_rows(args.hla_max_block, args.vectorPercentile)
+    return n, rows
+
+
+LOWRANK_GX_SCHEMES = ("low_rank", "gilr_gwh")
+LOWRANK_GX_MAX_BLOCK = 64
+
+
+def gx_token_rule(tokens: int):
+    """(n, rows) of the projection P along the tokens that the schemes "low_rank" and "gilr_gwh" apply to
+    g_y for the g_x product (utils/quant_matmul.py:229-233; P is make_WHT of the token count, :356-362):
+    the low-rank rule of args.hla_rule with blocks of at most 64 tokens (the expansion pass holds a block
+    per thread)."""
+    if args.hla_rule == "paper":
+        return (1, np.array([0])) if tokens % 16 else paper_rows(16, 8)
+    n, rows = hla_rows(tokens, args.vectorPercentile)
+    cap = min(int(args.hla_max_block), LOWRANK_GX_MAX_BLOCK)
+    if n > cap:
+        n, rows = hla_rows(cap, args.vectorPercentile)
     return n, rows
 
 
@@ -101,10 +123,13 @@ def options_for(tokens: int, layer_name: str = " ", out_features: int = 16) -> o
 
 
 def _options_uncached(tokens: int, layer_name: str, out_features: int) -> ops.HotOptions:
-    # "hadamard" differs from "gih_gwlr" in the token-wise transform only (token_rule); the low-rank
-    # schemes on the g_x side (low_rank, gilr_gwh, gilro_gwh) need an expansion pass that is not built
-    if args.transform_scheme not in ("gih_gwlr", "hadamard"):
-        raise NotImplementedError("transform scheme %r: gih_gwlr and hadamard run natively" % args.transform_scheme)
+    # "hadamard" differs from "gih_gwlr" in the token-wise transform only (token_rule); "low_rank" and
+    # "gilr_gwh" project g_y along the tokens for the g_x product as well (gx_token_rule, ops.gx_lowrank);
+    # "gilro_gwh" projects along the out-features and has no activation branch in the reference's
+    # setup_context (utils/quant_matmul.py:181-192 raises for it): not built
+    if args.transform_scheme not in ("gih_gwlr", "hadamard") + LOWRANK_GX_SCHEMES:
+        raise NotImplementedError("transform scheme %r: gih_gwlr, hadamard, low_rank and gilr_gwh run natively"
+                                  % args.transform_scheme)
     if not (args.TransformGogi and args.TransformWgt and args.TransformGogw and args.TransformInput):
         raise NotImplementedError("the native path needs all four Transform* flags on")
     n, rows = token_rule(tokens)
@@ -214,7 +239,27 @@ class FLinearQ(Function):
         wc = _pad8(_pad8(w).t()).t().contiguous() if (O % 8 or I % 8) else w.contiguous()   # [O8, I8]
         if go.dtype != wc.dtype:
             go = go.to(wc.dtype)
-        if go.dim() == 3 and args.batched_mode == "per_sample" and ctx.batched:
+        if args.transform_scheme in LOWRANK_GX_SCHEMES:
+            # g_x through the projection along the tokens and its expansion; g_W as in "gih_gwlr"
+            # ("low_rank") or "hadamard" ("gilr_gwh"): the token-wise kernel on g_y, then the INT8 product
+            if go.dim() == 3 and args.batched_mode == "per_sample":
+                raise NotImplementedError("transform scheme %r takes 2-D activations or batched_mode \"flatten\""
+                                          % args.transform_scheme)
+            if opt.gx_scale != ops.SCALE_TENSOR:
+                raise NotImplementedError("transform scheme %r: the projected g_y takes one step for the tensor "
+                                          "(quantBWDGogi int or stoch)" % args.transform_scheme)
+            go2 = _pad8(go.reshape(-1, go.shape[-1]))
+            n_gx, rows_gx = gx_token_rule(go2.shape[0])
+            gx = ops.gx_lowrank(go2, wc, replace(opt, hla_n=int(n_gx), hla_rows=tuple(int(v) for v in rows_gx)))
+            qgp, sgp, lp = ops.hla_tokenwise(go2, opt.hla_n, opt.hla_rows, bits=opt.gw_bits,
+                                             rounding="stoch" if opt.gw_round == ops.ROUND_STOCH else "nearest",
+                                             scale="row" if opt.gw_scale == ops.SCALE_ROW else "tensor",
+                                             seed=opt.seed, rng_stream=ops.STREAM_GW)
+            if opt.gw_bits != opt.act_bits:
+                raise NotImplementedError("GogwQuantBit and actQuantBit must match")
+            grad_w = ops.gemm_i8(qgp, xq, lp, opt.gw_bits, sgp, sx, post_scale=1.0 / opt.hla_n, out_dtype=wc.dtype)
+            grad_input = gx[:, :I].reshape(ctx.x_shape)
+        elif go.dim() == 3 and args.batched_mode == "per_sample" and ctx.batched:
             gx, grad_w = ops.linear_backward_batched(_pad8(go), wc, xq, sx, opt)
             grad_input = gx[..., :I]
         elif go.dim() == 3 and args.batched_mode == "per_sample":

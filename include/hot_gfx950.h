@@ -251,6 +251,22 @@ HOT_API int hot_linear_backward_batched(const void* gy, const void* w, int dtype
                                 void* workspace, size_t workspace_bytes, void* hip_stream);
 
 /*
+ * g_x of the schemes that project g_y to low rank along the TOKENS for that product
+ * (utils/quant_matmul.py, transform_scheme "low_rank" and "gilr_gwh": :229-233 g_y <- P g_y,
+ * :263-266 W untransformed, :288-290 the product and its two steps, :334-337 P^T (.) / n):
+ *   g_x [L, I] = P^T ( q(P g_y) [L', O] . q(W) [O, I] ) s_g s_w / hla_n.
+ * cfg->hla_n / hla_rows describe P (blocks up to 64 tokens), gx_bits / gx_round the quantiser of
+ * P g_y (one step for the tensor), w_bits (= gx_bits) / w_round / w_scale that of W.  The g_W side
+ * of those schemes is the g_W side of hot_linear_backward with the matching token-wise selection
+ * (hot_hla_tokenwise + hot_gemm_i8).  Four kernels on `hip_stream`, kept for completeness of the
+ * reference's scheme list.
+ */
+HOT_API size_t hot_gx_lowrank_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_config* cfg);
+HOT_API int hot_gx_lowrank(const void* gy, const void* w, int dtype, int64_t L, int64_t O, int64_t I,
+                   const hot_config* cfg, void* gx, int out_dtype, void* workspace,
+                   size_t workspace_bytes, void* hip_stream);
+
+/*
  * Number of K ranges into which the GEMMs inside hot_linear_backward cut a product of
  * M x N outputs over K codes of `bits` bits (1 = one kernel; more = a kernel per range
  * writing int32 partial tiles to the workspace, then a reduce kernel).  Products with

@@ -88,24 +88,44 @@ def setup_context(x: torch.Tensor, h_bs: torch.Tensor, cfg: PortConfig):
 
 def backward(grad_output: torch.Tensor, w: torch.Tensor, xq: torch.Tensor, scale_x, h_out: torch.Tensor,
              h_bs: torch.Tensor, cfg: PortConfig, scheme: str = "gih_gwlr"):
-    """quant_matmul.py:215-348, branch gih_gwlr, 2-D tensors; with scheme "hadamard" (h_bs = the block
-    Hadamard of make_hadamard for the token count) the g_W branch of that scheme (:294-295, :338-339)."""
-    g = _front(grad_output, h_out)                              # :238
+    """quant_matmul.py:215-348, 2-D tensors, the branches of transform_scheme:
+    "gih_gwlr" (h_out = block Hadamard of the out-features, h_bs = low-rank WHT rows of the tokens);
+    "hadamard" (h_bs = the block Hadamard of make_hadamard for the token count: g_W branch :294-295, :338-339);
+    "low_rank" (h_bs = low-rank WHT rows of the tokens for both products, W untransformed: :231-232, :263-264,
+    :296-297, :334-335); "gilr_gwh" (h_out = low-rank WHT rows of the TOKENS for the g_x product, h_bs = block
+    Hadamard of the tokens for the g_W product: :233-234, :265-266, :298-299, :336-338)."""
+    if scheme in ("gih_gwlr", "hadamard"):
+        g = _front(grad_output, h_out)                          # :230 / :238
+        wh = _back(h_out, w)                                    # :262 / :270
+    elif scheme == "low_rank":
+        g = _back(h_bs, grad_output)                            # :232
+        wh = w                                                  # :264
+    elif scheme == "gilr_gwh":
+        g = _back(h_out, grad_output)                           # :234
+        wh = w                                                  # :266
+    else:
+        raise NotImplementedError(scheme)
     g, s_g = _quant(g, cfg.gx_bits, cfg.gx_kind)                # :244-257
-    wh = _back(h_out, w)                                        # :270
     wh, s_w = _quant(wh, cfg.w_bits, cfg.w_kind)                # :276-285
     grad_input = (g @ wh) * s_g * s_w                           # :288-290
-    if scheme == "hadamard":
-        gp = _front(grad_output.T.contiguous(), h_bs)           # :295
+    if scheme in ("hadamard", "gilr_gwh"):
+        gp = _front(grad_output.T.contiguous(), h_bs)           # :295 / :299
     else:
-        gp = _back(h_bs, grad_output).T                         # :301
+        gp = _back(h_bs, grad_output).T                         # :297 / :301
     gp, s_gp = _quant(gp, cfg.gw_bits, cfg.gw_kind)             # :307-320
     grad_w = (gp @ xq.to(gp.dtype)) * s_gp * scale_x            # :322-324
-    grad_input = grad_input / orc.pow2_factor_max16(h_out.shape[0])   # :343
     if scheme == "hadamard":
-        grad_w = grad_w / orc.pow2_factor_max16(h_bs.shape[0])        # :339
+        grad_input = grad_input / orc.pow2_factor_max16(h_out.shape[0])      # :331
+        grad_w = grad_w / orc.pow2_factor_max16(h_bs.shape[0])               # :332
+    elif scheme == "low_rank":
+        grad_input = _back(h_bs.T.contiguous(), grad_input) / orc.pow2_factor(h_bs.shape[1])     # :334
+        grad_w = grad_w / orc.pow2_factor(h_bs.shape[1])                     # :335
+    elif scheme == "gilr_gwh":
+        grad_input = _back(h_out.T.contiguous(), grad_input) / orc.pow2_factor(h_out.shape[1])   # :337
+        grad_w = grad_w / orc.pow2_factor_max16(h_bs.shape[0])               # :338
     else:
-        grad_w = grad_w / orc.pow2_factor(h_bs.shape[1])              # :344
+        grad_input = grad_input / orc.pow2_factor_max16(h_out.shape[0])      # :343
+        grad_w = grad_w / orc.pow2_factor(h_bs.shape[1])                     # :344
     return grad_input, grad_w
 
 

@@ -463,6 +463,43 @@ def linear_backward(g_y: np.ndarray, w: np.ndarray, xq: np.ndarray, sx: np.ndarr
     return tr
 
 
+def hla_expand(t: np.ndarray, n: int, rows) -> np.ndarray:
+    """P^T t for the block-diagonal P of kept Walsh-Hadamard rows (lowering_matmul_back(h.mT, t),
+    utils/hadamard_matmul.py:143-161 with utils/quant_matmul.py:334-337): t [NB r, C] -> [NB n, C].
+    H is symmetric, so P^T c = H_n z with z the coefficients c put back at their natural rows and
+    zeros elsewhere; evaluated with the canonical butterflies (adding an exact zero changes nothing)."""
+    t = np.asarray(t, dtype=F32)
+    rows = np.asarray(rows)
+    r = len(rows)
+    nb = t.shape[0] // r
+    z = np.zeros((nb, n, t.shape[1]), dtype=F32)
+    z[:, rows, :] = t.reshape(nb, r, t.shape[1])
+    return fwht_blocks_first(z.reshape(nb * n, t.shape[1]), n)
+
+
+def gx_lowrank(g_y: np.ndarray, w: np.ndarray, cfg: HotConfig) -> BackwardTrace:
+    """grad_input of the schemes that project g_y to low rank along the TOKENS for the g_x product
+    (utils/quant_matmul.py, transform_scheme "low_rank" and "gilr_gwh"): :229-233 g_y <- P g_y [L', O];
+    :244-257 quantise (one step for the tensor); :263-266 W is NOT transformed; :276-285 quantise W;
+    :288-290 (q(P g_y) q(W)) s_g s_w [L', I]; :334-337 P^T (.) / n.  cfg.hla_n / cfg.hla_rows describe P,
+    cfg.gx_* the quantiser of P g_y, cfg.w_* that of W.  Element numbering of stochastic rounding: the
+    column-wise one, P g_y as [O channels][NB blocks][r], W as blocks of one row."""
+    g_y = np.asarray(g_y, dtype=F32)
+    w = np.asarray(w, dtype=F32)
+    L, O = g_y.shape
+    rows = np.asarray(cfg.hla_rows)
+    tr = BackwardTrace()
+    Gp = fwht_blocks_first(g_y, cfg.hla_n, rows)                                        # [L', O]
+    tr.qG, tr.sG = quant(Gp, cfg.gx_bits, SCALE_TENSOR, cfg.gx_round, cfg.seed, STREAM_GX,
+                         index=colwise_rng_index(O, L // cfg.hla_n, rows).T)
+    tr.qW, tr.sW = quant(w, cfg.w_bits, cfg.w_scale, cfg.w_round, cfg.seed, STREAM_W,
+                         index=colwise_rng_index(w.shape[1], w.shape[0], np.arange(1)).T)
+    tr.acc_x = int_gemm_nt(tr.qG, tr.qW.T)                                              # [L', I]
+    t = ((tr.acc_x.astype(F32) * tr.sG[0]).astype(F32) * tr.sW[0]).astype(F32)
+    tr.g_x = (hla_expand(t, cfg.hla_n, rows) / F32(cfg.hla_n)).astype(F32)
+    return tr
+
+
 def stoch_round_mantissa(x: np.ndarray) -> np.ndarray:
     """The reference CUDA op's pseudo-stochastic rounding
     (HLQ_backward_kernel.cu:19-36), kept only to characterise its bias; the

@@ -771,6 +771,75 @@ def test_hq_linear_scheme_hadamard(gpu, fresh_args, L):
     assert rel(lin.weight.grad.cpu().numpy(), gw_ref.numpy()) < REL_TOL
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L,O,I,rule,variant", [
+    (448, 192, 160, "python", dict()),                                            # n = 64, r = 36, INT4
+    (64 * 5, 208, 72, "python", dict(gx_bits=8, w_bits=8)),
+    (1344, 96, 264, "python", dict(gx_round=orc.ROUND_STOCH, w_round=orc.ROUND_STOCH, seed=11)),
+    (512, 256, 128, "paper", dict(w_scale=orc.SCALE_SAWB)),                       # n = 16, r = 8
+    (200, 40, 24, "python", dict(gx_round=orc.ROUND_STOCH, seed=4)),              # n = 8, one ragged strip
+    (49, 64, 32, "python", dict()),                                               # n = 1: nothing projected
+])
+def test_gx_lowrank_matches_oracle(gpu, dtype, L, O, I, rule, variant):
+    """g_x of the schemes "low_rank" / "gilr_gwh" (hot_gx_lowrank): the projected g_y stored untransposed,
+    W quantised without a transform, the product in fp32 and the expansion pass, bit for bit the oracle."""
+    from hot_amd import ops
+    x, w, gy = make_case(L, O, I, seed=L + I, dtype=dtype)
+    ocfg, opt = both_configs(L, rule=rule, **variant)
+    gx = ops.gx_lowrank(gy.to(gpu), w.to(gpu), opt)
+    tr = orc.gx_lowrank(gy.float().numpy(), w.float().numpy(), ocfg)
+    assert gx.dtype == dtype and tuple(gx.shape) == (L, I)
+    assert torch.equal(gx.cpu(), torch.from_numpy(tr.g_x).to(dtype))
+
+
+def test_gx_lowrank_refuses_what_it_cannot_do(gpu):
+    from hot_amd import ops
+    x, w, gy = make_case(256, 64, 32, seed=0)
+    _, opt = both_configs(256, gx_scale=orc.SCALE_ROW)
+    with pytest.raises(ops.HotError, match="one step for the tensor"):
+        ops.gx_lowrank(gy.to(gpu), w.to(gpu), opt)
+    n, rows = orc.hla_rows(128)
+    big = ops.HotOptions(hla_n=n, hla_rows=tuple(int(v) for v in rows))
+    with pytest.raises(ops.HotError, match="token blocks up to 64"):
+        ops.gx_lowrank(gy.to(gpu), w.to(gpu), big)
+
+
+@pytest.mark.parametrize("scheme", ["low_rank", "gilr_gwh"])
+@pytest.mark.parametrize("L", [448, 200])
+def test_hq_linear_lowrank_gx_schemes(gpu, fresh_args, scheme, L):
+    """transform_scheme "low_rank" (utils/quant_matmul.py:184-185,231-232,263-264,296-297,334-335) and
+    "gilr_gwh" (:186-187,233-234,265-266,298-299,336-338) through HQ_Linear: g_x by projection along the
+    tokens and expansion, g_W as in gih_gwlr / hadamard.  Bit-exact against the oracle, within the
+    tolerance against the op-for-op port of those branches."""
+    from hot_amd.quant_matmul import HQ_Linear
+    I, O = 96, 128
+    fresh_args.transform_scheme = scheme
+    torch.manual_seed(2)
+    lin = HQ_Linear(I, O, bias=False).to(gpu)
+    x = torch.randn(L, I, device=gpu, requires_grad=True)
+    gy = torch.randn(L, O, device=gpu) * 1e-3
+    lin(x).backward(gy)
+    xn, gyn, wn = x.detach().cpu().numpy(), gy.cpu().numpy(), lin.weight.detach().cpu().numpy()
+    n_lr, rows_lr = orc.hla_rows(L)                                      # 64 / 36 at 448, 8 / 5 at 200
+    cfg_gx = orc.HotConfig(hla_n=n_lr, hla_rows=tuple(int(v) for v in rows_lr))
+    if scheme == "low_rank":
+        cfg_gw = cfg_gx
+        h_out = torch.zeros(1, 1)
+        h_bs = torch.tensor(orc.make_WHT(L), dtype=torch.float32)
+    else:
+        n16 = orc.pow2_factor_max16(L)
+        cfg_gw = orc.HotConfig(hla_n=n16, hla_rows=tuple(range(n16)))
+        h_out = torch.tensor(orc.make_WHT(L), dtype=torch.float32)
+        h_bs = torch.tensor(orc.make_hadamard(L), dtype=torch.float32)
+    xq_ref, sx_ref = orc.abc_forward(xn, cfg_gw)
+    assert np.array_equal(x.grad.cpu().numpy(), orc.gx_lowrank(gyn, wn, cfg_gx).g_x)
+    assert np.array_equal(lin.weight.grad.cpu().numpy(), orc.linear_backward(gyn, wn, xq_ref, sx_ref, cfg_gw).g_w)
+    xq, sx = fq.setup_context(x.detach().cpu(), h_bs, fq.PortConfig())
+    gi_ref, gw_ref = fq.backward(gy.cpu(), lin.weight.detach().cpu(), xq, sx, h_out, h_bs, fq.PortConfig(), scheme=scheme)
+    assert rel(x.grad.cpu().numpy(), gi_ref.numpy()) < REL_TOL
+    assert rel(lin.weight.grad.cpu().numpy(), gw_ref.numpy()) < REL_TOL
+
+
 @pytest.mark.parametrize("variant", [dict(), dict(gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW,
                                                  gw_round=orc.ROUND_STOCH, gw_scale=orc.SCALE_ROW, seed=3)])
 def test_backward_fp16(gpu, variant):

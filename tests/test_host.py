@@ -116,7 +116,16 @@ def test_options_follow_args(fresh_args):
     o = options_for(12608)
     assert (o.hla_n, o.hla_r, o.hla_rows) == (16, 16, tuple(range(16)))
     assert options_for(197).hla_n == 1 and options_for(200).hla_n == 8
-    a.transform_scheme = "low_rank"
+    a.transform_scheme = "low_rank"                 # g_W side as gih_gwlr; the g_x side has a rule of its own
+    from hot_amd.quant_matmul import gx_token_rule
+    o = options_for(12608)
+    assert (o.hla_n, o.hla_r) == (64, 36)
+    assert gx_token_rule(8192)[0] == 64 and len(gx_token_rule(8192)[1]) == 36    # blocks of at most 64 tokens
+    a.transform_scheme = "gilr_gwh"                 # g_W side as hadamard
+    o = options_for(12608)
+    assert (o.hla_n, o.hla_r) == (16, 16)
+    assert gx_token_rule(12608)[0] == 64
+    a.transform_scheme = "gilro_gwh"
     with pytest.raises(NotImplementedError):
         options_for(64)
     a.transform_scheme = "gih_gwlr"

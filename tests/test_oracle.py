@@ -427,3 +427,49 @@ def test_batched_oracle_reduces_to_the_2d_path():
     gx1, gw1, _ = orc.linear_backward_batched(gy[:1], w, xq1, sx1, cfg)
     tr = orc.linear_backward(gy[0], w, xq2, sx2, cfg)
     assert np.array_equal(gx1[0], tr.g_x) and np.array_equal(gw1, tr.g_w)
+
+
+# ------------------------------------------------------------------ low-rank g_x schemes
+
+def test_hla_expand_is_the_transposed_projection():
+    """P^T t against the explicit block-diagonal matrix product (integer inputs: exact), P P^T = n I
+    (projecting the expansion gives n times the coefficients back), and the full-rank round trip."""
+    rng = np.random.default_rng(5)
+    for n, rows in (orc.hla_rows(64), orc.paper_rows(16, 8), orc.hla_rows(8), (1, np.array([0]))):
+        r, nb, C = len(rows), 3, 7
+        t = rng.integers(-40, 40, (nb * r, C)).astype(np.float32)
+        P = orc.hadamard(n).astype(np.float64)[np.asarray(rows)]
+        ref = np.concatenate([P.T @ t[b * r:(b + 1) * r].astype(np.float64) for b in range(nb)])
+        out = orc.hla_expand(t, n, rows)
+        assert out.dtype == np.float32 and np.array_equal(out, ref.astype(np.float32))
+        assert np.array_equal(orc.fwht_blocks_first(out, n, np.asarray(rows)), n * t)
+    x = rng.standard_normal((128, 3)).astype(np.float32)
+    full = np.arange(32)
+    assert np.abs(orc.hla_expand(orc.fwht_blocks_first(x, 32, full), 32, full) / 32 - x).max() < 1e-5
+
+
+def test_gx_lowrank_against_the_port_and_the_plain_product():
+    """The oracle's g_x of the schemes low_rank / gilr_gwh: within tolerance of the op-for-op port of those
+    branches, and, with INT8 codes and every coefficient kept, close to the plain product g_y W."""
+    import torch
+    from oracle import fakequant_port as fq
+    L, O, I = 448, 64, 40
+    torch.manual_seed(0)
+    x, w, gy = torch.randn(L, I), torch.randn(O, I) * 0.1, torch.randn(L, O) * 1e-3
+    n, rows = orc.hla_rows(L)
+    cfg = orc.HotConfig(hla_n=n, hla_rows=tuple(int(v) for v in rows))
+    got = orc.gx_lowrank(gy.numpy(), w.numpy(), cfg).g_x
+    P = torch.tensor(orc.make_WHT(L), dtype=torch.float32)
+    xq, sx = fq.setup_context(x, P, fq.PortConfig())
+    for scheme, h_out, h_bs in (("low_rank", torch.zeros(1, 1), P),
+                                ("gilr_gwh", P, torch.tensor(orc.make_hadamard(L), dtype=torch.float32))):
+        xq, sx = fq.setup_context(x, h_bs, fq.PortConfig())
+        gi, _ = fq.backward(gy, w, xq, sx, h_out, h_bs, fq.PortConfig(), scheme=scheme)
+        assert np.linalg.norm(got - gi.numpy()) / np.linalg.norm(gi.numpy()) < 1e-3
+    full = orc.HotConfig(hla_n=16, hla_rows=tuple(range(16)), gx_bits=8, w_bits=8)
+    exact = (gy @ w).numpy()
+    assert np.linalg.norm(orc.gx_lowrank(gy.numpy(), w.numpy(), full).g_x - exact) / np.linalg.norm(exact) < 0.02
+    # the projection loses what the dropped rows carried: g_x equals P^T P (g_y W) / n up to quantisation
+    proj = orc.hla_expand(orc.fwht_blocks_first(exact.astype(np.float32), n, np.asarray(rows)), n, rows) / n
+    hi = orc.HotConfig(hla_n=n, hla_rows=tuple(int(v) for v in rows), gx_bits=8, w_bits=8)
+    assert np.linalg.norm(orc.gx_lowrank(gy.numpy(), w.numpy(), hi).g_x - proj) / np.linalg.norm(proj) < 0.02
