@@ -221,3 +221,55 @@ def test_calibration_judges_the_first_batch(fresh_args):
     assert not torch.equal(seen[0], seen[1])
     with pytest.raises(ValueError):
         lqs.GradCapture(m, (HQ_Linear,), keep="middle")
+
+
+# ------------------------------------------------------------------ analytic calculators
+
+def test_bops_formulas_by_hand():
+    """utils/analysis_calculator.py:142-167 at a shape small enough to add up by hand."""
+    from hot_amd.analysis_calculator import backward_bops, forward_bops
+    L, O, I, r, n = 32, 8, 4, 8, 16
+    assert forward_bops(L, O, I) == 32 * 8 * 4 * 1024
+    assert backward_bops("FP", L, O, I) == backward_bops("LoRA", L, O, I) == 2 * 1024 * 1024
+    assert backward_bops("LBP", L, O, I) == (256 * 4 + 128 * 4 + 32 * 32 * 0.5) * 1024
+    assert backward_bops("LUQ", L, O, I) == 3 * (256 + 64 + 256) * 1024 + 2 * 1024 * 32
+    gx = 256 * 4 + 32 * 4 + 256 + 32
+    gw = 128 * 4 + 256 * 4 + 8 * 0.5 * 32 + 4 * 0.5 * 8
+    assert backward_bops("HLQ", L, O, I) == (gx + gw + 32 + 128) * 1024 + 8 * 0.5 * 32 * 4 * 64 + 1024 * 16
+    assert backward_bops("HLQ", L, O, I, frozen=True) == (gx + 128) * 1024 + 1024 * 16
+    # HLQ replaces two fp32 products by an INT4 and a half-length INT8 one: far fewer bit operations at real sizes
+    assert backward_bops("HLQ", 12608, 3072, 768) < 0.05 * backward_bops("FP", 12608, 3072, 768)
+    with pytest.raises(NotImplementedError):
+        backward_bops("other", 1, 1, 1)
+
+
+def test_bops_counter_and_memory_calculator_on_a_small_model():
+    from hot_amd.analysis_calculator import BOPsCounter, ModelMemoryCalculator, backward_bops, forward_bops
+    torch.manual_seed(0)
+    m = Tiny()
+    c = BOPsCounter("HLQ")
+    c.start_counting(m)
+    m(torch.randn(2, 2, 8, 8))
+    c.stop_counting()
+    tot = c.get_total_gbops()
+    # stem: 4 x 4 output positions, 16 out-channels, 2 * 2 * 2 in-features; block.0: [2, 16, 16] -> L = 16
+    assert tot["forward_gbops_by_layer"]["stem"] == forward_bops(16, 16, 8)
+    assert tot["backward_gbops_by_layer"]["block.0"] == backward_bops("HLQ", 16, 32, 16)
+    assert tot["forward_gbops_by_layer"]["head"] == forward_bops(2, 4, 16)          # 2-D input: rows are the tokens
+    assert tot["total_gbops"] == tot["total_forward_gbops"] + tot["total_backward_gbops"]
+    c.reset()
+    assert c.get_total_gbops()["total_gbops"] == 0
+
+    params = sum(p.numel() for p in m.parameters())
+    opt = torch.optim.AdamW(m.parameters())
+    fp = ModelMemoryCalculator(m, (2, 8, 8), batch_size=4, optimizer=opt).get_total_memory()
+    assert fp["parameters"] == fp["gradients"] == 4 * params and fp["optimizer_state"] == 8 * params
+    # outputs of stem [16, 4, 4], dw [16, 4, 4], block.0 [16, 32], block.2 [16, 16], head [4] per sample
+    outs = 256 + 256 + 512 + 256 + 4
+    assert fp["activations"] == outs * 4 * 4
+    hlq = ModelMemoryCalculator(m, (2, 8, 8), batch_size=4, optimizer=None, isHLQ=True).get_total_memory()
+    assert hlq["activations"] == (128 + 128 + 256 + 128 + 2) * 4 and hlq["optimizer_state"] == 0
+    m.head.weight.requires_grad_(False)
+    frozen = ModelMemoryCalculator(m, (2, 8, 8), batch_size=4).get_total_memory()
+    assert frozen["activations"] == (outs - 4) * 4 * 4 and frozen["parameters"] == 4 * (params - 64)
+    assert ModelMemoryCalculator.format_bytes(3 * 1024 ** 3) == "3.00GB"
