@@ -109,6 +109,12 @@ __global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
   const int kc = (int)(blockIdx.y - blk * a.nk);
   const int k = a.klist[kc];
   const int qmax = (1 << (a.bits - 1)) - 1;
+  // The table entries of this coefficient index (one per run) go through LDS: read from global memory
+  // inside the quantise loop they would sit between the loop's byte stores, and every such load then
+  // waits for the store before it (one memory round trip per kept row).
+  __shared__ int32_t s_tab[M];
+  if (tid < M) s_tab[tid] = a.tab[tid * 64 + k];
+  __syncthreads();
   float v[M];
   if (active) {
     const float* t = a.T + ((blk * M) * a.nk + kc) * a.C + c;
@@ -125,7 +131,7 @@ __global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
     double ssq = 0.0, sab = 0.0;
 #pragma unroll
     for (int j = 0; j < M; ++j) {
-      if (a.tab[j * 64 + k] >= 0) {
+      if (s_tab[j] >= 0) {
         cmax = fmaxf(cmax, fabsf(v[j]));
         if constexpr (SAWB) { ssq += (double)v[j] * (double)v[j]; sab += (double)fabsf(v[j]); }
       }
@@ -162,16 +168,17 @@ __global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
     if (a.mode == HOT_SCALE_ROW) d = a.colmax[c] / (float)qmax + 1e-11f;
     else if (a.mode == HOT_SCALE_TENSOR) d = a.stat[0] / (float)qmax + 1e-11f;
     else { d = a.stat[1] + 1e-11f; clip = a.stat[2]; }
+    const float rcp = 1.0f / d;
 #pragma unroll
     for (int j = 0; j < M; ++j) {
-      const int32_t e = a.tab[j * 64 + k];
+      const int32_t e = s_tab[j];
       if (e < 0) continue;
       const int slot = e & 0xFFFF, visit = e >> 16;
       float x = v[j];
       if constexpr (SAWB) x = fminf(fmaxf(x, -clip), clip);
       int q;
       if constexpr (ROUND == HOT_ROUND_NEAREST) {
-        q = (int)rintf(x / d);
+        q = (int)rint_div_fast(x, d, rcp);      // bit for bit rintf(x / d)
       } else {
         const uint64_t idx = ((uint64_t)c * (uint64_t)a.NB + (uint64_t)blk) * (uint64_t)a.rpad + (uint64_t)visit;
         q = clampi(q_stoch(x / d, uniform_of(idx, a.seed, a.stream)), -qmax, qmax);
