@@ -555,7 +555,7 @@ static BatchedLayout batched_layout(int64_t B, int64_t T, int64_t O, int64_t I, 
   size_t o = 0;
   b.off_colw = o; o += align256(colwise_workspace_bytes_impl(I));
   b.off_colg = o; o += align256(colwise_group_workspace_bytes_impl(O, (int)B));
-  b.off_hq = o;   o += align256((size_t)B * 4 > STAT_SLOT_BYTES ? (size_t)B * 4 : STAT_SLOT_BYTES);
+  b.off_hq = o;   o += align256((size_t)B * 128 > STAT_SLOT_BYTES ? (size_t)B * 128 : STAT_SLOT_BYTES);
   b.off_sg = o;   o += align256((size_t)L * 4);
   b.off_sw = o;   o += 256;
   b.off_sgp = o;  o += align256((size_t)B * (size_t)O * 4);

@@ -35,6 +35,8 @@ constexpr size_t COL_STAT_BYTES = 256 + STAT_SLOT_BYTES;   // step / clip words,
 constexpr int COLMAX_COPIES = 8;  // per-channel maxima: workgroup row y folds into copy y % 8 (fewer atomics per line)
 constexpr int CW_ROWS = 16;    // rows staged per step
 
+constexpr int GS = 32;   // floats between the statistics of two sample groups (one 128-byte line each)
+
 struct ColArgs {
   const void* in;
   int64_t R, C;       // input rows (transform dim) and channels
@@ -56,8 +58,9 @@ struct ColArgs {
   // Sample groups (3-D activations: one step per sample).  The R rows are `groups` samples of NBs
   // token blocks each; a workgroup's run of blocks never leaves its sample (`runs` runs per sample),
   // the codes of a sample take Kpad bytes of every output row (the tail zeroed), and the statistics
-  // are kept per sample: gstat[g] (absmax, TENSOR), gstat[groups + 2 g] / [.. + 1] (step / clip,
-  // SAWB), colmax[g * C + c] (ROW).  groups == 1: the whole input is one group with Kpad = ld_out.
+  // are kept per sample: gstat[GS g] (absmax, TENSOR), gstat[GS g + 1] / [GS g + 2] (step / clip,
+  // SAWB) -- a 128-byte line per sample, since every workgroup of a sample updates its absmax
+  // and updates of one line queue up behind each other at the memory side --, colmax[g * C + c] (ROW).  groups == 1: the whole input is one group with Kpad = ld_out.
   int32_t groups, runs;
   int64_t NBs, Kpad;
   float* gstat;
@@ -152,9 +155,18 @@ __device__ __forceinline__ void wait_stream() {
 }
 
 __device__ __forceinline__ void dma16_to_lds(uint32_t lds_addr, uint32_t voff, const uint8_t* sbase) {
+  // lds_addr and sbase are wave-uniform by construction; said explicitly, since the instruction takes
+  // them in scalar registers and the compiler keeps a uniform value in a vector register when it was
+  // computed past lane-dependent control flow.  (The builtin returns a signed int: every half goes
+  // through uint32_t, or a low half with its top bit set would sign-extend over the high half.)
+  const uint64_t b64 = (uint64_t)(uintptr_t)sbase;
+  const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b64 >> 32));
+  const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b64);
+  const uint8_t* base = reinterpret_cast<const uint8_t*>(((uint64_t)b_hi << 32) | (uint64_t)b_lo);
+  const uint32_t lds_u = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_addr);
   asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                :
-               : "s"(lds_addr), "v"(voff), "s"(sbase)
+               : "s"(lds_u), "v"(voff), "s"(base)
                : "memory", "m0");
 }
 
@@ -262,12 +274,12 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
         d = active ? sc + 1e-11f : 1.f;
         if (active && run == 0) a.scales_out[(int64_t)sample * a.C + c] = sc;
       } else if (a.mode == HOT_SCALE_TENSOR) {
-        const float sc = a.gstat[sample] / (float)qmax;
+        const float sc = a.gstat[GS * sample] / (float)qmax;
         d = sc + 1e-11f;
         if (bx == 0 && run == 0 && tid == 0) a.scales_out[sample] = sc;
       } else {
-        d = a.gstat[a.groups + 2 * sample] + 1e-11f;
-        clip = a.gstat[a.groups + 2 * sample + 1];
+        d = a.gstat[GS * sample + 1] + 1e-11f;
+        clip = a.gstat[GS * sample + 2];
       }
     } else if (a.mode == HOT_SCALE_ROW) {
       float cm = 0.f;
@@ -294,6 +306,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
   float x[XL];
 
   // Transforms and consumes the token blocks held in x; `bl` is the group-local index of the first.
+  philox_words u1 = {0u, 0u, 0u, 0u};
   auto consume = [&](int bl) {
     fwht_regs<N, XL, (RSP && N >= 2) ? 2 : 1>(x);   // the fused statistics pass runs stage h = 1 while loading
 #pragma unroll
@@ -304,6 +317,14 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
         if constexpr (PASS == 0) csum += x[g * N];
         int visited = 0;      // kept coefficients of this block quantised so far (stochastic rounding)
         float u[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        if constexpr (PASS == 1 && ROUND != HOT_ROUND_NEAREST && N == 1) {
+          // blocks of one token keep their one coefficient: element number = channel * NB + block, so
+          // eight consecutive blocks of a channel share a generator call (u1 lives across the blocks
+          // of this step; a new call at the first block and wherever the number passes a multiple of 8)
+          const uint64_t e = (uint64_t)c * (uint64_t)a.NB + (uint64_t)(blk0 + blk);
+          if (g == 0 || (e & 7u) == 0) u1 = sr_octet_words(e >> 3, a.seed, a.stream);
+          u[0] = sr_uniform_of(u1, (uint32_t)e);
+        }
 #pragma unroll
         for (int i = 0; i < N; ++i) {
           int sl;
@@ -322,10 +343,18 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
                 q = (int)rint_div_fast(v, d, rcp);
               } else {
                 // counter = ((channel * NB + block) * rpad + visit index) / 8, slot = visit index % 8
-                if ((visited & 7) == 0) {
-                  const uint64_t oct = ((uint64_t)c * (uint64_t)a.NB + (uint64_t)(blk0 + blk)) * (uint64_t)(a.rpad >> 3) +
-                                       (uint64_t)(visited >> 3);
-                  sr_uniform8(oct, a.seed, a.stream, u);
+                // (blocks of one token: u[0] was drawn above)
+                if (N > 1 && (visited & 7) == 0) {
+                  if (a.r == 1) {
+                    // a single kept coefficient per block: numbered channel * NB + block, like the
+                    // one-token blocks above
+                    const uint64_t e = (uint64_t)c * (uint64_t)a.NB + (uint64_t)(blk0 + blk);
+                    u[0] = sr_uniform_of(sr_octet_words(e >> 3, a.seed, a.stream), (uint32_t)e);
+                  } else {
+                    const uint64_t oct = ((uint64_t)c * (uint64_t)a.NB + (uint64_t)(blk0 + blk)) * (uint64_t)(a.rpad >> 3) +
+                                         (uint64_t)(visited >> 3);
+                    sr_uniform8(oct, a.seed, a.stream, u);
+                  }
                 }
                 q = q_stoch_div(v, d, rcp, u[visited & 7]);
                 ++visited;
@@ -463,7 +492,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
       if (tid == 0) {
         float mm = s_max[0];
         for (int i = 1; i < CW / 64; ++i) mm = fmaxf(mm, s_max[i]);
-        if (a.groups > 1) atomic_max_nonneg(a.gstat + sample, mm);
+        if (a.groups > 1) atomic_max_nonneg(a.gstat + GS * sample, mm);
         else stat_slot_update(a.slots, wg_id, mm);
       }
       return;
@@ -584,8 +613,8 @@ __global__ void __launch_bounds__(256) colwise_finalize_kernel(const ColArgs a, 
     const float clip = (float)(12.1 * sqrt(s_q[0] / cnt) - 12.2 * (s_b[0] / cnt));
     const float s = clip / qmax;
     if (a.groups > 1) {
-      a.gstat[a.groups + 2 * g] = s;
-      a.gstat[a.groups + 2 * g + 1] = clip;
+      a.gstat[GS * g + 1] = s;
+      a.gstat[GS * g + 2] = clip;
       a.scales_out[g] = s;
     } else {
       a.stat[1] = s;
@@ -678,7 +707,7 @@ size_t colwise_workspace_bytes_impl(int64_t C) {
 
 // with sample groups: stat | per-sample per-channel max | per-sample statistics | partial sums
 static size_t group_colmax_bytes(int64_t C, int groups) { return (size_t)round_up(C * 4 * (int64_t)groups, 256); }
-static size_t group_gstat_bytes(int groups) { return (size_t)round_up((int64_t)groups * 3 * 4, 256); }
+static size_t group_gstat_bytes(int groups) { return (size_t)round_up((int64_t)groups * GS * 4, 256); }
 size_t colwise_group_workspace_bytes_impl(int64_t C, int groups) {
   if (groups <= 1) return colwise_workspace_bytes_impl(C);
   return COL_STAT_BYTES + group_colmax_bytes(C, groups) + group_gstat_bytes(groups) + (size_t)(2 * sizeof(double)) * 65536;
@@ -749,7 +778,7 @@ static int launch_colwise(ColArgs& a, hipStream_t st) {
   const dim3 grid((unsigned)gx, (unsigned)gy);
   if (!a.stats_cleared) {
     const int64_t ncolmax = a.mode == HOT_SCALE_ROW ? (a.groups > 1 ? a.C * a.groups : a.C * COLMAX_COPIES) : 0;
-    const int64_t ngstat = a.groups > 1 ? 3 * (int64_t)a.groups : 0;
+    const int64_t ngstat = a.groups > 1 ? GS * (int64_t)a.groups : 0;
     int64_t nclr = (int64_t)(COL_STAT_BYTES / 4);
     if (ncolmax > nclr) nclr = ncolmax;
     if (ngstat > nclr) nclr = ngstat;

@@ -337,7 +337,7 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
   uint8_t* ws = (uint8_t*)workspace;
   BigArgs a;
   a.in = in; a.T = (float*)(ws + b.off_T); a.tmp = (int8_t*)(ws + b.off_tmp); a.tab = (const int32_t*)(ws + b.off_tab);
-  a.R = R; a.C = C; a.NB = NB; a.n = n; a.r = r; a.rpad = (r + 7) & ~7; a.bits = bits; a.rounding = rounding;
+  a.R = R; a.C = C; a.NB = NB; a.n = n; a.r = r; a.rpad = r == 1 ? 1 : (r + 7) & ~7; a.bits = bits; a.rounding = rounding;
   a.mode = scale_mode; a.stat = (float*)ws; a.colmax = (float*)(ws + b.off_colmax);
   a.partial = (double*)(ws + b.off_partial); a.scales_out = scales_out; a.seed = seed; a.stream = rng_stream;
   a.kmask = kmask; a.nk = 0;

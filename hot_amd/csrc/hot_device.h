@@ -144,6 +144,25 @@ __device__ __forceinline__ void sr_uniform8(uint64_t oct, uint64_t seed, uint32_
   }
 }
 
+// The same numbers one at a time, for callers that walk element indices which are not a compile-time
+// sequence: the four output words of the call for octet e / 8 live in named registers (no array, so
+// nothing the compiler could turn into an indexed access to scratch memory) and the uniform of
+// element e is picked with selects and a shift.
+struct philox_words { uint32_t w0, w1, w2, w3; };
+__device__ __forceinline__ philox_words sr_octet_words(uint64_t oct, uint64_t seed, uint32_t stream) {
+  const philox4 p = philox4x32_10((uint32_t)oct, (uint32_t)(oct >> 32), stream, 0u,
+                                  (uint32_t)seed, (uint32_t)(seed >> 32));
+  philox_words o;
+  o.w0 = p.w[0]; o.w1 = p.w[1]; o.w2 = p.w[2]; o.w3 = p.w[3];
+  return o;
+}
+__device__ __forceinline__ float sr_uniform_of(const philox_words& p, uint32_t e) {
+  const uint32_t i = (e >> 1) & 3u;
+  const uint32_t lo = (i & 1u) ? p.w1 : p.w0, hi = (i & 1u) ? p.w3 : p.w2;
+  const uint32_t w = (i & 2u) ? hi : lo;
+  return (float)((w >> ((e & 1u) * 16u)) & 0xFFFFu) * 1.52587890625e-05f;
+}
+
 // ---- quantisation of one value --------------------------------------------
 
 // y = x / d already divided.  Nearest: ties to even.

@@ -36,7 +36,7 @@ int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int 
                     bool absmax_ready = false, int64_t group_rows = 0, float* group_steps = nullptr);
 // group_rows > 0 (per-tensor steps only): every run of group_rows rows is a sample with a step of its
 // own; scales_out then holds M entries (the step of each row's sample, the form the GEMM epilogue
-// reads), group_steps (may be null) the M / group_rows steps, and the workspace 4 bytes per sample.
+// reads), group_steps (may be null) the M / group_rows steps, and the workspace 128 bytes per sample.
 
 int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r,
                        int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,

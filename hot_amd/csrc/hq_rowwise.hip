@@ -212,6 +212,9 @@ __global__ void hq_tensor_kernel(const T* __restrict__ in, int64_t nchunks, int6
 }
 
 // ---- one scale per group of rows (3-D activations: a group is a sample) -------------------------
+// The absmax of group g is collected at gmax[g * GROUP_STAT_STRIDE]: a 128-byte line per group, since
+// every workgroup of a group updates it and updates of one line queue up at the memory side.
+constexpr int GROUP_STAT_STRIDE = 32;
 // grid (blocks per group, groups); a block walks its group's chunks with a stride of the group's blocks
 
 template <typename T, int N>
@@ -234,7 +237,7 @@ __global__ void hq_group_absmax_kernel(const T* __restrict__ in, int64_t chunks_
   if (threadIdx.x == 0) {
     float m = s_red[0];
     for (int i = 1; i < (int)(blockDim.x >> 6); ++i) m = fmaxf(m, s_red[i]);
-    atomic_max_nonneg(gmax + g, m);
+    atomic_max_nonneg(gmax + g * GROUP_STAT_STRIDE, m);
   }
 }
 
@@ -248,7 +251,7 @@ __global__ void hq_group_quant_kernel(const T* __restrict__ in, int64_t chunks_p
   const int lane = threadIdx.x & 63;
   const int64_t g = blockIdx.y;
   constexpr float QMAXF = (float)((1 << (BITS - 1)) - 1);
-  const float s = gmax[g] / QMAXF;
+  const float s = gmax[g * GROUP_STAT_STRIDE] / QMAXF;
   const float d = s + 1e-11f;
   const float rcp = 1.0f / d;
   if (group_steps && blockIdx.x == 0 && threadIdx.x == 0) group_steps[g] = s;
@@ -338,7 +341,7 @@ static int launch_groups(const void* in, int64_t M, int64_t K, void* codes, int6
   if (bx < 1) bx = 1;
   if (groups > 65535) return fail(HOT_ERR_UNSUPPORTED, "hot_hq_rowwise: more than 65535 sample groups");
   const dim3 grid((unsigned)bx, (unsigned)groups);
-  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((groups + 255) / 256)), dim3(256), 0, st, (uint32_t*)gmax, 0u, (int)groups);
+  hipLaunchKernelGGL(fill_u32_kernel, dim3((unsigned)((groups * GROUP_STAT_STRIDE + 255) / 256)), dim3(256), 0, st, (uint32_t*)gmax, 0u, (int)(groups * GROUP_STAT_STRIDE));
   hipLaunchKernelGGL((hq_group_absmax_kernel<T, N>), grid, dim3(256), 0, st, (const T*)in, cpg, gmax, nrt);
   hipLaunchKernelGGL((hq_group_quant_kernel<T, N, BITS, ROUND>), grid, dim3(256), 0, st, (const T*)in, cpg, K / EPL, ld, gmax,
                      (int8_t*)codes, scales, group_steps, seed, stream_id, nrt);
@@ -405,7 +408,7 @@ int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int 
   if (group_rows < 0 || (group_rows > 0 && (M % group_rows || scale_mode != HOT_SCALE_TENSOR)))
     return fail(HOT_ERR_INVALID, "hot_hq_rowwise: %lld rows are not whole groups of %lld rows with one step each", (long long)M, (long long)group_rows);
   if (scale_mode == HOT_SCALE_TENSOR) {
-    const size_t need = group_rows > 0 ? (size_t)(M / group_rows) * 4 : STAT_SLOT_BYTES;
+    const size_t need = group_rows > 0 ? (size_t)(M / group_rows) * 128 : STAT_SLOT_BYTES;
     if (!workspace || workspace_bytes < need) return fail(HOT_ERR_WORKSPACE, "hot_hq_rowwise: per-tensor scale needs a %zu-byte workspace", need);
     absmax = (float*)workspace;
   }

@@ -407,10 +407,12 @@ def colwise_rng_index(C: int, NB: int, rows) -> np.ndarray:
     matrix, laid out [C, NB * r] (K-major).  The kernels walk the kept
     coefficients of a block in increasing natural-row order and number them
     ((c * NB + block) * rpad + visit) with rpad = r rounded up to 8, so that one
-    Philox call serves eight consecutive visits of a channel."""
+    Philox call serves eight consecutive visits of a channel.  Blocks with a single kept
+    coefficient (r = 1: the one-token blocks of token counts no power of two divides) are numbered
+    c * NB + block (rpad = 1), so that eight consecutive blocks of a channel share a call."""
     rows = np.asarray(rows)
     r = len(rows)
-    rpad = (r + 7) // 8 * 8
+    rpad = 1 if r == 1 else (r + 7) // 8 * 8
     visit = np.argsort(np.argsort(rows))                      # rank of rows[k] among the kept rows
     c = np.arange(C, dtype=np.int64)[:, None, None]
     b = np.arange(NB, dtype=np.int64)[None, :, None]

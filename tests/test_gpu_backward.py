@@ -358,6 +358,8 @@ def test_hq_linear_3d_input(gpu, fresh_args, mode):
     (7, 48, 64, 40, dict(gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW, gw_round=orc.ROUND_STOCH,
                          gw_scale=orc.SCALE_ROW, gx_bits=8, w_bits=8, seed=5)),
     (130, 197, 128, 64, dict()),                                                  # more samples than a ViT batch
+    (6, 197, 80, 136, dict(gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW, gw_round=orc.ROUND_STOCH,
+                           act_round=orc.ROUND_STOCH, seed=9)),                      # one-token blocks, stochastic
 ])
 def test_backward_batched_matches_oracle(gpu, dtype, B, T, O, I, variant):
     """3-D activations through the batched entry points (one call per layer, one set of steps per

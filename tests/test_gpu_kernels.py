@@ -205,6 +205,26 @@ def test_hla_tokenwise_stochastic_matches_oracle(gpu, scale):
     assert np.array_equal(codes.cpu().numpy()[:, :kout], q_ref)
 
 
+@pytest.mark.parametrize("scale", ["tensor", "row"])
+@pytest.mark.parametrize("L,C,n,rows", [
+    (197, 264, 1, [0]),          # one-token blocks: eight consecutive blocks of a channel share a generator call
+    (49, 72, 1, [0]),
+    (1000, 520, 1, [0]),         # three channel strips, runs of blocks that start off a multiple of eight
+    (16 * 21, 40, 16, [5]),      # a single kept row of a 16-token block: numbered the same way
+])
+def test_hla_tokenwise_stochastic_single_coefficient_blocks(gpu, scale, L, C, n, rows):
+    from hot_amd import ops
+    x, xn = hla_case(L, C, "f32", seed=L)
+    codes, s, kout = ops.hla_tokenwise(x.to(gpu), n, rows, bits=8, rounding="stoch", scale=scale, seed=31)
+    t = np.ascontiguousarray(orc.fwht_blocks_first(xn, n, np.asarray(rows)).T)
+    mode = orc.SCALE_ROW if scale == "row" else orc.SCALE_TENSOR
+    idx = orc.colwise_rng_index(C, L // n, rows)
+    assert np.array_equal(idx, np.arange(C * (L // n)).reshape(C, L // n))      # channel * NB + block
+    q_ref, s_ref = orc.quant(t, 8, mode, orc.ROUND_STOCH, 31, orc.STREAM_GW, index=idx)
+    assert np.array_equal(s.cpu().numpy(), s_ref)
+    assert np.array_equal(codes.cpu().numpy()[:, :kout], q_ref)
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("bits", [4, 8])
 @pytest.mark.parametrize("n", [16, 32, 64])
