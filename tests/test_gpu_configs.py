@@ -1,6 +1,7 @@
 """The benchmark configurations at their own size, through the C ABI, against the CPU oracle.
 
-  * the four ViT-B layer shapes at 64 x 197 tokens, fp32 and bf16, quantiser variants;
+  * the four ViT-B layer shapes at 64 x 197 tokens, fp32 and bf16, quantiser variants; two of them as
+    [64, 197, C] activations with per-sample steps (the reference's own treatment of a batch);
   * the kernel-level sweep of the row-wise Hadamard quantiser (M up to 65536, K up to 11008, per-channel
     scales drawn log-uniform), oracle on sampled rows: rows are independent under per-token steps;
   * the Llama-7B shapes at 8192 tokens with heavy-tailed (Student-t) gradient columns: steps of the
@@ -93,6 +94,38 @@ def test_vit_b_layers_full_size_quantiser_variants(gpu, layer, dtype, variant):
 
 
 # ------------------------------------------------------------ kernel-level sweep of the row-wise quantiser
+
+@pytest.mark.parametrize("layer,variant", [
+    ("proj", dict()),
+    ("qkv", dict(gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW, gw_round=orc.ROUND_STOCH, seed=5)),
+])
+def test_vit_b_layers_per_sample_steps(gpu, layer, variant):
+    """The reference's own treatment of the ViT batch: [64, 197, C] activations, every sample with steps
+    of its own (197 tokens: one-token blocks, nothing projected), through the batched entry points at
+    the layer's real size; activation buffer, g_x and the summed g_W against the oracle, bf16."""
+    from hot_amd import ops
+    O, I = VIT_SHAPES[layer]
+    B, T = 64, 197
+    x, w, gy = vit_inputs(B * T, O, I, torch.bfloat16, seed=O + I + 1)
+    g = torch.Generator().manual_seed(3)
+    mag = (10.0 ** (torch.rand(B, 1, 1, generator=g) * 2 - 1)).to(torch.bfloat16)        # samples of different size
+    x3, gy3 = x.reshape(B, T, I), (gy.reshape(B, T, O) * mag).contiguous()
+    ocfg = orc.HotConfig.python_rule(T, **variant)
+    assert ocfg.hla_n == 1
+    opt = options_pair(ocfg)
+    xq, sx = ops.abc_forward_batched(x3.to(gpu), opt)
+    gx, gw = ops.linear_backward_batched(gy3.to(gpu), w.to(gpu), xq, sx, opt)
+    ranges = ops.backward_batched_ranges(B, T, O, I, opt)
+    xq_ref, sx_ref = orc.abc_forward_batched(x3.float().numpy(), ocfg)
+    gx_ref, gw_ref, _ = orc.linear_backward_batched(gy3.float().numpy(), w.float().numpy(), xq_ref, sx_ref, ocfg,
+                                                    gw_ranges=ranges)
+    kg = ops.kpad_group(T, opt)
+    got = xq.cpu().numpy().reshape(I, B, kg)
+    assert np.array_equal(got[:, :, :T], xq_ref.transpose(2, 0, 1)) and not got[:, :, T:].any()
+    assert np.array_equal(sx.cpu().numpy(), sx_ref)
+    assert torch.equal(gx.cpu(), torch.from_numpy(gx_ref).to(torch.bfloat16))
+    assert torch.equal(gw.cpu(), torch.from_numpy(gw_ref).to(torch.bfloat16))
+
 
 @pytest.mark.parametrize("M", [4096, 16384, 65536])
 @pytest.mark.parametrize("K", [768, 3072, 4096, 11008])
