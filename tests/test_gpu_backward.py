@@ -360,6 +360,9 @@ def test_hq_linear_3d_input(gpu, fresh_args, mode):
     (130, 197, 128, 64, dict()),                                                  # more samples than a ViT batch
     (6, 197, 80, 136, dict(gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW, gw_round=orc.ROUND_STOCH,
                            act_round=orc.ROUND_STOCH, seed=9)),                      # one-token blocks, stochastic
+    (1, 128, 48, 24, dict()),                                                     # a batch of one
+    (3, 64, 16, 8, dict(gw_scale=orc.SCALE_ROW)),                                 # one block per sample, smallest widths
+    (2, 576, 256, 384, dict(gx_bits=8, w_bits=8)),                                # 324 codes per sample: three stages per group
 ])
 def test_backward_batched_matches_oracle(gpu, dtype, B, T, O, I, variant):
     """3-D activations through the batched entry points (one call per layer, one set of steps per
