@@ -218,16 +218,33 @@ def gemm_i8(a: torch.Tensor, b: torch.Tensor, k: int, bits: int, scale_a: torch.
     return (out, acc) if return_acc else out
 
 
-def abc_forward(x: torch.Tensor, opt: HotOptions):
-    """INT8 Hadamard-compressed activation buffer: (xq int8 [I, kpad(L')], sx fp32 [1])."""
+def _launch_stream(side: Optional["torch.cuda.Stream"]) -> int:
+    return _stream() if side is None else side.cuda_stream
+
+
+def _join(side: Optional["torch.cuda.Stream"]) -> None:
+    # the current stream waits for what `side` was given: enqueued before the call returns (and so
+    # before its workspace goes back to the allocator), which orders every later use of the outputs
+    # and of the workspace's memory on the current stream behind the kernels
+    if side is not None:
+        torch.cuda.current_stream().wait_stream(side)
+
+
+def abc_forward(x: torch.Tensor, opt: HotOptions, side: Optional["torch.cuda.Stream"] = None):
+    """INT8 Hadamard-compressed activation buffer: (xq int8 [I, kpad(L')], sx fp32 [1]).
+    With `side` the kernels run on that stream (which must already wait for x) beside whatever the
+    current stream is doing, and the current stream joins it before the call returns."""
     _need_gpu_2d(x, "X")
     L, I = x.shape
     cfg = opt.to_c()
     xq = torch.empty((I, kpad(opt.lprime(L))), dtype=torch.int8, device=x.device)
     sx = torch.empty((1,), dtype=torch.float32, device=x.device)
     ws = _ws(_lib.lib().hot_abc_workspace_bytes(L, I, C.byref(cfg)), x.device)
-    _lib.check(_lib.lib().hot_abc_forward(x.data_ptr(), _dt(x), L, I, C.byref(cfg), xq.data_ptr(), sx.data_ptr(),
-                                          ws.data_ptr(), ws.numel(), _stream()))
+    try:
+        _lib.check(_lib.lib().hot_abc_forward(x.data_ptr(), _dt(x), L, I, C.byref(cfg), xq.data_ptr(), sx.data_ptr(),
+                                              ws.data_ptr(), ws.numel(), _launch_stream(side)))
+    finally:
+        _join(side)
     return xq, sx
 
 
@@ -288,9 +305,9 @@ def backward_batched_ranges(B: int, T: int, O: int, I: int, opt: HotOptions) -> 
     return int(_lib.lib().hot_backward_batched_ranges(int(B), int(T), int(O), int(I), C.byref(opt.to_c())))
 
 
-def abc_forward_batched(x: torch.Tensor, opt: HotOptions):
+def abc_forward_batched(x: torch.Tensor, opt: HotOptions, side: Optional["torch.cuda.Stream"] = None):
     """Activation buffer of a 3-D input [B, T, I] with one step per sample (hot_abc_forward_batched):
-    (xq int8 [I, B * kpad_group(T)], sx fp32 [B])."""
+    (xq int8 [I, B * kpad_group(T)], sx fp32 [B]).  `side`: as in abc_forward."""
     if not x.is_cuda or x.dim() != 3 or not x.is_contiguous():
         raise RuntimeError("X must be a contiguous CUDA tensor [B, T, I]!")
     B, T, I = x.shape
@@ -299,8 +316,11 @@ def abc_forward_batched(x: torch.Tensor, opt: HotOptions):
     xq = torch.empty((I, B * kg), dtype=torch.int8, device=x.device)
     sx = torch.empty((B,), dtype=torch.float32, device=x.device)
     ws = _ws(_lib.lib().hot_abc_batched_workspace_bytes(B, T, I, C.byref(cfg)), x.device)
-    _lib.check(_lib.lib().hot_abc_forward_batched(x.data_ptr(), _dt(x), B, T, I, C.byref(cfg), xq.data_ptr(), sx.data_ptr(),
-                                                  ws.data_ptr(), ws.numel(), _stream()))
+    try:
+        _lib.check(_lib.lib().hot_abc_forward_batched(x.data_ptr(), _dt(x), B, T, I, C.byref(cfg), xq.data_ptr(),
+                                                      sx.data_ptr(), ws.data_ptr(), ws.numel(), _launch_stream(side)))
+    finally:
+        _join(side)
     return xq, sx
 
 

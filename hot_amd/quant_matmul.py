@@ -18,6 +18,7 @@ from __future__ import annotations
 
 from typing import Optional, Tuple
 
+import threading
 from dataclasses import replace
 
 import numpy as np
@@ -169,6 +170,40 @@ def _pad8(t: Tensor) -> Tensor:
 _PLAIN_APPLY = hasattr(torch._C, "_are_functorch_transforms_active")
 
 
+# The activation buffer is written beside the forward GEMM, not behind it: the two read the same x and
+# neither needs the other (the GEMM is bound by the matrix cores, the buffer kernels by memory).
+# forward() records an event on the current stream before it launches the GEMM; setup_context, which
+# autograd calls right after forward on the same thread, lets a side stream wait for that event, runs
+# the buffer kernels there and makes the current stream wait for them.  One side stream per device,
+# default priority.  Not under stream capture (a capture must not be forked behind its back).
+_FWD = threading.local()
+_SIDE_STREAMS: dict = {}
+overlap_buffer_write = True
+
+
+def _mark_input_ready(x: Tensor) -> None:
+    _FWD.event = None
+    if not (overlap_buffer_write and x.is_cuda) or hot_switched_off() or torch.cuda.is_current_stream_capturing():
+        return
+    ev = torch.cuda.Event()
+    ev.record()
+    _FWD.event = (ev, x.data_ptr())
+
+
+def _buffer_stream(x: Tensor):
+    """The side stream for the buffer kernels of this layer, already waiting for x; None = run in line."""
+    mark = getattr(_FWD, "event", None)
+    _FWD.event = None
+    if mark is None or mark[1] != x.data_ptr():
+        return None
+    key = x.device.index
+    side = _SIDE_STREAMS.get(key)
+    if side is None:
+        side = _SIDE_STREAMS[key] = torch.cuda.Stream(device=x.device)
+    side.wait_event(mark[0])
+    return side
+
+
 class FLinearQ(Function):
     """torch.autograd.Function with the reference's forward / setup_context /
     backward triple (utils/quant_matmul.py:169-348)."""
@@ -186,6 +221,7 @@ class FLinearQ(Function):
         # `bias` is an addition to the reference's five arguments (which adds the bias after the
         # Function, utils/quant_matmul.py:419-420): inside, it rides in the GEMM epilogue instead of
         # costing a pass over the output
+        _mark_input_ready(x)
         return F.linear(x, w, bias)
 
     @staticmethod
@@ -201,6 +237,7 @@ class FLinearQ(Function):
         # the kernels move 16-byte vectors: feature counts that are not multiples of 8 are padded with
         # zero channels, which change neither a Hadamard block of the real channels nor any absmax
         ctx.batched = False
+        side = _buffer_stream(x)
         if x.dim() == 3 and args.batched_mode == "per_sample":
             # the reference's treatment of 3-D activations: every sample has steps of its own
             tokens = x.shape[1]
@@ -209,7 +246,7 @@ class FLinearQ(Function):
             if opt.hla_n <= 128:
                 # one call per layer: the library keeps the samples apart
                 ctx.batched = True
-                xq, sx = ops.abc_forward_batched(_pad8(x), opt)
+                xq, sx = ops.abc_forward_batched(_pad8(x), opt, side=side if x.shape[-1] % 8 == 0 and x.is_contiguous() else None)
             else:
                 bufs = [ops.abc_forward(_pad8(x[b]), opt) for b in range(x.shape[0])]
                 xq = torch.stack([b[0] for b in bufs])
@@ -218,7 +255,7 @@ class FLinearQ(Function):
             x2 = x.reshape(-1, x.shape[-1])
             opt = options_for(x2.shape[0], name, w.shape[0])
             _check_padding(w, opt)
-            xq, sx = ops.abc_forward(_pad8(x2), opt)
+            xq, sx = ops.abc_forward(_pad8(x2), opt, side=side if x2.shape[-1] % 8 == 0 and x2.data_ptr() == x.data_ptr() and x2.is_contiguous() else None)
         ctx.opt = opt
         args.sr_step += 1
         ctx.save_for_backward(xq, w, sx)
