@@ -529,6 +529,73 @@ int hot_gx_lowrank(const void* gy, const void* w, int dtype, int64_t L, int64_t 
   return hla_expand_impl(t, L / cfg->hla_n, I, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, 1.0f / (float)cfg->hla_n, gx, out_dtype, st);
 }
 
+// ---- g_x with the logarithmic quantiser on g_y -----------------------------------------------------
+// quantBWDGogi = "luq" (utils/quant_matmul.py:238,252-253,270,276-285,288-290,343): g_y blkdiag(H) through
+// luq_quantizer_BWD, blkdiag(H) W through the weight quantiser, their integer product, the two steps,
+// / n_o.  The LUQ codes are powers of two up to 2^(lev + 1) and travel as two INT8 planes (q = 16 a + b);
+// W's INT4-range codes are stored as bytes and doubled into [16 w | w]; one INT8 product over twice the K.
+
+struct LuqLayout {
+  int64_t kp;
+  size_t off_colw, off_slots, off_sg, off_sw, off_qg, off_qw, off_qw2, total;
+};
+
+static LuqLayout luq_layout(int64_t L, int64_t O, int64_t I) {
+  LuqLayout b;
+  b.kp = round_up(O, GEMM_KTILE);
+  size_t o = 0;
+  b.off_colw = o;  o += align256(colwise_workspace_bytes_impl(I));
+  b.off_slots = o; o += STAT_SLOT_BYTES;
+  b.off_sg = o;    o += 256;
+  b.off_sw = o;    o += 256;
+  b.off_qg = o;    o += align256((size_t)L * 2 * b.kp);
+  b.off_qw = o;    o += align256((size_t)I * b.kp);
+  b.off_qw2 = o;   o += align256((size_t)I * 2 * b.kp);
+  b.total = o;
+  return b;
+}
+
+static int check_luq(const hot_config* cfg, int64_t L, int64_t O, int64_t I, const char* who) {
+  if (int e = check_cfg(cfg, who)) return e;
+  if (L <= 0 || O <= 0 || I <= 0 || O % 8 || I % 8) return fail(HOT_ERR_INVALID, "%s: L=%lld, O=%lld and I=%lld must be positive, O and I multiples of 8", who, (long long)L, (long long)O, (long long)I);
+  if (O % cfg->n_o) return fail(HOT_ERR_INVALID, "%s: O=%lld is not a multiple of n_o=%d", who, (long long)O, cfg->n_o);
+  if (cfg->gx_bits != 4 || cfg->w_bits != 4) return fail(HOT_ERR_UNSUPPORTED, "%s: the logarithmic quantiser runs at 4 bits against 4-bit weights", who);
+  if (cfg->w_scale == HOT_SCALE_ROW) return fail(HOT_ERR_UNSUPPORTED, "%s: W uses one step per tensor", who);
+  return HOT_OK;
+}
+
+size_t hot_gx_luq_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_config* cfg) {
+  if (check_luq(cfg, L, O, I, "hot_gx_luq_workspace_bytes")) return 0;
+  return luq_layout(L, O, I).total;
+}
+
+int hot_gx_luq(const void* gy, const void* w, int dtype, int64_t L, int64_t O, int64_t I, const hot_config* cfg,
+               void* gx, int out_dtype, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  const char* who = "hot_gx_luq";
+  if (int e = check_luq(cfg, L, O, I, who)) return e;
+  if (!gy || !w || !gx) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
+  if (O * I * 4 >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "%s: W exceeds the 32-bit offsets of the loader", who);
+  const LuqLayout b = luq_layout(L, O, I);
+  if (!workspace || workspace_bytes < b.total) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, b.total, workspace_bytes);
+  if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
+  hipStream_t st = (hipStream_t)hip_stream;
+  uint8_t* ws = (uint8_t*)workspace;
+  float* sg = (float*)(ws + b.off_sg);
+  float* sw = (float*)(ws + b.off_sw);
+  // W: Hadamard along O + 4-bit quantiser, codes kept one per byte, stored [I, kp]; then [16 w | w]
+  int rc = colwise_quant_impl(w, dtype, O, I, cfg->n_o, identity_rows(), cfg->n_o, cfg->w_bits, cfg->w_round, cfg->seed,
+                              HOT_STREAM_W, cfg->w_scale, ws + b.off_qw, b.kp, 0, sw, ws + b.off_colw,
+                              colwise_workspace_bytes_impl(I), st, who);
+  if (rc) return rc;
+  rc = luq_pair_impl(ws + b.off_qw, I, b.kp, ws + b.off_qw2, st);
+  if (rc) return rc;
+  rc = hq_luq_impl(gy, dtype, L, O, cfg->n_o, cfg->gx_bits, cfg->seed, ws + b.off_qg, b.kp, sg, ws + b.off_slots,
+                   STAT_SLOT_BYTES, st);
+  if (rc) return rc;
+  return gemm_i8_impl(ws + b.off_qg, 2 * b.kp, ws + b.off_qw2, 2 * b.kp, 8, L, I, 2 * b.kp, sg, 0, sw,
+                      1.0f / (float)cfg->n_o, gx, out_dtype, I, nullptr, st);
+}
+
 // ---- 3-D activations: one set of steps per sample --------------------------------------------------
 // The reference vmaps its quantisers over the batch dimension of [B, T, C] tensors
 // (utils/quant_matmul.py:33-37,102-106,118-122), applies the token-wise transform inside each sample

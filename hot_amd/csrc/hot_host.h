@@ -38,6 +38,13 @@ int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int 
 // own; scales_out then holds M entries (the step of each row's sample, the form the GEMM epilogue
 // reads), group_steps (may be null) the M / group_rows steps, and the workspace 128 bytes per sample.
 
+// Logarithmic quantiser of the row-wise transformed tensor (luq_quantizer_BWD): codes 0 / +-2^j split as
+// 16 a + b into two planes of kp bytes per row ([M, 2 kp]), one step; the workspace holds STAT_SLOT_BYTES.
+int hq_luq_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, uint64_t seed, void* codes_out,
+                int64_t kp, float* scale_out, void* workspace, size_t workspace_bytes, hipStream_t st);
+// [rows, 2 kp] = [16 w | w] from INT8-stored codes w [rows, kp] with |w| <= 8
+int luq_pair_impl(const void* qw, int64_t rows, int64_t kp, void* out, hipStream_t st);
+
 int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r,
                        int bits, int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode,
                        void* codes_out, int64_t ld_out, int store4, float* scales_out, void* workspace,

@@ -267,6 +267,100 @@ __global__ void hq_group_quant_kernel(const T* __restrict__ in, int64_t chunks_p
   }
 }
 
+// ---- logarithmic unbiased quantiser (luq_quantizer_BWD, utils/quant_matmul.py:58-77) ---------------
+// s = max(t) / 2^lev (the maximum, not the largest magnitude), lev = 2^(bits-1) - 1.  A magnitude below
+// s becomes s with probability |t| / s, else 0; a magnitude m s with 2^k <= m < 2^(k+1) becomes 2^k s
+// or 2^(k+1) s, the larger with probability m / 2^k - 1 (noise = 2^k (u2 - 1/2); 2^floor(log2((m + noise)
+// 4 / 3)), never below 2^k).  The codes are 0 or +-2^j in units of s, j up to lev + 1 (more for negative
+// elements beyond the maximum): not an INT4 / INT8 grid.  For the integer GEMM every code q is split as
+// q = 16 a + b and stored in two planes of a row, a in bytes [0, Kp) and b in bytes [Kp, 2 Kp); the other
+// operand carries 16 w in its first plane and w in its second, so one INT8 product over 2 Kp codes
+// is the exact sum of q w.  Element e draws the uniforms 2 e and 2 e + 1 of the stream.
+constexpr uint32_t LUQ_STREAM = 4;
+
+__device__ __forceinline__ int luq_code(float x, float s, float u1, float u2) {
+#pragma clang fp contract(off)
+  const float ax = fabsf(x);
+  if (!(s > 0.f) || x == 0.f || ax < s * u1) return 0;
+  const float m = (ax < s ? s : ax) / s;                       // >= 1
+  const int k = (int)((as_u(m) >> 23) & 0xFFu) - 127;          // floor(log2 m)
+  const float noise = as_f((uint32_t)(k + 127) << 23) * (u2 - 0.5f);
+  const float v = ((m + noise) * 4.0f) / 3.0f;
+  int j = (int)((as_u(v) >> 23) & 0xFFu) - 127;
+  j = j < k ? k : j;
+  j = j > 10 ? 10 : j;                                         // 16 a + b with a <= 127 holds up to 2^10
+  const int q = 1 << j;
+  return x < 0.f ? -q : q;
+}
+
+template <typename T, int N>
+__global__ void hq_posmax_kernel(const T* __restrict__ in, int64_t nchunks, float* __restrict__ slots, int nrt) {
+  __shared__ float s_red[16];
+  const int lane = threadIdx.x & 63;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  float mx = 0.f;
+  for (int64_t ch = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ch < nchunks; ch += stride) {
+    float x[EPL];
+    load_chunk<T>(in + ch * EPL, x);
+    fwht_lanes<N>(x, lane, nrt);
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) mx = fmaxf(mx, x[j]);
+  }
+  mx = wave_max(mx);
+  if (lane == 0) s_red[threadIdx.x >> 6] = mx;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    float m = s_red[0];
+    for (int i = 1; i < (int)(blockDim.x >> 6); ++i) m = fmaxf(m, s_red[i]);
+    stat_slot_update(slots, blockIdx.x, m);
+  }
+}
+
+template <typename T, int N>
+__global__ void hq_luq_kernel(const T* __restrict__ in, int64_t nchunks, int64_t nch_row, int64_t ld, int64_t kp,
+                              const float* __restrict__ slots, float inv_levels, int8_t* __restrict__ codes,
+                              float* __restrict__ scale_out, uint64_t seed, int nrt) {
+  const int lane = threadIdx.x & 63;
+  const float s = stat_slots_max(slots, lane) * inv_levels;       // a power of two: exact
+  if (blockIdx.x == 0 && threadIdx.x == 0) *scale_out = s;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t ch = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; ch < nchunks; ch += stride) {
+    float x[EPL];
+    load_chunk<T>(in + ch * EPL, x);
+    fwht_lanes<N>(x, lane, nrt);
+    float u[2 * EPL];
+    sr_uniform8((uint64_t)ch * 2, seed, LUQ_STREAM, u);          // uniforms 16 ch .. 16 ch + 15
+    sr_uniform8((uint64_t)ch * 2 + 1, seed, LUQ_STREAM, u + EPL);
+    uint32_t hi0 = 0, hi1 = 0, lo0 = 0, lo1 = 0;
+#pragma unroll
+    for (int j = 0; j < EPL; ++j) {
+      const int q = luq_code(x[j], s, u[2 * j], u[2 * j + 1]);
+      const int mag = q < 0 ? -q : q;
+      const int a = q < 0 ? -(mag >> 4) : (mag >> 4), b = q < 0 ? -(mag & 15) : (mag & 15);
+      if (j < 4) { hi0 |= (uint32_t)(a & 0xFF) << (8 * j); lo0 |= (uint32_t)(b & 0xFF) << (8 * j); }
+      else { hi1 |= (uint32_t)(a & 0xFF) << (8 * (j - 4)); lo1 |= (uint32_t)(b & 0xFF) << (8 * (j - 4)); }
+    }
+    const int64_t row = ch / nch_row, col = ch - row * nch_row;
+    int8_t* o = codes + row * ld + col * EPL;
+    *reinterpret_cast<uint2*>(o) = make_uint2(hi0, hi1);
+    *reinterpret_cast<uint2*>(o + kp) = make_uint2(lo0, lo1);
+  }
+}
+
+// second operand of a product with two-plane LUQ codes: [16 w | w] from INT8-stored codes w in [-8, 7]
+__global__ void luq_pair_kernel(const int8_t* __restrict__ qw, int64_t rows, int64_t kp, int8_t* __restrict__ out) {
+  const int64_t nq = kp / 16;
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= rows * nq) return;
+  const int64_t row = i / nq, c = (i - row * nq) * 16;
+  const uint4 v = *reinterpret_cast<const uint4*>(qw + row * kp + c);
+  uint4 h;
+  h.x = (v.x << 4) & 0xF0F0F0F0u; h.y = (v.y << 4) & 0xF0F0F0F0u;
+  h.z = (v.z << 4) & 0xF0F0F0F0u; h.w = (v.w << 4) & 0xF0F0F0F0u;
+  *reinterpret_cast<uint4*>(out + row * 2 * kp + c) = h;
+  *reinterpret_cast<uint4*>(out + row * 2 * kp + kp + c) = v;
+}
+
 // zero the bytes [row_bytes, ld) of every row (K padding for the GEMM)
 __global__ void zero_pad_kernel(int8_t* codes, int64_t M, int64_t row_bytes, int64_t ld) {
   const int64_t padw = (ld - row_bytes) / 4;
@@ -388,6 +482,60 @@ static int dispatch_n(int n, int bits, int rounding, int scale_mode, const void*
     case 32: return dispatch_bits<T, 32>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n, group_rows, group_steps);
     default: return dispatch_bits<T, 64>(bits, rounding, scale_mode, in, M, K, codes, ld, scales, absmax, seed, stream_id, st, absmax_ready, n, group_rows, group_steps);
   }
+}
+
+template <typename T, int N>
+static int launch_luq(const void* in, int64_t M, int64_t K, int bits, void* codes, int64_t ld, int64_t kp, float* scale,
+                      float* slots, uint64_t seed, hipStream_t st, int nrt) {
+  const int64_t nch = M * K / EPL;
+  int64_t blocks = (nch + 255) / 256;
+  if (blocks > 256 * 16) blocks = 256 * 16;
+  if (blocks < 1) blocks = 1;
+  const int lev = (1 << (bits - 1)) - 1;
+  hipLaunchKernelGGL(fill_u32_kernel, dim3(2), dim3(256), 0, st, (uint32_t*)slots, 0u, (int)(STAT_SLOT_BYTES / 4));
+  hipLaunchKernelGGL((hq_posmax_kernel<T, N>), dim3((unsigned)blocks), dim3(256), 0, st, (const T*)in, nch, slots, nrt);
+  hipLaunchKernelGGL((hq_luq_kernel<T, N>), dim3((unsigned)blocks), dim3(256), 0, st, (const T*)in, nch, K / EPL, ld, kp,
+                     slots, 1.0f / (float)(1 << lev), (int8_t*)codes, scale, seed, nrt);
+  return check_launch("hq_luq_kernel");
+}
+
+template <typename T>
+static int dispatch_luq(int n, const void* in, int64_t M, int64_t K, int bits, void* codes, int64_t ld, int64_t kp,
+                        float* scale, float* slots, uint64_t seed, hipStream_t st) {
+  switch (n) {
+    case 1: case 2: case 4: case 8: return launch_luq<T, 8>(in, M, K, bits, codes, ld, kp, scale, slots, seed, st, n);
+    case 16: return launch_luq<T, 16>(in, M, K, bits, codes, ld, kp, scale, slots, seed, st, n);
+    case 32: return launch_luq<T, 32>(in, M, K, bits, codes, ld, kp, scale, slots, seed, st, n);
+    default: return launch_luq<T, 64>(in, M, K, bits, codes, ld, kp, scale, slots, seed, st, n);
+  }
+}
+
+int hq_luq_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, uint64_t seed, void* codes_out,
+                int64_t kp, float* scale_out, void* workspace, size_t workspace_bytes, hipStream_t st) {
+  const char* who = "hq_luq";
+  if (!in || !codes_out || !scale_out) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
+  if (M <= 0 || K <= 0 || K % 8) return fail(HOT_ERR_INVALID, "%s: bad shape M=%lld K=%lld (K a multiple of 8)", who, (long long)M, (long long)K);
+  if (n < 1 || n > 64 || (n & (n - 1)) || K % n) return fail(HOT_ERR_UNSUPPORTED, "%s: Hadamard block %d (a power of two up to 64 dividing K)", who, n);
+  if (bits != 4) return fail(HOT_ERR_UNSUPPORTED, "%s: bits=%d (the two-plane code layout is sized for 4)", who, bits);
+  if (kp < K || (kp & 15)) return fail(HOT_ERR_INVALID, "%s: plane width %lld must be a multiple of 16 and >= K", who, (long long)kp);
+  if (!workspace || workspace_bytes < STAT_SLOT_BYTES) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed", who, STAT_SLOT_BYTES);
+  if (((uintptr_t)in & 15) || ((uintptr_t)codes_out & 15)) return fail(HOT_ERR_INVALID, "%s: pointers must be 16-byte aligned", who);
+  // bytes [K, 2 kp) of every row first: the K padding of both planes (the second plane is written afterwards)
+  zero_pad_impl(codes_out, M, K, 2 * kp, st);
+  float* slots = (float*)workspace;
+  switch (dtype) {
+    case HOT_F32: return dispatch_luq<float>(n, in, M, K, bits, codes_out, 2 * kp, kp, scale_out, slots, seed, st);
+    case HOT_BF16: return dispatch_luq<bf16_t>(n, in, M, K, bits, codes_out, 2 * kp, kp, scale_out, slots, seed, st);
+    case HOT_F16: return dispatch_luq<f16_t>(n, in, M, K, bits, codes_out, 2 * kp, kp, scale_out, slots, seed, st);
+    default: return fail(HOT_ERR_INVALID, "%s: bad dtype %d", who, dtype);
+  }
+}
+
+int luq_pair_impl(const void* qw, int64_t rows, int64_t kp, void* out, hipStream_t st) {
+  if (!qw || !out || rows <= 0 || kp <= 0 || (kp & 15)) return fail(HOT_ERR_INVALID, "luq_pair: bad arguments");
+  const int64_t n = rows * (kp / 16);
+  hipLaunchKernelGGL(luq_pair_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, (const int8_t*)qw, rows, kp, (int8_t*)out);
+  return check_launch("luq_pair_kernel");
 }
 
 int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, int rounding,

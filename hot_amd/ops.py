@@ -374,6 +374,27 @@ def gx_lowrank(gy: torch.Tensor, w: torch.Tensor, opt: HotOptions, out_dtype=Non
     return gx
 
 
+def gx_luq(gy: torch.Tensor, w: torch.Tensor, opt: HotOptions, out_dtype=None) -> torch.Tensor:
+    """g_x [L, I] with the logarithmic quantiser on g_y (hot_gx_luq; quantBWDGogi = "luq"): opt.n_o, the 4-bit
+    widths, opt.w_round / w_scale for W and opt.seed are read."""
+    _need_gpu_2d(gy, "Go")
+    _need_gpu_2d(w, "Wt")
+    L, O = gy.shape
+    if w.shape[0] != O or w.dtype != gy.dtype:
+        raise RuntimeError("W must be [O, I] with O = Go.shape[1], in the dtype of Go")
+    I = w.shape[1]
+    out_dtype = out_dtype or gy.dtype
+    cfg = opt.to_c()
+    need = _lib.lib().hot_gx_luq_workspace_bytes(L, O, I, C.byref(cfg))
+    if need == 0:
+        raise HotError("bad configuration: %s" % _lib.lib().hot_last_error().decode())
+    ws = _ws(need, gy.device)
+    gx = torch.empty((L, I), dtype=out_dtype, device=gy.device)
+    _lib.check(_lib.lib().hot_gx_luq(gy.data_ptr(), w.data_ptr(), _dt(gy), L, O, I, C.byref(cfg), gx.data_ptr(),
+                                     _DTYPES[out_dtype], ws.data_ptr(), ws.numel(), _stream()))
+    return gx
+
+
 def measure_ceilings(device=None):
     """(copy GB/s, INT8 MFMA TOP/s) of this box from the library's two plain ceiling kernels."""
     device = device or torch.device("cuda", torch.cuda.current_device())

@@ -41,9 +41,20 @@ _QUANT_SCHEMES = {
     "stoch_quantizer": (ops.ROUND_STOCH, ops.SCALE_TENSOR),
     "norm_quantizer": (ops.ROUND_STOCH, ops.SCALE_ROW),
     "sawb_quantizer": (ops.ROUND_NEAREST, ops.SCALE_SAWB),
+    # the logarithmic quantiser has an entry point of its own for the g_x product (ops.gx_luq, see
+    # gx_uses_luq); the pair below only fills the option fields that entry point does not read
+    "luq_quantizer": (ops.ROUND_STOCH, ops.SCALE_TENSOR),
 }
 _FLAG_SCHEMES = {"int": "int_quantizer", "stoch": "stoch_quantizer", "nq": "norm_quantizer",
-                 "sawb": "sawb_quantizer"}
+                 "sawb": "sawb_quantizer", "luq": "luq_quantizer"}
+
+
+def gx_uses_luq(layer_name: str = " ") -> bool:
+    """True when the g_y quantiser of the g_x product is luq_quantizer (args.quantBWDGogi == "luq", or the
+    layer's entry of args.layer_quant_dict under quantAuto; utils/quant_matmul.py:244-253)."""
+    if args.quantAuto and len(args.layer_quant_dict) > 0:
+        return args.layer_quant_dict.get(layer_name + "_gx") == "luq_quantizer"
+    return args.quantBWDGogi == "luq"
 
 
 def _scheme(flag: str, what: str, allowed) -> Tuple[int, int]:
@@ -140,8 +151,10 @@ def _options_uncached(tokens: int, layer_name: str, out_features: int) -> ops.Ho
         gx_round, gx_scale = _QUANT_SCHEMES[args.layer_quant_dict[layer_name + "_gx"]]
         gw_round, gw_scale = _QUANT_SCHEMES[args.layer_quant_dict[layer_name + "_gw"]]
         gw_bits = args.GogiQuantBit
+        if args.layer_quant_dict[layer_name + "_gw"] == "luq_quantizer":
+            raise NotImplementedError("the logarithmic quantiser runs on the g_x product only (its codes are no INT8 grid)")
     else:
-        gx_round, gx_scale = _scheme(args.quantBWDGogi, "GradHo", ("int", "stoch", "nq"))
+        gx_round, gx_scale = _scheme(args.quantBWDGogi, "GradHo", ("int", "stoch", "nq", "luq"))
         gw_round, gw_scale = _scheme(args.quantBWDGogw, "GradHb", ("int", "stoch", "nq"))
     w_round, w_scale = _scheme(args.quantBWDWgt, "Weight", ("int", "stoch", "sawb"))
     act_round, act_scale = _scheme(args.quantBWDAct, "Activation", ("int", "stoch", "sawb"))
@@ -276,18 +289,25 @@ class FLinearQ(Function):
         wc = _pad8(_pad8(w).t()).t().contiguous() if (O % 8 or I % 8) else w.contiguous()   # [O8, I8]
         if go.dtype != wc.dtype:
             go = go.to(wc.dtype)
-        if args.transform_scheme in LOWRANK_GX_SCHEMES:
-            # g_x through the projection along the tokens and its expansion; g_W as in "gih_gwlr"
-            # ("low_rank") or "hadamard" ("gilr_gwh"): the token-wise kernel on g_y, then the INT8 product
+        luq = gx_uses_luq(ctx.name)
+        if args.transform_scheme in LOWRANK_GX_SCHEMES or luq:
+            # g_x by an entry point of its own -- the projection along the tokens and its expansion
+            # ("low_rank", "gilr_gwh"), or the logarithmic quantiser on g_y --, g_W as in "gih_gwlr" /
+            # "hadamard": the token-wise kernel on g_y, then the INT8 product
+            what = "quantBWDGogi luq" if luq else "transform scheme %r" % args.transform_scheme
             if go.dim() == 3 and args.batched_mode == "per_sample":
-                raise NotImplementedError("transform scheme %r takes 2-D activations or batched_mode \"flatten\""
-                                          % args.transform_scheme)
-            if opt.gx_scale != ops.SCALE_TENSOR:
+                raise NotImplementedError("%s takes 2-D activations or batched_mode \"flatten\"" % what)
+            if luq and args.transform_scheme in LOWRANK_GX_SCHEMES:
+                raise NotImplementedError("quantBWDGogi luq runs with the schemes gih_gwlr and hadamard")
+            if not luq and opt.gx_scale != ops.SCALE_TENSOR:
                 raise NotImplementedError("transform scheme %r: the projected g_y takes one step for the tensor "
                                           "(quantBWDGogi int or stoch)" % args.transform_scheme)
             go2 = _pad8(go.reshape(-1, go.shape[-1]))
-            n_gx, rows_gx = gx_token_rule(go2.shape[0])
-            gx = ops.gx_lowrank(go2, wc, replace(opt, hla_n=int(n_gx), hla_rows=tuple(int(v) for v in rows_gx)))
+            if luq:
+                gx = ops.gx_luq(go2, wc, opt)
+            else:
+                n_gx, rows_gx = gx_token_rule(go2.shape[0])
+                gx = ops.gx_lowrank(go2, wc, replace(opt, hla_n=int(n_gx), hla_rows=tuple(int(v) for v in rows_gx)))
             qgp, sgp, lp = ops.hla_tokenwise(go2, opt.hla_n, opt.hla_rows, bits=opt.gw_bits,
                                              rounding="stoch" if opt.gw_round == ops.ROUND_STOCH else "nearest",
                                              scale="row" if opt.gw_scale == ops.SCALE_ROW else "tensor",

@@ -267,6 +267,21 @@ HOT_API int hot_gx_lowrank(const void* gy, const void* w, int dtype, int64_t L, 
                    size_t workspace_bytes, void* hip_stream);
 
 /*
+ * g_x with the logarithmic unbiased quantiser on g_y (quantBWDGogi = "luq",
+ * utils/quant_matmul.py:58-83,252-253): g_x = (luq(g_y blkdiag(H)) . q(blkdiag(H) W)) s_g s_w / n_o.
+ * luq_quantizer_BWD: s = max(t) / 2^lev, lev = 2^(bits-1) - 1; magnitudes below s become s with
+ * probability |t| / s, else 0; others 2^k s or 2^(k+1) s with the probabilities that keep the
+ * expectation.  gx_bits = w_bits = 4.  The codes (0, +-2^j) are no uniform grid: they go through
+ * the INT8 product as two planes (q = 16 a + b) against [16 w | w].  Element e of the row-major
+ * transformed g_y draws the uniforms 2 e and 2 e + 1 of Philox stream 4 under cfg->seed
+ * (cfg->gx_round and gx_scale are not read).
+ */
+HOT_API size_t hot_gx_luq_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_config* cfg);
+HOT_API int hot_gx_luq(const void* gy, const void* w, int dtype, int64_t L, int64_t O, int64_t I,
+               const hot_config* cfg, void* gx, int out_dtype, void* workspace,
+               size_t workspace_bytes, void* hip_stream);
+
+/*
  * Number of K ranges into which the GEMMs inside hot_linear_backward cut a product of
  * M x N outputs over K codes of `bits` bits (1 = one kernel; more = a kernel per range
  * writing int32 partial tiles to the workspace, then a reduce kernel).  Products with

@@ -502,6 +502,58 @@ def gx_lowrank(g_y: np.ndarray, w: np.ndarray, cfg: HotConfig) -> BackwardTrace:
     return tr
 
 
+STREAM_LUQ = 4  # the two uniforms per element of the logarithmic quantiser
+
+
+def luq_quant(t: np.ndarray, bits: int, seed: int, stream: int = STREAM_LUQ, index: Optional[np.ndarray] = None):
+    """luq_quantizer_BWD (utils/quant_matmul.py:58-77): logarithmic unbiased quantisation.  With
+    lev = 2^(bits-1) - 1 and s = max(t) / 2^lev (the maximum, not the largest magnitude, :60-61):
+      * magnitudes below s become s with probability |t| / s, else 0 (:62-67: u1 ~ U[0, 1));
+      * every other magnitude m s, 2^k <= m < 2^(k+1), becomes 2^k s or 2^(k+1) s, the larger with
+        probability m / 2^k - 1 (:71-74: noise = 2^k (u2 - 1/2), 2^floor(log2((m + noise) 4 / 3)),
+        never below 2^k), so that the expectation is t;
+    Returns (codes in units of s: 0 or +-2^j as int32, s fp32 [1]).  floor(log2(.)) is taken from the
+    binary exponent (torch's float log2 can round an argument just below a power of two up to it).
+    A tensor without a positive element has s <= 0 in the reference; here all codes are 0 then.
+    Element e draws u1, u2 = the uniforms 2 e and 2 e + 1 of `stream`."""
+    t = np.asarray(t, dtype=F32)
+    lev = 2 ** (bits - 1) - 1
+    mx = max(float(t.max()), 0.0) if t.size else 0.0
+    s = F32(F32(mx) / F32(2.0 ** lev))
+    idx = np.arange(t.size, dtype=np.int64).reshape(t.shape) if index is None else np.asarray(index, dtype=np.int64)
+    u1 = sr_uniform(2 * idx, seed, stream)
+    u2 = sr_uniform(2 * idx + 1, seed, stream)
+    if s <= 0:
+        return np.zeros(t.shape, dtype=np.int32), np.array([s], dtype=F32)
+    ax = np.abs(t)
+    zero = (ax < (s * u1).astype(F32)) | (t == 0)
+    m = (np.where(ax < s, s, ax).astype(F32) / s).astype(F32)                   # >= 1
+    k = np.frexp(m)[1].astype(np.int64) - 1                                      # floor(log2 m)
+    noise = (np.ldexp(F32(1.0), k).astype(F32) * (u2 - F32(0.5)).astype(F32)).astype(F32)
+    v = (((m + noise).astype(F32) * F32(4.0)).astype(F32) / F32(3.0)).astype(F32)
+    j = np.maximum(np.frexp(v)[1].astype(np.int64) - 1, k)
+    q = (np.sign(t).astype(np.int64) * (np.int64(1) << j)).astype(np.int64)
+    q[zero] = 0
+    return q.astype(np.int32), np.array([s], dtype=F32)
+
+
+def gx_luq(g_y: np.ndarray, w: np.ndarray, cfg: HotConfig) -> BackwardTrace:
+    """grad_input with quantBWDGogi = "luq" (utils/quant_matmul.py:238, 252-253, 270, 276-285, 288-290, 343):
+    g_y blkdiag(H) through the logarithmic quantiser (cfg.gx_bits, one step for the tensor), blkdiag(H) W
+    through cfg's weight quantiser, their integer product, the two steps, / n_o."""
+    g_y = np.asarray(g_y, dtype=F32)
+    w = np.asarray(w, dtype=F32)
+    tr = BackwardTrace()
+    G = fwht_blocks_last(g_y, cfg.n_o)
+    tr.qG, tr.sG = luq_quant(G, cfg.gx_bits, cfg.seed)
+    Wh = fwht_blocks_first(w, cfg.n_o)
+    tr.qW, tr.sW = quant(Wh, cfg.w_bits, cfg.w_scale, cfg.w_round, cfg.seed, STREAM_W,
+                         index=colwise_rng_index(Wh.shape[1], Wh.shape[0] // cfg.n_o, np.arange(cfg.n_o)).T)
+    tr.acc_x = int_gemm_nt(tr.qG, tr.qW.T)
+    tr.g_x = (((tr.acc_x.astype(F32) * tr.sG[0]).astype(F32) * tr.sW[0]).astype(F32) / F32(cfg.n_o)).astype(F32)
+    return tr
+
+
 def stoch_round_mantissa(x: np.ndarray) -> np.ndarray:
     """The reference CUDA op's pseudo-stochastic rounding
     (HLQ_backward_kernel.cu:19-36), kept only to characterise its bias; the

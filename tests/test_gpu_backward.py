@@ -845,6 +845,48 @@ def test_hq_linear_lowrank_gx_schemes(gpu, fresh_args, scheme, L):
     assert rel(lin.weight.grad.cpu().numpy(), gw_ref.numpy()) < REL_TOL
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L,O,I,variant", [
+    (448, 192, 160, dict(seed=1)),
+    (1000, 208, 72, dict(seed=2, w_scale=orc.SCALE_SAWB)),          # K padded from 208 to 256 in both planes
+    (197, 80, 264, dict(seed=3, w_round=orc.ROUND_STOCH)),
+    (4096, 768, 512, dict(seed=4)),
+])
+def test_gx_luq_matches_oracle(gpu, dtype, L, O, I, variant):
+    """g_x with the logarithmic quantiser on g_y (hot_gx_luq): codes 0 / +-2^j as two INT8 planes against
+    [16 w | w], bit for bit the oracle (same uniforms, same float operations)."""
+    from hot_amd import ops
+    x, w, gy = make_case(L, O, I, seed=L + O, dtype=dtype)
+    ocfg = orc.HotConfig(**variant)
+    opt = ops.HotOptions(n_o=ocfg.n_o, w_round=ocfg.w_round, w_scale=ocfg.w_scale, seed=ocfg.seed)
+    gx = ops.gx_luq(gy.to(gpu), w.to(gpu), opt)
+    tr = orc.gx_luq(gy.float().numpy(), w.float().numpy(), ocfg)
+    assert int(np.abs(tr.qG).max()) >= 128                           # the top level is in use
+    assert torch.equal(gx.cpu(), torch.from_numpy(tr.g_x).to(dtype))
+
+
+def test_hq_linear_with_luq_on_the_gx_path(gpu, fresh_args):
+    """quantBWDGogi = "luq" through HQ_Linear: g_x from hot_gx_luq, g_W as with any other setting."""
+    from hot_amd.quant_matmul import HQ_Linear
+    L, I, O = 448, 96, 128
+    fresh_args.quantBWDGogi = "luq"
+    torch.manual_seed(3)
+    lin = HQ_Linear(I, O, bias=False).to(gpu)
+    x = torch.randn(L, I, device=gpu, requires_grad=True)
+    gy = torch.randn(L, O, device=gpu) * 1e-3
+    step = fresh_args.sr_step
+    lin(x).backward(gy)
+    xn, gyn, wn = x.detach().cpu().numpy(), gy.cpu().numpy(), lin.weight.detach().cpu().numpy()
+    seed = (int(fresh_args.sr_seed) << 20) + step
+    ocfg, _ = both_configs(L, seed=seed)
+    xq_ref, sx_ref = orc.abc_forward(xn, ocfg)
+    assert np.array_equal(x.grad.cpu().numpy(), orc.gx_luq(gyn, wn, ocfg).g_x)
+    assert np.array_equal(lin.weight.grad.cpu().numpy(), orc.linear_backward(gyn, wn, xq_ref, sx_ref, ocfg).g_w)
+    fresh_args.batched_mode = "per_sample"
+    with pytest.raises(NotImplementedError):
+        lin(torch.randn(2, 64, I, device=gpu, requires_grad=True)).sum().backward()
+
+
 @pytest.mark.parametrize("variant", [dict(), dict(gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW,
                                                  gw_round=orc.ROUND_STOCH, gw_scale=orc.SCALE_ROW, seed=3)])
 def test_backward_fp16(gpu, variant):

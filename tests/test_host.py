@@ -108,10 +108,15 @@ def test_options_follow_args(fresh_args):
     o = options_for(8192)
     assert (o.hla_n, o.hla_r) == (16, 8)
     a.hla_rule = "python"
-    a.quantBWDGogi = "luq"
+    a.quantBWDGogi = "luq"                          # an entry point of its own for the g_x product
+    from hot_amd.quant_matmul import gx_uses_luq
+    assert gx_uses_luq() and options_for(64).gx_bits == 4
+    a.quantBWDGogw = "luq"                          # not for the g_W product
     with pytest.raises(NotImplementedError):
         options_for(64)
+    a.quantBWDGogw = "int"
     a.quantBWDGogi = "int"
+    assert not gx_uses_luq()
     a.transform_scheme = "hadamard"                 # block Hadamard along the tokens, nothing dropped
     o = options_for(12608)
     assert (o.hla_n, o.hla_r, o.hla_rows) == (16, 16, tuple(range(16)))

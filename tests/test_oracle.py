@@ -473,3 +473,57 @@ def test_gx_lowrank_against_the_port_and_the_plain_product():
     proj = orc.hla_expand(orc.fwht_blocks_first(exact.astype(np.float32), n, np.asarray(rows)), n, rows) / n
     hi = orc.HotConfig(hla_n=n, hla_rows=tuple(int(v) for v in rows), gx_bits=8, w_bits=8)
     assert np.linalg.norm(orc.gx_lowrank(gy.numpy(), w.numpy(), hi).g_x - proj) / np.linalg.norm(proj) < 0.02
+
+
+# ------------------------------------------------------------------ logarithmic quantiser
+
+def test_luq_levels_step_and_expectation():
+    """luq_quantizer_BWD (utils/quant_matmul.py:58-77): the step is max / 2^7, codes are 0 or +-2^j, the
+    maximum maps to 2^7 exactly, a value between two levels lands on one of the two, and the mean over many
+    seeds converges on the value: both for the underflow region (|t| < s: s with probability |t| / s) and for
+    the logarithmic rounding (the larger level with probability m / 2^k - 1)."""
+    rng = np.random.default_rng(1)
+    t = (rng.standard_normal((48, 40)) * 2e-3).astype(np.float32)
+    t[0, 0] = np.float32(9e-3)                               # the maximum
+    t[0, 1:6] = np.float32(9e-3) * np.array([2.0 ** -9, 2.0 ** -8, 3 * 2.0 ** -7, 0.75, -0.6], dtype=np.float32)
+    q, s = orc.luq_quant(t, 4, seed=0)
+    assert s[0] == np.float32(9e-3) / np.float32(128) and q[0, 0] == 128
+    mags = np.unique(np.abs(q))
+    assert set(mags.tolist()) <= {0} | {2 ** j for j in range(11)}
+    m = np.abs(t) / s[0]
+    inside = (m >= 1) & (np.abs(t) <= t.max())
+    k = np.floor(np.log2(m[inside])).astype(int)
+    assert np.all((np.abs(q[inside]) == 2 ** k) | (np.abs(q[inside]) == 2 ** (k + 1)))
+    assert np.array_equal(np.sign(q[q != 0]), np.sign(t[q != 0]))
+    small = m < 1
+    assert set(np.abs(q[small]).tolist()) <= {0, 1}
+    N = 800
+    acc = np.zeros(t.shape)
+    for seed in range(N):
+        acc += orc.luq_quant(t, 4, seed=seed)[0]
+    mean = acc / N * s[0]
+    ok = np.abs(t) <= t.max()
+    # standard error of a two-point variable with gap <= 2^k s <= |t|: <= |t| / (2 sqrt N); five sigma
+    assert np.all(np.abs(mean - t)[ok] <= 5 * np.maximum(np.abs(t), s[0])[ok] / (2 * np.sqrt(N)) + 1e-12)
+    # exact levels stay where they are; zero stays zero; a tensor without a positive element gives zeros
+    lv = (np.array([[1, 2, 4, 64, 128, 0, -8]], dtype=np.float32) * np.float32(2.0 ** -10))
+    q2, s2 = orc.luq_quant(lv, 4, seed=3)
+    assert s2[0] == np.float32(2.0 ** -10) and np.array_equal(q2, [[1, 2, 4, 64, 128, 0, -8]])
+    q3, s3 = orc.luq_quant(-np.abs(t), 4, seed=0)
+    assert not q3.any() and s3[0] <= 0
+
+
+def test_gx_luq_close_to_the_plain_product():
+    rng = np.random.default_rng(2)
+    L, O, I = 256, 64, 48
+    gy = (rng.standard_normal((L, O)) * 1e-3).astype(np.float32)
+    w = (rng.standard_normal((O, I)) * 0.1).astype(np.float32)
+    exact = gy @ w
+    acc = np.zeros_like(exact, dtype=np.float64)
+    for seed in range(40):
+        acc += orc.gx_luq(gy, w, orc.HotConfig(seed=seed)).g_x
+    # unbiased in g_y; what remains is the 4-bit weight quantiser
+    wq, sw = orc.quant(orc.fwht_blocks_first(w, 16), 4)
+    w_hat = orc.fwht_blocks_first((wq * sw[0]).astype(np.float32), 16) / 16
+    target = gy @ w_hat
+    assert np.linalg.norm(acc / 40 - target) / np.linalg.norm(target) < 0.08
