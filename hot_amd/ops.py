@@ -7,6 +7,7 @@ all arithmetic happens in libhot_gfx950.so.
 from __future__ import annotations
 
 import ctypes as C
+import functools
 from dataclasses import dataclass, field, replace
 from typing import Optional, Sequence, Tuple
 
@@ -48,6 +49,7 @@ def _ws(nbytes: int, device) -> torch.Tensor:
     return torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
 
 
+@functools.lru_cache(maxsize=4096)
 def kpad(k: int) -> int:
     return int(_lib.lib().hot_kpad(int(k)))
 
@@ -268,9 +270,13 @@ def linear_backward(gy: torch.Tensor, w: torch.Tensor, xq: torch.Tensor, sx: tor
     lp = opt.lprime(L)
     if tuple(xq.shape) != (I, kpad(lp)) or xq.dtype != torch.int8:
         raise RuntimeError("xq must be the int8 [I, kpad(L')] buffer written by abc_forward")
-    need = _lib.lib().hot_backward_workspace_bytes(L, O, I, C.byref(cfg))
-    if need == 0:
-        raise HotError("bad configuration: %s" % _lib.lib().hot_last_error().decode())
+    sizes = opt.__dict__.setdefault("_ws_bytes", {})      # per options object: the query is a pure function of these
+    need = sizes.get((L, O, I))
+    if need is None:
+        need = _lib.lib().hot_backward_workspace_bytes(L, O, I, C.byref(cfg))
+        if need == 0:
+            raise HotError("bad configuration: %s" % _lib.lib().hot_last_error().decode())
+        sizes[(L, O, I)] = need
     if workspace is None or workspace.numel() < need:
         workspace = _ws(need, gy.device)
     gx = torch.empty((L, I), dtype=out_dtype, device=gy.device)
