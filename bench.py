@@ -59,7 +59,7 @@ def _events(fn, iters, warm):
 
 
 def make_layer(L, O, I, dtype, dev, nsets, seed=0):
-    """Synthetic inputs of configuration 2: x ~ N(0,1); g_y ~ N(0, 1e-3) with
+    """Synthetic inputs of the GPU benchmark workloads: x ~ N(0,1); g_y ~ N(0, 1e-3) with
     1 % of the entries x50; W uniform(+-1/sqrt(I)) (kaiming-uniform)."""
     import torch
     g = torch.Generator(device=dev).manual_seed(seed)

@@ -191,7 +191,7 @@ def test_bf16_inputs_against_the_reference_bf16_evaluation(gpu):
 
 
 def test_vit_fc1_full_size(gpu):
-    """BASELINE configuration 1 at full size (L = 12608, O = 3072, I = 768):
+    """The headline workload (ViT-B fc1) at full size (L = 12608, O = 3072, I = 768):
     bit-exact against the canonical oracle, 1e-3 against the fake-quant port."""
     L, O, I = 12608, 3072, 768
     x, w, gy = fq.config1_inputs(L, O, I, seed=0)
