@@ -21,6 +21,7 @@ Prints ONE JSON line.  Besides the contract fields it carries
   kernels       per-kernel microseconds and achieved rates for this layer
   layers        the same step at every ViT-B and Llama-7B layer shape, bf16 and fp32
   llama_gate_up per-kernel pass at the Llama-7B gate/up shape
+  llama_gate_up_python_rule  the same layer with the reference's own low-rank rule (n = 8192, r = 2080)
   hq_rowwise_sweep  the row-wise quantise kernel alone over the kernel-level sweep (launches replayed
                 from a HIP graph, so no host time is in the figures)
   quantiser_grid the step over bits x rounding x step granularity x low-rank setting
@@ -561,7 +562,20 @@ def main():
                                 "hla": "n=16 r=8", "int8_tops": round((2.0 * Ll * Ol * Il + 2.0 * Ol * Il * (Ll // 2)) / lsec / 1e12, 1),
                                 # kernels launched one after the other: [us, fraction of the 8 TB/s or 5 POP/s peak]
                                 "kernels_serial": {r["key"]: [r["us"], r["frac"]] for r in ltable}}
-        del lw, lsets, lbufs, lws
+        # the same layer at the reference's own low-rank rule for 8192 tokens (utils/hadamard_matmul.py:209-226:
+        # one block of n = 8192, r = 2080 kept sequencies; the two-level token-wise path)
+        try:
+            rn, rrow = hla_rows(Ll)
+            ropt = ops.HotOptions(n_o=16, hla_n=int(rn), hla_rows=tuple(int(v) for v in rrow))
+            del lbufs, lws
+            rsec, rbufs, rws = step_time(lw, lsets, ropt, max(5, a.steps // 5), max(2, a.warmup // 5))
+            out["llama_gate_up_python_rule"] = {"us_per_layer": round(rsec * 1e6, 1), "L": Ll, "O": Ol, "I": Il,
+                                                "hla": "n=%d r=%d" % (ropt.hla_n, ropt.hla_r),
+                                                "ratio_to_paper_rule": round(rsec / lsec, 3)}
+            del rbufs, rws
+        except Exception as e:              # an extra: never costs the headline line
+            out["llama_gate_up_python_rule"] = {"error": repr(e)[:200]}
+        del lw, lsets
     if not a.no_extras and not a.table_only:
         for key, fn in (("layers", lambda: layer_table(dev)), ("measure_py", lambda: measure_py(dev))):
             try:

@@ -224,12 +224,36 @@ def _launch_stream(side: Optional["torch.cuda.Stream"]) -> int:
     return _stream() if side is None else side.cuda_stream
 
 
-def _join(side: Optional["torch.cuda.Stream"]) -> None:
-    # the current stream waits for what `side` was given: enqueued before the call returns (and so
-    # before its workspace goes back to the allocator), which orders every later use of the outputs
-    # and of the workspace's memory on the current stream behind the kernels
+class _on_stream:
+    """Allocation context of a call whose kernels run on `side`: the outputs and the workspace are
+    taken from the allocator UNDER that stream, so that they come from the side stream's own pool.  A
+    block the current stream has just released (an operand copy of the GEMM that may still be running
+    there) can then never be handed out and overwritten by the side stream's kernels."""
+
+    def __init__(self, side):
+        self.ctx = torch.cuda.stream(side) if side is not None else None
+
+    def __enter__(self):
+        if self.ctx is not None:
+            self.ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self.ctx is not None:
+            self.ctx.__exit__(*exc)
+        return False
+
+
+def _join(side: Optional["torch.cuda.Stream"], *outputs: torch.Tensor) -> None:
+    # the current stream waits for what `side` was given: enqueued before the call returns, which
+    # orders every later use of the outputs on the current stream behind the kernels.  The outputs
+    # belong to the side stream's pool; the allocator is told that the current stream uses them too.
+    # (The workspace is released to the side stream's pool, whose next user is ordered behind the
+    # kernels by that stream itself.)
     if side is not None:
-        torch.cuda.current_stream().wait_stream(side)
+        cur = torch.cuda.current_stream()
+        cur.wait_stream(side)
+        for t in outputs:
+            t.record_stream(cur)
 
 
 def abc_forward(x: torch.Tensor, opt: HotOptions, side: Optional["torch.cuda.Stream"] = None):
@@ -239,14 +263,15 @@ def abc_forward(x: torch.Tensor, opt: HotOptions, side: Optional["torch.cuda.Str
     _need_gpu_2d(x, "X")
     L, I = x.shape
     cfg = opt.to_c()
-    xq = torch.empty((I, kpad(opt.lprime(L))), dtype=torch.int8, device=x.device)
-    sx = torch.empty((1,), dtype=torch.float32, device=x.device)
-    ws = _ws(_lib.lib().hot_abc_workspace_bytes(L, I, C.byref(cfg)), x.device)
+    with _on_stream(side):
+        xq = torch.empty((I, kpad(opt.lprime(L))), dtype=torch.int8, device=x.device)
+        sx = torch.empty((1,), dtype=torch.float32, device=x.device)
+        ws = _ws(_lib.lib().hot_abc_workspace_bytes(L, I, C.byref(cfg)), x.device)
     try:
         _lib.check(_lib.lib().hot_abc_forward(x.data_ptr(), _dt(x), L, I, C.byref(cfg), xq.data_ptr(), sx.data_ptr(),
                                               ws.data_ptr(), ws.numel(), _launch_stream(side)))
     finally:
-        _join(side)
+        _join(side, xq, sx)
     return xq, sx
 
 
@@ -319,14 +344,15 @@ def abc_forward_batched(x: torch.Tensor, opt: HotOptions, side: Optional["torch.
     B, T, I = x.shape
     cfg = opt.to_c()
     kg = kpad_group(T, opt)
-    xq = torch.empty((I, B * kg), dtype=torch.int8, device=x.device)
-    sx = torch.empty((B,), dtype=torch.float32, device=x.device)
-    ws = _ws(_lib.lib().hot_abc_batched_workspace_bytes(B, T, I, C.byref(cfg)), x.device)
+    with _on_stream(side):
+        xq = torch.empty((I, B * kg), dtype=torch.int8, device=x.device)
+        sx = torch.empty((B,), dtype=torch.float32, device=x.device)
+        ws = _ws(_lib.lib().hot_abc_batched_workspace_bytes(B, T, I, C.byref(cfg)), x.device)
     try:
         _lib.check(_lib.lib().hot_abc_forward_batched(x.data_ptr(), _dt(x), B, T, I, C.byref(cfg), xq.data_ptr(),
                                                       sx.data_ptr(), ws.data_ptr(), ws.numel(), _launch_stream(side)))
     finally:
-        _join(side)
+        _join(side, xq, sx)
     return xq, sx
 
 

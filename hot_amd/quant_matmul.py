@@ -19,6 +19,7 @@ from __future__ import annotations
 from typing import Optional, Tuple
 
 import threading
+import warnings
 from dataclasses import replace
 
 import numpy as np
@@ -85,6 +86,7 @@ def token_rule(tokens: int):
 
 LOWRANK_GX_SCHEMES = ("low_rank", "gilr_gwh")
 LOWRANK_GX_MAX_BLOCK = 64
+_LOWRANK_CAP_WARNED: set = set()
 
 
 def gx_token_rule(tokens: int):
@@ -97,6 +99,12 @@ def gx_token_rule(tokens: int):
     n, rows = hla_rows(tokens, args.vectorPercentile)
     cap = min(int(args.hla_max_block), LOWRANK_GX_MAX_BLOCK)
     if n > cap:
+        if n > LOWRANK_GX_MAX_BLOCK and tokens not in _LOWRANK_CAP_WARNED:
+            _LOWRANK_CAP_WARNED.add(tokens)
+            warnings.warn("transform scheme %r at %d tokens: the reference's rule gives token blocks of %d for the g_x "
+                          "projection; the native expansion pass takes blocks up to %d, so g_x is projected with "
+                          "n = %d and differs numerically from the reference's" %
+                          (args.transform_scheme, tokens, n, LOWRANK_GX_MAX_BLOCK, cap), stacklevel=2)
         n, rows = hla_rows(cap, args.vectorPercentile)
     return n, rows
 
@@ -312,9 +320,9 @@ class FLinearQ(Function):
                                              rounding="stoch" if opt.gw_round == ops.ROUND_STOCH else "nearest",
                                              scale="row" if opt.gw_scale == ops.SCALE_ROW else "tensor",
                                              seed=opt.seed, rng_stream=ops.STREAM_GW)
-            if opt.gw_bits != opt.act_bits:
-                raise NotImplementedError("GogwQuantBit and actQuantBit must match")
-            grad_w = ops.gemm_i8(qgp, xq, lp, opt.gw_bits, sgp, sx, post_scale=1.0 / opt.hla_n, out_dtype=wc.dtype)
+            # both operands hold one code per byte whatever their widths (the token-wise kernel and the
+            # activation buffer never pack): an INT8 product, as in the fused path
+            grad_w = ops.gemm_i8(qgp, xq, lp, 8, sgp, sx, post_scale=1.0 / opt.hla_n, out_dtype=wc.dtype)
             grad_input = gx[:, :I].reshape(ctx.x_shape)
         elif go.dim() == 3 and args.batched_mode == "per_sample" and ctx.batched:
             gx, grad_w = ops.linear_backward_batched(_pad8(go), wc, xq, sx, opt)

@@ -275,6 +275,10 @@ HOT_API int hot_gx_lowrank(const void* gy, const void* w, int dtype, int64_t L, 
  * the INT8 product as two planes (q = 16 a + b) against [16 w | w].  Element e of the row-major
  * transformed g_y draws the uniforms 2 e and 2 e + 1 of Philox stream 4 under cfg->seed
  * (cfg->gx_round and gx_scale are not read).
+ * Stated deviation: the two planes carry codes up to +-2^10, and larger ones saturate there.  The
+ * reference's step comes from the maximum, not from the largest magnitude (:60-61), so a negative
+ * element of at least eight times the positive maximum of the transformed tensor would take a larger
+ * code in the reference (which multiplies in floating point); here it is held at -2^10 s.
  */
 HOT_API size_t hot_gx_luq_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_config* cfg);
 HOT_API int hot_gx_luq(const void* gy, const void* w, int dtype, int64_t L, int64_t O, int64_t I,

@@ -505,7 +505,11 @@ def gx_lowrank(g_y: np.ndarray, w: np.ndarray, cfg: HotConfig) -> BackwardTrace:
 STREAM_LUQ = 4  # the two uniforms per element of the logarithmic quantiser
 
 
-def luq_quant(t: np.ndarray, bits: int, seed: int, stream: int = STREAM_LUQ, index: Optional[np.ndarray] = None):
+LUQ_PRODUCT_MAX_EXP = 10  # largest exponent j of a code +-2^j that the two-plane INT8 product carries
+
+
+def luq_quant(t: np.ndarray, bits: int, seed: int, stream: int = STREAM_LUQ, index: Optional[np.ndarray] = None,
+              max_exp: Optional[int] = None):
     """luq_quantizer_BWD (utils/quant_matmul.py:58-77): logarithmic unbiased quantisation.  With
     lev = 2^(bits-1) - 1 and s = max(t) / 2^lev (the maximum, not the largest magnitude, :60-61):
       * magnitudes below s become s with probability |t| / s, else 0 (:62-67: u1 ~ U[0, 1));
@@ -515,7 +519,12 @@ def luq_quant(t: np.ndarray, bits: int, seed: int, stream: int = STREAM_LUQ, ind
     Returns (codes in units of s: 0 or +-2^j as int32, s fp32 [1]).  floor(log2(.)) is taken from the
     binary exponent (torch's float log2 can round an argument just below a power of two up to it).
     A tensor without a positive element has s <= 0 in the reference; here all codes are 0 then.
-    Element e draws u1, u2 = the uniforms 2 e and 2 e + 1 of `stream`."""
+    Element e draws u1, u2 = the uniforms 2 e and 2 e + 1 of `stream`.
+    `max_exp` = None is the reference: since s comes from the maximum and not from the largest
+    magnitude, a negative element beyond -max(t) takes a code as large as its size asks for.  With
+    `max_exp` = J codes saturate at +-2^J, which changes a code only where |t| >= 2^J s (the code is
+    at most 2^(k+1) with 2^k <= |t| / s), i.e. for negative elements of at least 2^(J - lev) times the
+    positive maximum: the form gx_luq uses."""
     t = np.asarray(t, dtype=F32)
     lev = 2 ** (bits - 1) - 1
     mx = max(float(t.max()), 0.0) if t.size else 0.0
@@ -532,20 +541,26 @@ def luq_quant(t: np.ndarray, bits: int, seed: int, stream: int = STREAM_LUQ, ind
     noise = (np.ldexp(F32(1.0), k).astype(F32) * (u2 - F32(0.5)).astype(F32)).astype(F32)
     v = (((m + noise).astype(F32) * F32(4.0)).astype(F32) / F32(3.0)).astype(F32)
     j = np.maximum(np.frexp(v)[1].astype(np.int64) - 1, k)
+    if max_exp is not None:
+        j = np.minimum(j, max_exp)
     q = (np.sign(t).astype(np.int64) * (np.int64(1) << j)).astype(np.int64)
     q[zero] = 0
     return q.astype(np.int32), np.array([s], dtype=F32)
 
 
-def gx_luq(g_y: np.ndarray, w: np.ndarray, cfg: HotConfig) -> BackwardTrace:
+def gx_luq(g_y: np.ndarray, w: np.ndarray, cfg: HotConfig, max_exp: Optional[int] = LUQ_PRODUCT_MAX_EXP) -> BackwardTrace:
     """grad_input with quantBWDGogi = "luq" (utils/quant_matmul.py:238, 252-253, 270, 276-285, 288-290, 343):
     g_y blkdiag(H) through the logarithmic quantiser (cfg.gx_bits, one step for the tensor), blkdiag(H) W
-    through cfg's weight quantiser, their integer product, the two steps, / n_o."""
+    through cfg's weight quantiser, their integer product, the two steps, / n_o.
+    STATED DEVIATION from the reference: the codes saturate at +-2^max_exp (default 10: what an INT8
+    product of two code planes q = 16 a + b against [16 w | w] can carry; the reference multiplies in
+    floating point and has no bound).  It is reached only by negative elements of g_y blkdiag(H) beyond
+    eight times the tensor's positive maximum; max_exp = None gives the reference's unbounded codes."""
     g_y = np.asarray(g_y, dtype=F32)
     w = np.asarray(w, dtype=F32)
     tr = BackwardTrace()
     G = fwht_blocks_last(g_y, cfg.n_o)
-    tr.qG, tr.sG = luq_quant(G, cfg.gx_bits, cfg.seed)
+    tr.qG, tr.sG = luq_quant(G, cfg.gx_bits, cfg.seed, max_exp=max_exp)
     Wh = fwht_blocks_first(w, cfg.n_o)
     tr.qW, tr.sW = quant(Wh, cfg.w_bits, cfg.w_scale, cfg.w_round, cfg.seed, STREAM_W,
                          index=colwise_rng_index(Wh.shape[1], Wh.shape[0] // cfg.n_o, np.arange(cfg.n_o)).T)

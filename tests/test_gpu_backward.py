@@ -865,6 +865,30 @@ def test_gx_luq_matches_oracle(gpu, dtype, L, O, I, variant):
     assert torch.equal(gx.cpu(), torch.from_numpy(tr.g_x).to(dtype))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("tail", [10.0, 1000.0])
+def test_gx_luq_negative_tail_beyond_the_maximum(gpu, dtype, tail):
+    """The step of the logarithmic quantiser comes from the MAXIMUM of the transformed tensor
+    (utils/quant_matmul.py:60-61), so negative elements beyond it take larger codes; the two-plane
+    product holds them at -2^10 (a stated deviation, restated by the oracle's gx_luq).  Whole blocks of
+    g_y at -tail x the largest entry put such elements into the transform."""
+    from hot_amd import ops
+    L, O, I = 448, 192, 160
+    x, w, gy = make_case(L, O, I, seed=77, dtype=torch.float32)
+    top = float(gy.abs().max())
+    gy[5, 32:48] = -tail * top
+    gy[200, 0:16] = -tail * top * 0.37
+    gy[447, 176:192] = tail * top * 1e-3            # positive side: nothing special
+    gy, w = gy.to(dtype), w.to(dtype)
+    ocfg = orc.HotConfig(seed=6)
+    opt = ops.HotOptions(n_o=ocfg.n_o, seed=ocfg.seed)
+    gx = ops.gx_luq(gy.to(gpu), w.to(gpu), opt)
+    tr = orc.gx_luq(gy.float().numpy(), w.float().numpy(), ocfg)
+    free = orc.gx_luq(gy.float().numpy(), w.float().numpy(), ocfg, max_exp=None)
+    assert int(np.abs(tr.qG).max()) == 1024 and int(np.abs(free.qG).max()) > 1024      # the bound is active
+    assert torch.equal(gx.cpu(), torch.from_numpy(tr.g_x).to(dtype))
+
+
 def test_hq_linear_with_luq_on_the_gx_path(gpu, fresh_args):
     """quantBWDGogi = "luq" through HQ_Linear: g_x from hot_gx_luq, g_W as with any other setting."""
     from hot_amd.quant_matmul import HQ_Linear
@@ -885,6 +909,73 @@ def test_hq_linear_with_luq_on_the_gx_path(gpu, fresh_args):
     fresh_args.batched_mode = "per_sample"
     with pytest.raises(NotImplementedError):
         lin(torch.randn(2, 64, I, device=gpu, requires_grad=True)).sum().backward()
+
+
+def test_hq_linear_under_autocast_matches_the_inline_buffer_write(gpu, fresh_args):
+    """The reference trains under autocast (ViT_main.py:386): x stays fp32, F.linear makes and releases
+    a bf16 copy of it while the buffer kernels run on the side stream.  Their outputs and workspace come
+    from the side stream's own pool, so the released copy cannot be handed to them; the buffer, g_x and
+    g_W equal those of the same step with the buffer written in line, over several layers in a row."""
+    from hot_amd import quant_matmul as qm
+    L, I, O = 3200, 256, 512
+    torch.manual_seed(4)
+    lins = [qm.HQ_Linear(I, O).to(gpu), qm.HQ_Linear(O, I).to(gpu), qm.HQ_Linear(I, O).to(gpu)]
+    x0 = torch.randn(L, I, device=gpu)
+    gy = torch.randn(L, O, device=gpu) * 1e-3
+
+    def run(overlap):
+        qm.overlap_buffer_write = overlap
+        fresh_args.sr_step = 0
+        for m in lins:
+            m.zero_grad(set_to_none=True)
+        x = x0.clone().requires_grad_(True)
+        with torch.autocast("cuda", dtype=torch.bfloat16):
+            h = x
+            for m in lins:
+                h = m(h).float()                    # fp32 activations between the layers, as x is
+        h.backward(gy)
+        torch.cuda.synchronize()
+        return [x.grad.clone()] + [m.weight.grad.clone() for m in lins] + [m.bias.grad.clone() for m in lins]
+
+    try:
+        ref = run(False)
+        for _ in range(3):
+            got = run(True)
+            for a, b in zip(got, ref):
+                assert torch.equal(a, b)
+    finally:
+        qm.overlap_buffer_write = True
+
+
+@pytest.mark.parametrize("gw_bits,act_bits", [(4, 8), (4, 4), (8, 4)])
+@pytest.mark.parametrize("path", ["luq", "low_rank"])
+def test_hq_linear_gw_widths_on_the_separate_gx_paths(gpu, fresh_args, path, gw_bits, act_bits):
+    """quantBWDGogi = "luq" and transform_scheme = "low_rank" compute g_W by the token-wise kernel and an
+    INT8 product of byte codes, whatever GogwQuantBit / actQuantBit are (utils/quant_matmul.py:307-324:
+    4-bit codes are integers in [-7, 7] all the same): every width pair against the oracle."""
+    from hot_amd.quant_matmul import HQ_Linear
+    L, I, O = 448, 96, 128
+    fresh_args.GogwQuantBit, fresh_args.actQuantBit = gw_bits, act_bits
+    if path == "luq":
+        fresh_args.quantBWDGogi = "luq"
+    else:
+        fresh_args.transform_scheme = "low_rank"
+    torch.manual_seed(9)
+    lin = HQ_Linear(I, O, bias=False).to(gpu)
+    x = torch.randn(L, I, device=gpu, requires_grad=True)
+    gy = torch.randn(L, O, device=gpu) * 1e-3
+    step = fresh_args.sr_step
+    lin(x).backward(gy)
+    xn, gyn, wn = x.detach().cpu().numpy(), gy.cpu().numpy(), lin.weight.detach().cpu().numpy()
+    seed = (int(fresh_args.sr_seed) << 20) + step
+    ocfg, _ = both_configs(L, seed=seed, gw_bits=gw_bits, act_bits=act_bits)
+    xq_ref, sx_ref = orc.abc_forward(xn, ocfg)
+    assert int(np.abs(xq_ref).max()) == (7 if act_bits == 4 else 127)
+    tr = orc.linear_backward(gyn, wn, xq_ref, sx_ref, ocfg)
+    assert int(np.abs(tr.qGp).max()) == (7 if gw_bits == 4 else 127)
+    assert np.array_equal(lin.weight.grad.cpu().numpy(), tr.g_w)
+    gx_ref = orc.gx_luq(gyn, wn, ocfg).g_x if path == "luq" else orc.gx_lowrank(gyn, wn, ocfg).g_x
+    assert np.array_equal(x.grad.cpu().numpy(), gx_ref)
 
 
 @pytest.mark.parametrize("variant", [dict(), dict(gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW,

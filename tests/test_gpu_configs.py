@@ -234,6 +234,116 @@ def test_llama_layers_full_size(gpu, O, I):
     assert torch.equal(gw_c[:, c], deq(np.rint(f64(qGp) @ f64(xqT[:, c])), sGp[0], sx_ref[0], 16))
 
 
+def _hla_in_strips(a, n, rows, strip=1024):
+    """fwht_blocks_first(a, n, rows) evaluated strip by strip of channels (the columns are independent):
+    the same arithmetic without a second and third copy of the whole tensor."""
+    out = np.empty(((a.shape[0] // n) * len(rows), a.shape[1]), dtype=F32)
+    for c0 in range(0, a.shape[1], strip):
+        out[:, c0:c0 + strip] = orc.fwht_blocks_first(np.ascontiguousarray(a[:, c0:c0 + strip]), n, rows)
+    return out
+
+
+@pytest.mark.parametrize("O,I", [(11008, 4096), (4096, 11008)])
+def test_llama_layers_full_size_reference_rule(gpu, O, I):
+    """Llama-7B gate/up and down at 8192 tokens with the reference's own low-rank rule
+    (utils/hadamard_matmul.py:209-226: 8192 tokens -> one block of n = 8192, r = 2080 kept sequencies),
+    bf16, Student-t gradient columns: the two-level token-wise path over every channel strip of the full
+    widths.  Steps of the whole tensors, every code of the activation buffer and of (P g_y)^T, g_W and
+    g_x on sampled rows and columns that touch every output tile."""
+    from hot_amd import ops
+    L = 8192
+    x, w, gy, heavy = llama_inputs(L, O, I, seed=O + I + 1)
+    ocfg = orc.HotConfig.python_rule(L)
+    assert (ocfg.hla_n, len(ocfg.hla_rows)) == (8192, 2080)
+    opt = options_pair(ocfg)
+    xd, wd, gyd = x.to(gpu), w.to(gpu), gy.to(gpu)
+    xq, sx = ops.abc_forward(xd, opt)
+    gx, gw = ops.linear_backward(gyd, wd, xq, sx, opt)
+    qgp_d, sgp_d, lp = ops.hla_tokenwise(gyd, ocfg.hla_n, list(ocfg.hla_rows), bits=8)
+    torch.cuda.synchronize()
+    assert lp == 2080
+    rows_sel = np.asarray(ocfg.hla_rows)
+    gyn, wn, xn = gy.float().numpy(), w.float().numpy(), x.float().numpy()
+    # activation buffer: every code, the step
+    xq_ref, sx_ref = orc.quant(_hla_in_strips(xn, L, rows_sel), 8, orc.SCALE_TENSOR)          # [L', I]
+    got = xq.cpu().numpy()
+    assert np.array_equal(sx.cpu().numpy(), sx_ref)
+    assert np.array_equal(got[:, :lp], xq_ref.T) and not got[:, lp:].any()
+    # (P g_y)^T: every code of every channel strip, the step of the whole tensor
+    GpT = np.ascontiguousarray(_hla_in_strips(gyn, L, rows_sel).T)                           # [O, L']
+    qGp, sGp = orc.quant(GpT, 8, orc.SCALE_TENSOR)
+    del GpT
+    got = qgp_d.cpu().numpy()
+    assert np.array_equal(sgp_d.cpu().numpy(), sGp)
+    assert np.array_equal(got[:, :lp], qGp) and not got[:, lp:].any()
+    # the g_x operands as in the paper-rule test; the products on sampled rows and columns
+    qG, sG = orc.quant(orc.fwht_blocks_last(gyn, 16), 4, orc.SCALE_TENSOR)
+    qW, sW = orc.quant(orc.fwht_blocks_first(wn, 16), 4, orc.SCALE_TENSOR)
+    rng = np.random.default_rng(I)
+    def sample(n):
+        return np.unique(np.concatenate([[0, 255, 256, n - 1], rng.integers(0, n, 28)]))
+    def deq(acc, sa, sb, div):
+        return torch.from_numpy((((acc.astype(F32) * F32(sa)).astype(F32) * F32(sb)).astype(F32) / F32(div)).astype(F32)
+                                ).to(torch.bfloat16)
+    f32 = lambda a: a.astype(np.float32)
+    f64 = lambda a: a.astype(np.float64)
+    gx_c, gw_c = gx.cpu(), gw.cpu()
+    r, c = sample(L), sample(I)
+    assert torch.equal(gx_c[r], deq(f32(qG[r]) @ f32(qW), sG[0], sW[0], 16))
+    assert torch.equal(gx_c[:, c], deq(f32(qG) @ f32(qW[:, c]), sG[0], sW[0], 16))
+    r, c = sample(O), sample(I)
+    assert torch.equal(gw_c[r], deq(np.rint(f64(qGp[r]) @ f64(xq_ref)), sGp[0], sx_ref[0], L))
+    assert torch.equal(gw_c[:, c], deq(np.rint(f64(qGp) @ f64(xq_ref[:, c])), sGp[0], sx_ref[0], L))
+
+
+def test_llama_layer_full_size_per_token_stochastic(gpu):
+    """Llama-7B q/k/v/o (8192 tokens, 4096 -> 4096), bf16, Student-t gradient columns, with the quantisers
+    the layer-wise selection picks most often: per-token steps and stochastic rounding on both g_y
+    operands (norm_quantizer_BWD, utils/quant_matmul.py:19-31), n = 16 / r = 8.  Every code and step of
+    both operands against the oracle under the same counter-based generator; the products on samples."""
+    from hot_amd import ops
+    L, O, I = 8192, 4096, 4096
+    x, w, gy, heavy = llama_inputs(L, O, I, seed=99)
+    ocfg = orc.HotConfig.paper(16, 8, gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW, gw_round=orc.ROUND_STOCH,
+                               gw_scale=orc.SCALE_ROW, seed=21)
+    opt = options_pair(ocfg)
+    xd, wd, gyd = x.to(gpu), w.to(gpu), gy.to(gpu)
+    xq, sx = ops.abc_forward(xd, opt)
+    gx, gw = ops.linear_backward(gyd, wd, xq, sx, opt)
+    qg_d, sg_d = ops.hq_rowwise(gyd, n=16, bits=4, rounding="stoch", scale="row", seed=21)
+    qgp_d, sgp_d, lp = ops.hla_tokenwise(gyd, 16, list(ocfg.hla_rows), bits=8, rounding="stoch", scale="row", seed=21)
+    torch.cuda.synchronize()
+    gyn, wn, xn = gy.float().numpy(), w.float().numpy(), x.float().numpy()
+    rows_sel = np.asarray(ocfg.hla_rows)
+    xq_ref, sx_ref = orc.abc_forward(xn, ocfg)
+    assert np.array_equal(xq.cpu().numpy()[:, :lp], xq_ref.T) and np.array_equal(sx.cpu().numpy(), sx_ref)
+    qG, sG = orc.quant(orc.fwht_blocks_last(gyn, 16), 4, orc.SCALE_ROW, orc.ROUND_STOCH, seed=21, stream=orc.STREAM_GX)
+    assert np.array_equal(sg_d.cpu().numpy(), sG)
+    assert np.array_equal(orc.unpack_int4(qg_d.cpu().numpy())[:, :O], qG)
+    GpT = np.ascontiguousarray(orc.fwht_blocks_first(gyn, 16, rows_sel).T)                   # [O, L']
+    qGp, sGp = orc.quant(GpT, 8, orc.SCALE_ROW, orc.ROUND_STOCH, seed=21, stream=orc.STREAM_GW,
+                         index=orc.colwise_rng_index(O, L // 16, rows_sel))
+    del GpT
+    assert np.array_equal(sgp_d.cpu().numpy(), sGp)
+    assert np.array_equal(qgp_d.cpu().numpy()[:, :lp], qGp)
+    qW, sW = orc.quant(orc.fwht_blocks_first(wn, 16), 4, orc.SCALE_TENSOR)
+    rng = np.random.default_rng(3)
+    def sample(n):
+        return np.unique(np.concatenate([[0, 255, 256, n - 1], rng.integers(0, n, 28)]))
+    def deq(acc, sa, sb, div):
+        return torch.from_numpy((((acc.astype(F32) * sa.astype(F32)).astype(F32) * F32(sb)).astype(F32) / F32(div)).astype(F32)
+                                ).to(torch.bfloat16)
+    f32 = lambda a: a.astype(np.float32)
+    f64 = lambda a: a.astype(np.float64)
+    gx_c, gw_c = gx.cpu(), gw.cpu()
+    r, c = sample(L), sample(I)
+    assert torch.equal(gx_c[r], deq(f32(qG[r]) @ f32(qW), sG[r, None], sW[0], 16))
+    assert torch.equal(gx_c[:, c], deq(f32(qG) @ f32(qW[:, c]), sG[:, None], sW[0], 16))
+    r, c = sample(O), sample(I)
+    assert torch.equal(gw_c[r], deq(np.rint(f64(qGp[r]) @ f64(xq_ref)), sGp[r, None], sx_ref[0], 16))
+    assert torch.equal(gw_c[:, c], deq(np.rint(f64(qGp) @ f64(xq_ref[:, c])), sGp[:, None], sx_ref[0], 16))
+
+
 # ------------------------------------------------------------ the whole ViT-B/16 step
 
 def test_vit_b16_full_model_step(gpu):

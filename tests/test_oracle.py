@@ -513,6 +513,38 @@ def test_luq_levels_step_and_expectation():
     assert not q3.any() and s3[0] <= 0
 
 
+def test_luq_saturation_of_the_product_form():
+    """The reference's logarithmic codes have no upper bound (the step is max(t) / 2^7, not absmax / 2^7:
+    utils/quant_matmul.py:60-61,71-74); the two-plane INT8 product saturates at 2^10.  The bound changes
+    a code only for negative elements of at least eight times the positive maximum, and then to -2^10."""
+    t = np.array([[1e-3, -0.5, 2e-4, -3e-2, -7.9e-3, 5e-4]], dtype=np.float32)
+    free, s = orc.luq_quant(t, 4, seed=0)
+    held, s2 = orc.luq_quant(t, 4, seed=0, max_exp=orc.LUQ_PRODUCT_MAX_EXP)
+    assert s[0] == s2[0] == np.float32(1e-3) / np.float32(128)
+    assert free[0, 1] == -65536 and free[0, 3] in (-2048, -4096)       # 500 x and 30 x the maximum
+    assert held[0, 1] == -1024 and held[0, 3] == -1024
+    below = np.abs(t[0]) < 1024 * s[0]
+    assert np.array_equal(free[0, below], held[0, below]) and below.tolist() == [True, False, True, False, True, True]
+    # -7.9e-3 is 1011 s: its code may round up to 1024 but not beyond; held and free agree whenever free <= 1024
+    assert abs(int(held[0, 4])) in (512, 1024) and (free[0, 4] == held[0, 4])
+    rng = np.random.default_rng(5)
+    for seed in range(20):
+        u = (rng.standard_normal((16, 32)) * 1e-3).astype(np.float32)
+        a, _ = orc.luq_quant(u, 4, seed=seed)
+        b, _ = orc.luq_quant(u, 4, seed=seed, max_exp=10)
+        assert np.array_equal(np.clip(a, -1024, 1024), b)
+        if np.abs(u).max() < 8 * u.max():
+            assert np.array_equal(a, b)
+    # gx_luq is the product form: saturated by default, the reference's codes on request
+    gy = (rng.standard_normal((32, 32)) * 1e-3).astype(np.float32)
+    gy[3, :16] = -0.4                                  # one block whose transform is far below -max
+    w = (rng.standard_normal((32, 24)) * 0.1).astype(np.float32)
+    tr_h, tr_f = orc.gx_luq(gy, w, orc.HotConfig(seed=1)), orc.gx_luq(gy, w, orc.HotConfig(seed=1), max_exp=None)
+    assert np.abs(tr_h.qG).max() == 1024 and np.abs(tr_f.qG).max() > 1024
+    keep = np.ones(32, bool); keep[3] = False
+    assert np.array_equal(tr_h.g_x[keep], tr_f.g_x[keep])
+
+
 def test_gx_luq_close_to_the_plain_product():
     rng = np.random.default_rng(2)
     L, O, I = 256, 64, 48
