@@ -6,6 +6,7 @@
 // low-rank -> GEMM x2 -> dequantise) with the numerics of FLinearQ.backward,
 // scheme gih_gwlr (utils/quant_matmul.py:215-348).  hot_abc_forward is the
 // forward-side activation buffer of FLinearQ.setup_context (:178-212).
+#include <stdlib.h>
 #include <string.h>
 
 #include <mutex>
@@ -295,7 +296,8 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   // beside the g_y statistics.
   std::unique_lock<std::mutex> side_guard(g_side_mutex, std::defer_lock);
   SideLane* side = nullptr;
-  if (!ev) {
+  static const bool sw_serial = [] { const char* v = getenv("HOT_SERIAL"); return v && *v == '1'; }();   // developer switch
+  if (!ev && !sw_serial) {
     side_guard.lock();
     side = side_lane_locked();
     if (!side) side_guard.unlock();
@@ -325,8 +327,7 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   // g_y: HLA along tokens + quantise, transposed (g_W operand); Hadamard along O + quantise (g_x
   // operand).  With one step per tensor both quantisers need the absmax of their transform first:
   // the statistics pass of the token-wise kernel delivers both from a single read of g_y.
-  const bool fuse = cfg->gx_scale == HOT_SCALE_TENSOR && cfg->n_o == 16 && O % 16 == 0 && cfg->gw_scale != HOT_SCALE_SAWB &&
-                    cfg->hla_n <= COL_MAX_N;
+  const bool fuse = cfg->gx_scale == HOT_SCALE_TENSOR && cfg->n_o == 16 && O % 16 == 0 && cfg->gw_scale != HOT_SCALE_SAWB;
   // Side stream, beside the g_W GEMM on the main stream: always the row-wise quantise pass of g_y (a
   // streaming kernel next to a matrix kernel); the g_x GEMM too when the g_W GEMM has fewer tiles
   // than the chip has CUs and cannot fill it alone (two large GEMMs only get in each other's way).

@@ -300,6 +300,7 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
     }
     rcp = 1.0f / d;
   }
+  const float rcpk = rcp * 65536.0f;       // stochastic rounding works in units of 2^-16
 
   float cmax = 0.f, rmax = 0.f, csum = 0.f;
   double ssq = 0.0, sab = 0.0;
@@ -316,14 +317,14 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
         // coefficient 0 of a block is the sum of its tokens (row 0 of H is all ones)
         if constexpr (PASS == 0) csum += x[g * N];
         int visited = 0;      // kept coefficients of this block quantised so far (stochastic rounding)
-        float u[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        uint32_t u[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};   // 16-bit uniform integers of eight visits
         if constexpr (PASS == 1 && ROUND != HOT_ROUND_NEAREST && N == 1) {
           // blocks of one token keep their one coefficient: element number = channel * NB + block, so
           // eight consecutive blocks of a channel share a generator call (u1 lives across the blocks
           // of this step; a new call at the first block and wherever the number passes a multiple of 8)
           const uint64_t e = (uint64_t)c * (uint64_t)a.NB + (uint64_t)(blk0 + blk);
           if (g == 0 || (e & 7u) == 0) u1 = sr_octet_words(e >> 3, a.seed, a.stream);
-          u[0] = sr_uniform_of(u1, (uint32_t)e);
+          u[0] = sr_bits_of(u1, (uint32_t)e);
         }
 #pragma unroll
         for (int i = 0; i < N; ++i) {
@@ -349,16 +350,15 @@ __global__ void __launch_bounds__(CW) colwise_kernel(const ColArgs a) {
                     // a single kept coefficient per block: numbered channel * NB + block, like the
                     // one-token blocks above
                     const uint64_t e = (uint64_t)c * (uint64_t)a.NB + (uint64_t)(blk0 + blk);
-                    u[0] = sr_uniform_of(sr_octet_words(e >> 3, a.seed, a.stream), (uint32_t)e);
+                    u[0] = sr_bits_of(sr_octet_words(e >> 3, a.seed, a.stream), (uint32_t)e);
                   } else {
                     const uint64_t oct = ((uint64_t)c * (uint64_t)a.NB + (uint64_t)(blk0 + blk)) * (uint64_t)(a.rpad >> 3) +
                                          (uint64_t)(visited >> 3);
-                    sr_uniform8(oct, a.seed, a.stream, u);
+                    sr_bits8(oct, a.seed, a.stream, u);
                   }
                 }
-                q = q_stoch_div(v, d, rcp, u[visited & 7]);
+                q = q_stoch_fix(v, rcpk, u[visited & 7], qmax);   // (the minimum inside: floor + 1 may step past qmax at the very top)
                 ++visited;
-                q = clampi(q, -qmax, qmax);   // floor + 1 may step past qmax at the very top
               }
               stage[tid * pitch + blk * a.r + sl] = (uint8_t)(q & 0xFF);
             }
@@ -893,7 +893,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   }
   if (n > COL_MAX_N) {
     // blocks one thread cannot hold: the two-level path
-    if (store4 || row16_absmax_out) return fail(HOT_ERR_UNSUPPORTED, "%s: blocks above %d tokens have no packed-INT4 store and no fused row statistic", who, COL_MAX_N);
+    if (store4) return fail(HOT_ERR_UNSUPPORTED, "%s: blocks above %d tokens have no packed-INT4 store", who, COL_MAX_N);
     if (R % n) return fail(HOT_ERR_INVALID, "%s: R=%lld is not a multiple of the block %d", who, (long long)R, n);
     if (r < 1 || r > n) return fail(HOT_ERR_INVALID, "%s: r=%d outside [1, %d]", who, r, n);
     if (bits != 4 && bits != 8) return fail(HOT_ERR_UNSUPPORTED, "%s: bits=%d (4 or 8)", who, bits);
@@ -910,7 +910,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
       }
     }
     return hla_big_impl(in, dtype, R, C, n, rows, r, bits, rounding, seed, rng_stream, scale_mode, codes_out, ld_out,
-                        scales_out, workspace, workspace_bytes, st, who, after_stats);
+                        scales_out, workspace, workspace_bytes, st, who, after_stats, row16_absmax_out);
   }
   if (n < 1 || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (a power of two)", who, n);
   if (R % n) return fail(HOT_ERR_INVALID, "%s: R=%lld is not a multiple of the block %d", who, (long long)R, n);

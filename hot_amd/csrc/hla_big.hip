@@ -48,6 +48,7 @@ struct BigArgs {
   float* colmax;       // per-channel absmax (ROW)
   double* partial;     // SAWB: 2 doubles per workgroup
   float* scales_out;
+  float* row_absmax;   // stage 1 with RS: absmax of the row-wise 16-point Hadamard (STAT_SLOTS partial maxima), or null
   uint64_t seed;
   uint32_t stream;
 };
@@ -72,15 +73,67 @@ __device__ __forceinline__ void fwht(float (&v)[N]) {
   }
 }
 
-template <typename T>
+// RS: the pass also tracks the absmax of the ROW-wise 16-point block Hadamard of the same input (the
+// statistic of the row-wise quantiser of g_y, so that g_y is not read a further time for it).
+// Adjacent lanes hold adjacent channels; within each group of 16 lanes the channels are dealt out so
+// that the four stages of the 16-point transform pair lanes at the distances a single DPP operand
+// reaches (channel bit 0 <-> lane xor 1, bit 1 <-> xor 2, bit 2 <-> xor 15, bit 3 <-> xor 8).  A stage
+// computes own + s * partner with s = -1 on the lane of the upper channel of a pair: a lane's value
+// may come out negated, magnitudes are those of the add / sub butterflies (the product with +-1 is
+// exact).  C must be a multiple of 16: a group of 16 lanes is whole or absent.
+template <typename T, bool RS>
 __global__ void __launch_bounds__(BT) big_stage1_kernel(const BigArgs a) {
-  const int64_t c = (int64_t)blockIdx.x * BT + threadIdx.x;
-  if (c >= a.C) return;
+  __shared__ float s_max[BT / 64];
+  const int tid = threadIdx.x;
+  const int chan = RS ? (tid ^ ((tid & 4) ? 0xB : 0)) : tid;
+  const int64_t c = (int64_t)blockIdx.x * BT + chan;
+  const bool active = c < a.C;
+  if (!RS && !active) return;
   const int64_t row0 = (int64_t)blockIdx.y * 64;
-  const T* in = reinterpret_cast<const T*>(a.in) + row0 * a.C + c;
+  const T* in = reinterpret_cast<const T*>(a.in) + row0 * a.C + (active ? c : 0);
   float v[64];
 #pragma unroll
   for (int i = 0; i < 64; ++i) v[i] = load_f32<T>(in + (int64_t)i * a.C);
+  if constexpr (RS) {
+    const float sg1 = (chan & 1) ? -1.f : 1.f, sg2 = (chan & 2) ? -1.f : 1.f;
+    const float sg4 = (chan & 4) ? -1.f : 1.f, sg8 = (chan & 8) ? -1.f : 1.f;
+    float rmax = 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      float t[16];
+#pragma unroll
+      for (int i = 0; i < 16; ++i) t[i] = v[16 * g + i];
+      // every row is in its register before the first DPP read (the compiler's hazard check does not
+      // look into asm statements); the stages run row-major over the sixteen rows, so no DPP read
+      // follows the write of its register within two instructions
+      asm volatile("s_nop 1"
+                   : "+v"(t[0]), "+v"(t[1]), "+v"(t[2]), "+v"(t[3]), "+v"(t[4]), "+v"(t[5]), "+v"(t[6]), "+v"(t[7]),
+                     "+v"(t[8]), "+v"(t[9]), "+v"(t[10]), "+v"(t[11]), "+v"(t[12]), "+v"(t[13]), "+v"(t[14]), "+v"(t[15]));
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        asm volatile("v_fmac_f32_dpp %0, %0, %1 quad_perm:[1,0,3,2] row_mask:0xf bank_mask:0xf" : "+v"(t[i]) : "v"(sg1));
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        asm volatile("v_fmac_f32_dpp %0, %0, %1 quad_perm:[2,3,0,1] row_mask:0xf bank_mask:0xf" : "+v"(t[i]) : "v"(sg2));
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        asm volatile("v_fmac_f32_dpp %0, %0, %1 row_mirror row_mask:0xf bank_mask:0xf" : "+v"(t[i]) : "v"(sg4));
+#pragma unroll
+      for (int i = 0; i < 16; ++i)
+        asm volatile("v_fmac_f32_dpp %0, %0, %1 row_ror:8 row_mask:0xf bank_mask:0xf" : "+v"(t[i]) : "v"(sg8));
+#pragma unroll
+      for (int i = 0; i < 16; ++i) rmax = fmaxf(rmax, fabsf(t[i]));
+    }
+    const float m = wave_max(active ? rmax : 0.f);
+    if ((tid & 63) == 0) s_max[tid >> 6] = m;
+    __syncthreads();
+    if (tid == 0) {
+      float mm = s_max[0];
+      for (int i = 1; i < BT / 64; ++i) mm = fmaxf(mm, s_max[i]);
+      stat_slot_update(a.row_absmax, blockIdx.y * gridDim.x + blockIdx.x, mm);
+    }
+    if (!active) return;
+  }
   fwht<64>(v);
   float* out = a.T + (int64_t)blockIdx.y * a.nk * a.C + c;    // T [run][needed coefficient][channel]
 #pragma unroll
@@ -88,13 +141,9 @@ __global__ void __launch_bounds__(BT) big_stage1_kernel(const BigArgs a) {
     if ((a.kmask >> i) & 1ull) { *out = v[i]; out += a.C; }
 }
 
-__device__ __forceinline__ float uniform_of(uint64_t e, uint64_t seed, uint32_t stream) {
-  float u[8];
-  sr_uniform8(e >> 3, seed, stream, u);
-  float r = u[0];
-#pragma unroll
-  for (int i = 1; i < 8; ++i) r = ((uint32_t)e & 7u) == (uint32_t)i ? u[i] : r;
-  return r;
+// the 16-bit uniform integer of element e
+__device__ __forceinline__ uint32_t bits_of(uint64_t e, uint64_t seed, uint32_t stream) {
+  return sr_bits_of(sr_octet_words(e >> 3, seed, stream), (uint32_t)e);
 }
 
 // blockIdx.y = block * nk + (index of k among the needed coefficients)
@@ -181,7 +230,7 @@ __global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
         q = (int)rint_div_fast(x, d, rcp);      // bit for bit rintf(x / d)
       } else {
         const uint64_t idx = ((uint64_t)c * (uint64_t)a.NB + (uint64_t)blk) * (uint64_t)a.rpad + (uint64_t)visit;
-        q = clampi(q_stoch(x / d, uniform_of(idx, a.seed, a.stream)), -qmax, qmax);
+        q = q_stoch_fix(x, rcp * 65536.0f, bits_of(idx, a.seed, a.stream), qmax);
       }
       a.tmp[(blk * a.r + slot) * a.C + c] = (int8_t)q;
     }
@@ -307,7 +356,7 @@ size_t hla_big_workspace_bytes_impl(int64_t R, int64_t C, int n, int r) {
 int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r, int bits,
                  int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_out,
                  float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st, const char* who,
-                 hipEvent_t after_stats) {
+                 hipEvent_t after_stats, float* row16_absmax_out) {
   const int m = n / 64;
   if (n < 256 || n > 8192 || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (a power of two, 256 .. 8192)", who, n);
   const int64_t NB = R / n, kout = NB * r;
@@ -365,10 +414,22 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
   }
   if (int rc = check_launch("big_table_kernel")) return rc;
   const dim3 g1((unsigned)gx, (unsigned)(R / 64));
+  a.row_absmax = row16_absmax_out;
+  if (row16_absmax_out && (C % 16 || scale_mode == HOT_SCALE_SAWB))
+    return fail(HOT_ERR_UNSUPPORTED, "%s: fused row statistic unavailable for this configuration", who);
   switch (dtype) {
-    case HOT_F32: hipLaunchKernelGGL(big_stage1_kernel<float>, g1, dim3(BT), 0, st, a); break;
-    case HOT_BF16: hipLaunchKernelGGL(big_stage1_kernel<bf16_t>, g1, dim3(BT), 0, st, a); break;
-    case HOT_F16: hipLaunchKernelGGL(big_stage1_kernel<f16_t>, g1, dim3(BT), 0, st, a); break;
+    case HOT_F32:
+      if (row16_absmax_out) hipLaunchKernelGGL((big_stage1_kernel<float, true>), g1, dim3(BT), 0, st, a);
+      else hipLaunchKernelGGL((big_stage1_kernel<float, false>), g1, dim3(BT), 0, st, a);
+      break;
+    case HOT_BF16:
+      if (row16_absmax_out) hipLaunchKernelGGL((big_stage1_kernel<bf16_t, true>), g1, dim3(BT), 0, st, a);
+      else hipLaunchKernelGGL((big_stage1_kernel<bf16_t, false>), g1, dim3(BT), 0, st, a);
+      break;
+    case HOT_F16:
+      if (row16_absmax_out) hipLaunchKernelGGL((big_stage1_kernel<f16_t, true>), g1, dim3(BT), 0, st, a);
+      else hipLaunchKernelGGL((big_stage1_kernel<f16_t, false>), g1, dim3(BT), 0, st, a);
+      break;
     default: return fail(HOT_ERR_INVALID, "%s: bad dtype %d", who, dtype);
   }
   if (int rc = check_launch("big_stage1_kernel")) return rc;

@@ -112,14 +112,17 @@ template <> __device__ __forceinline__ void store_scalar<float>(float* p, float 
 template <> __device__ __forceinline__ void store_scalar<bf16_t>(bf16_t* p, float v) { p->v = f32_to_bf16_rne(v); }
 template <> __device__ __forceinline__ void store_scalar<f16_t>(f16_t* p, float v) { p->v = (_Float16)v; }
 
-// ---- Philox-4x32-10 -------------------------------------------------------
+// ---- Philox-4x32-7 --------------------------------------------------------
+// The counter-based generator of stochastic rounding: seven rounds of Philox-4x32 (the fewest that
+// Random123 reports as passing BigCrush; its default of ten adds a margin that rounding does not need).
 
 struct philox4 { uint32_t w[4]; };
+constexpr int SR_PHILOX_ROUNDS = 7;
 
-__device__ __forceinline__ philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+__device__ __forceinline__ philox4 philox4x32_sr(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
                                                  uint32_t k0, uint32_t k1) {
 #pragma unroll
-  for (int r = 0; r < 10; ++r) {
+  for (int r = 0; r < SR_PHILOX_ROUNDS; ++r) {
     // one 32 x 32 -> 64 multiply per product (v_mad_u64_u32) instead of a high and a low multiply
     const uint64_t p0 = (uint64_t)0xD2511F53u * (uint64_t)c0, p1 = (uint64_t)0xCD9E8D57u * (uint64_t)c2;
     const uint32_t hi0 = (uint32_t)(p0 >> 32), lo0 = (uint32_t)p0;
@@ -135,7 +138,7 @@ __device__ __forceinline__ philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint3
 // Uniforms (2^-16 grid) for the eight elements whose linear indices are 8*oct .. 8*oct+7: element
 // 2 i + h takes the low (h = 0) or high (h = 1) half of output word i of one Philox call.
 __device__ __forceinline__ void sr_uniform8(uint64_t oct, uint64_t seed, uint32_t stream, float* u) {
-  const philox4 p = philox4x32_10((uint32_t)oct, (uint32_t)(oct >> 32), stream, 0u,
+  const philox4 p = philox4x32_sr((uint32_t)oct, (uint32_t)(oct >> 32), stream, 0u,
                                   (uint32_t)seed, (uint32_t)(seed >> 32));
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -150,43 +153,43 @@ __device__ __forceinline__ void sr_uniform8(uint64_t oct, uint64_t seed, uint32_
 // element e is picked with selects and a shift.
 struct philox_words { uint32_t w0, w1, w2, w3; };
 __device__ __forceinline__ philox_words sr_octet_words(uint64_t oct, uint64_t seed, uint32_t stream) {
-  const philox4 p = philox4x32_10((uint32_t)oct, (uint32_t)(oct >> 32), stream, 0u,
+  const philox4 p = philox4x32_sr((uint32_t)oct, (uint32_t)(oct >> 32), stream, 0u,
                                   (uint32_t)seed, (uint32_t)(seed >> 32));
   philox_words o;
   o.w0 = p.w[0]; o.w1 = p.w[1]; o.w2 = p.w[2]; o.w3 = p.w[3];
   return o;
 }
-__device__ __forceinline__ float sr_uniform_of(const philox_words& p, uint32_t e) {
+// The same draws as 16-bit integers (what the fixed-point rounding below adds): r[2 i + h] = the low
+// (h = 0) or high half of output word i of the call for octet `oct`.
+__device__ __forceinline__ void sr_bits8(uint64_t oct, uint64_t seed, uint32_t stream, uint32_t* r) {
+  const philox4 p = philox4x32_sr((uint32_t)oct, (uint32_t)(oct >> 32), stream, 0u, (uint32_t)seed, (uint32_t)(seed >> 32));
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    r[2 * i] = p.w[i] & 0xFFFFu;
+    r[2 * i + 1] = p.w[i] >> 16;
+  }
+}
+__device__ __forceinline__ uint32_t sr_bits_of(const philox_words& p, uint32_t e) {
   const uint32_t i = (e >> 1) & 3u;
   const uint32_t lo = (i & 1u) ? p.w1 : p.w0, hi = (i & 1u) ? p.w3 : p.w2;
   const uint32_t w = (i & 2u) ? hi : lo;
-  return (float)((w >> ((e & 1u) * 16u)) & 0xFFFFu) * 1.52587890625e-05f;
+  return (w >> ((e & 1u) * 16u)) & 0xFFFFu;
 }
 
 // ---- quantisation of one value --------------------------------------------
 
+// Stochastic rounding of x / d in 16.16 fixed point, rcpk = fl32(1 / d) * 65536, r a 16-bit uniform
+// integer: p = fma(|x|, rcpk, 0.5) is |x / d| in units of 2^-16, rounded to the nearest; adding r
+// carries into the integer part with probability frac(|x / d|) on a 2^-16 grid.  One fused
+// multiply-add, a conversion, an add, a shift, a minimum and the sign: no division, no branch.
+__device__ __forceinline__ int q_stoch_fix(float x, float rcpk, uint32_t r, int qmax) {
+  const float p = __builtin_fmaf(fabsf(x), rcpk, 0.5f);
+  const uint32_t m = min(((uint32_t)p + r) >> 16, (uint32_t)qmax);
+  return x < 0.f ? -(int)m : (int)m;
+}
+
 // y = x / d already divided.  Nearest: ties to even.
 __device__ __forceinline__ int q_nearest(float y) { return (int)rintf(y); }
-
-__device__ __forceinline__ int q_stoch(float y, float u) {
-  const float ay = fabsf(y);
-  const float fl = floorf(ay);
-  const float frac = ay - fl;
-  const int m = (int)fl + (u < frac ? 1 : 0);
-  return y < 0.f ? -m : m;
-}
-
-// q_stoch(x / d, u) with rcp = 1 / d precomputed.  p = x * rcp is within 2^-15 of the IEEE quotient
-// (|x / d| <= 128), so floor and the comparison with u come out the same unless the fractional part
-// lies within 2^-14 of 0, of 1 or of u; only then is the division carried out.
-__device__ __forceinline__ int q_stoch_div(float x, float d, float rcp, float u) {
-  const float eps = 6.103515625e-05f;
-  const float p = x * rcp;
-  const float ap = fabsf(p), fl = floorf(ap), frac = ap - fl;
-  if (__builtin_expect(fabsf(frac - u) < eps || frac < eps || frac > 1.0f - eps, 0)) return q_stoch(x / d, u);
-  const int m = (int)fl + (u < frac ? 1 : 0);
-  return p < 0.f ? -m : m;
-}
 
 __device__ __forceinline__ int clampi(int v, int lo, int hi) { return v < lo ? lo : (v > hi ? hi : v); }
 

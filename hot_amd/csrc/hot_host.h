@@ -73,11 +73,13 @@ size_t colwise_workspace_bytes_impl(int64_t C);
 size_t colwise_stats_bytes_impl(int64_t C);  // leading part of the workspace that must be zero before the statistics pass
 
 // Blocks of 256 .. 8192 tokens (two-level transform through an fp32 workspace); same contract as
-// colwise_quant_impl without the packed-INT4 store and the fused row statistic.
+// colwise_quant_impl without the packed-INT4 store.
 int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r, int bits,
                  int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_out,
                  float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st, const char* who,
-                 hipEvent_t after_stats = nullptr);
+                 hipEvent_t after_stats = nullptr, float* row16_absmax_out = nullptr);
+// row16_absmax_out (STAT_SLOTS partial maxima, zero before the call; C a multiple of 16, absmax steps):
+// stage 1 also delivers the absmax of the row-wise 16-point Hadamard of the input.
 size_t hla_big_workspace_bytes_impl(int64_t R, int64_t C, int n, int r);
 // Workspace of a token-wise transform of [R, C] with blocks of n tokens and r kept rows, either path.
 size_t hla_workspace_bytes_impl(int64_t R, int64_t C, int n, int r);

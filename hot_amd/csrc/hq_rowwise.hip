@@ -82,10 +82,11 @@ __device__ __forceinline__ void quant_store_chunk(const float* x, float d, float
 #pragma unroll
     for (int j = 0; j < EPL; ++j) q[j] = (int)rint_div_fast(x[j], d, rcp);
   } else {
-    float u[EPL];
-    sr_uniform8(e0 >> 3, seed, stream, u);       // e0 is a multiple of EPL = 8
+    uint32_t r[EPL];
+    sr_bits8(e0 >> 3, seed, stream, r);          // e0 is a multiple of EPL = 8
+    const float rcpk = rcp * 65536.0f;
 #pragma unroll
-    for (int j = 0; j < EPL; ++j) q[j] = clampi(q_stoch_div(x[j], d, rcp, u[j]), -QMAX, QMAX);
+    for (int j = 0; j < EPL; ++j) q[j] = q_stoch_fix(x[j], rcpk, r[j], QMAX);
   }
   if constexpr (BITS == 4) {
     uint32_t w = 0;

@@ -41,7 +41,7 @@
 extern "C" {
 #endif
 
-#define HOT_ABI_VERSION 3
+#define HOT_ABI_VERSION 4
 #define HOT_API __attribute__((visibility("default")))
 
 enum hot_status {
@@ -53,6 +53,14 @@ enum hot_status {
 };
 
 enum hot_dtype { HOT_F32 = 0, HOT_BF16 = 1, HOT_F16 = 2 };
+/* HOT_ROUND_NEAREST: rint(x / fl32(s + 1e-11)), ties to even, IEEE division (int_quantizer_BWD,
+ *   utils/quant_matmul.py:108-116).
+ * HOT_ROUND_STOCH: floor|y| + 1 with probability frac|y|, y = x / fl32(s + 1e-11) (stoch_quantizer_BWD /
+ *   norm_quantizer_BWD, :19-31, 86-100), from a counter-based generator instead of the reference's global
+ *   one: element e draws the 16-bit integer r_e = halfword (e & 7) of the Philox-4x32-7 output for counter
+ *   (e >> 3 lo, e >> 3 hi, stream, 0) under key (seed lo, seed hi), and the code is
+ *   sign(x) min((trunc(fma(|x|, fl32(1 / d) 2^16, 0.5)) + r_e) >> 16, qmax): the expectation is y within
+ *   2^-15 of a step.  The numbering of the elements is stated with every entry point. */
 enum hot_rounding { HOT_ROUND_NEAREST = 0, HOT_ROUND_STOCH = 1 };
 enum hot_scale_mode {
   HOT_SCALE_TENSOR = 0, /* one absmax step for the whole tensor */

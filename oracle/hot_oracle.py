@@ -12,9 +12,10 @@ file:line is given per function.  Two deliberate, documented differences:
   ``fwht_kernel`` (HLQ_backward_kernel.cu:63-78), instead of the BLAS matmul
   ``reshape(-1, n) @ H`` of hadamard_matmul.py:121-161 whose last-ulp
   summation order depends on the BLAS build.  Mathematically identical.
-* Stochastic rounding draws its uniforms from Philox-4x32-10 keyed by
+* Stochastic rounding draws 16-bit uniforms from Philox-4x32-7 keyed by
   (seed, element index) instead of the global torch generator
-  (quant_matmul.py:96), so that CPU and GPU agree bit for bit.
+  (quant_matmul.py:96) and rounds in 16.16 fixed point (sr_codes), so that CPU
+  and GPU agree bit for bit.
 
 How each function is pinned (tests/test_oracle_*.py):
   pow2_factor / pow2_factor_max16   closed form n & -n; hand-derived table
@@ -228,21 +229,53 @@ def philox4x32(c0, c1, c2, c3, k0: int, k1: int, rounds: int = 10):
     return (c0.astype(np.uint32), c1.astype(np.uint32), c2.astype(np.uint32), c3.astype(np.uint32))
 
 
-def sr_uniform(index: np.ndarray, seed: int, stream: int) -> np.ndarray:
-    """u in [0, 1) on a 2^-16 grid for the element with linear index ``index``
-    (int64 array).  One Philox call serves eight consecutive elements:
-    counter = (index>>3 lo, index>>3 hi, stream, 0), key = (seed lo, seed hi);
-    element index & 7 = 2 i + h takes the low (h = 0) or high (h = 1) 16 bits of
-    output word i, u = halfword * 2^-16.  (Sixteen bits bound the bias of a
-    rounding probability by 2^-16 of a quantisation step.)"""
+SR_PHILOX_ROUNDS = 7   # Philox-4x32-7: the fewest rounds Random123 reports as passing BigCrush (10 is its default margin)
+
+
+def sr_bits16(index: np.ndarray, seed: int, stream: int) -> np.ndarray:
+    """A 16-bit uniform integer (uint32 array) for the element with linear index
+    ``index`` (int64 array).  One Philox-4x32-7 call serves eight consecutive
+    elements: counter = (index>>3 lo, index>>3 hi, stream, 0), key = (seed lo,
+    seed hi); element index & 7 = 2 i + h takes the low (h = 0) or high (h = 1)
+    16 bits of output word i.  The 10-round function is pinned by Random123's
+    known answers; seven rounds are the same round function and key schedule
+    applied seven times."""
     index = np.asarray(index, dtype=np.uint64)
     q = index >> np.uint64(3)
     w = philox4x32(q & _MASK, q >> np.uint64(32), np.full(q.shape, stream, np.uint64),
-                   np.zeros(q.shape, np.uint64), seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF)
+                   np.zeros(q.shape, np.uint64), seed & 0xFFFFFFFF, (seed >> 32) & 0xFFFFFFFF, rounds=SR_PHILOX_ROUNDS)
     slot = (index & np.uint64(7)).astype(np.int64)
     word = np.choose(slot >> 1, w).astype(np.uint32)
-    half = np.where((slot & 1) == 0, word & np.uint32(0xFFFF), word >> np.uint32(16))
-    return (half.astype(F32) * F32(2.0 ** -16)).astype(F32)
+    return np.where((slot & 1) == 0, word & np.uint32(0xFFFF), word >> np.uint32(16)).astype(np.uint32)
+
+
+def sr_uniform(index: np.ndarray, seed: int, stream: int) -> np.ndarray:
+    """u in [0, 1) on a 2^-16 grid: sr_bits16 * 2^-16 (the logarithmic quantiser's two uniforms)."""
+    return (sr_bits16(index, seed, stream).astype(F32) * F32(2.0 ** -16)).astype(F32)
+
+
+def sr_codes(t: np.ndarray, d: np.ndarray, qmax: int, index: np.ndarray, seed: int, stream: int) -> np.ndarray:
+    """Stochastic rounding of t / d to integers of magnitude <= qmax, in the fixed-point form the
+    kernels use: with rcp = fl32(1 / d),
+        p = fl32(|t| * (rcp * 2^16) + 0.5)        one fused multiply-add: |t| / d in units of 2^-16, rounded
+        q = sign(t) * min((trunc(p) + r) >> 16, qmax),   r = sr_bits16(element)
+    i.e. floor(|y|) + 1 with probability frac(|y|) taken on a 2^-16 grid, y = t / d: the stochastic
+    rounding of stoch_quantizer_BWD / norm_quantizer_BWD (utils/quant_matmul.py:19-31, 86-100) with a
+    counter-based generator.  The product with the reciprocal stands for the division (at most 1.5 ulp
+    apart) and the grid rounds the probability to the nearest 2^-16: E[q] is within 2^-15 of y."""
+    return sr_round(t, d, qmax, sr_bits16(index, seed, stream))
+
+
+def sr_round(t: np.ndarray, d: np.ndarray, qmax: int, r: np.ndarray) -> np.ndarray:
+    """The arithmetic of sr_codes for given 16-bit integers r."""
+    t = np.asarray(t, dtype=F32)
+    rcpk = ((F32(1.0) / np.asarray(d, dtype=F32)).astype(F32) * F32(65536.0)).astype(F32)
+    # fused multiply-add in fp32 = the exact product and sum, rounded once.  The product of two fp32
+    # numbers is exact in float64, and so is the sum with 0.5 wherever it can reach 1 (48 significant
+    # bits from 2^-1 up); below that the truncation gives 0 whatever the last bit
+    p = (np.abs(t).astype(np.float64) * rcpk.astype(np.float64) + 0.5).astype(F32)
+    m = np.minimum((np.trunc(p).astype(np.int64) + np.asarray(r).astype(np.int64)) >> 16, qmax)
+    return np.where(t < 0, -m, m)
 
 
 # --------------------------------------------------------------------------
@@ -292,7 +325,7 @@ def quant(t: np.ndarray, bits: int, mode: int = SCALE_TENSOR, rounding: int = RO
     y = clamp(t, -clip, clip) / fl32(s + 1e-11)           (IEEE fp32 division)
     nearest:     q = rint(y), ties to even   (int_quantizer_BWD  :112-116,
                                               sawb_quantizer_BWD :40-49)
-    stochastic:  q = sign(y) (floor|y| + (u < |y| - floor|y|))
+    stochastic:  q = sign(y) (floor|y| + Bernoulli(|y| - floor|y|)), evaluated by sr_codes
                                              (stoch_quantizer_BWD :86-100,
                                               norm_quantizer_BWD  :19-31)
     ``index`` gives the RNG element index of every entry (default: row-major
@@ -306,11 +339,7 @@ def quant(t: np.ndarray, bits: int, mode: int = SCALE_TENSOR, rounding: int = RO
     else:
         if index is None:
             index = np.arange(t.size, dtype=np.int64).reshape(t.shape)
-        u = sr_uniform(index, seed, stream)
-        ay = np.abs(y)
-        fl = np.floor(ay)
-        frac = (ay - fl).astype(F32)
-        q = np.sign(y) * (fl + (u < frac))
+        q = sr_codes(np.clip(t, -clip, clip).astype(F32), d, _qmax(bits), index, seed, stream)
     qm = _qmax(bits)
     q = np.clip(q, -qm, qm)  # never active for absmax scales; guards sawb/eps
     s_out = s.reshape(-1) if mode == SCALE_ROW else np.asarray(s, dtype=F32).reshape(1)

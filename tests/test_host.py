@@ -209,7 +209,7 @@ def test_library_exports_every_declared_symbol():
     lib = C.CDLL(_lib.LIB_PATH)
     for n in names:
         assert hasattr(lib, n), n
-    assert _lib.lib().hot_abi_version() == 3
+    assert _lib.lib().hot_abi_version() == 4
     header = open(os.path.join(ROOT, "include", "hot_gfx950.h")).read()
     for name in ("HOT_MAX_HLA_N", "HOT_MAX_HLA_BIG", "HOT_HQ_WORKSPACE_BYTES", "HOT_STATIC_MAX_CHANNELS"):   # the binding repeats these constants
         assert int(re.search(r"#define\s+%s\s+(\d+)" % name, header).group(1)) == getattr(_lib, name)
