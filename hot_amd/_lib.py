@@ -26,7 +26,7 @@ STREAM_GX, STREAM_GW, STREAM_W, STREAM_ACT = 0, 1, 2, 3
 HOT_STATIC_MAX_CHANNELS = 16384
 
 EXPORTS = (
-    "hot_last_error", "hot_abi_version", "hot_kpad", "hot_hq_rowwise", "hot_hla_tokenwise",
+    "hot_last_error", "hot_abi_version", "hot_backward_streams", "hot_kpad", "hot_hq_rowwise", "hot_hla_tokenwise",
     "hot_wq_colwise", "hot_colwise_workspace_bytes", "hot_gemm_i8", "hot_abc_workspace_bytes",
     "hot_abc_forward", "hot_backward_workspace_bytes", "hot_linear_backward", "hot_linear_backward_kernels",
     "hot_gemm_splits", "hot_hla_workspace_bytes", "hot_linear_backward_bias",
@@ -48,6 +48,7 @@ class HotConfig(C.Structure):
         ("gx_scale", C.c_int32), ("w_scale", C.c_int32), ("gw_scale", C.c_int32), ("act_scale", C.c_int32),
         ("seed", C.c_uint64),
         ("hla_rows_big", C.POINTER(C.c_int32)),
+        ("streams", C.c_int32), ("reserved", C.c_int32),
     ]
 
 
@@ -65,6 +66,8 @@ def _declare(lib):
     lib.hot_last_error.argtypes = []
     lib.hot_abi_version.restype = i32
     lib.hot_abi_version.argtypes = []
+    lib.hot_backward_streams.restype = i32
+    lib.hot_backward_streams.argtypes = [i64, i64, i64, cfgp]
     lib.hot_kpad.restype = i64
     lib.hot_kpad.argtypes = [i64]
     lib.hot_hq_rowwise.restype = i32

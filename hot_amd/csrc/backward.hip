@@ -6,7 +6,6 @@
 // low-rank -> GEMM x2 -> dequantise) with the numerics of FLinearQ.backward,
 // scheme gih_gwlr (utils/quant_matmul.py:215-348).  hot_abc_forward is the
 // forward-side activation buffer of FLinearQ.setup_context (:178-212).
-#include <stdlib.h>
 #include <string.h>
 
 #include <mutex>
@@ -41,6 +40,7 @@ static int check_cfg(const hot_config* c, const char* who) {
   if (c->hla_n < 1 || c->hla_n > HOT_MAX_HLA_BIG || (c->hla_n & (c->hla_n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: hla_n=%d (power of two up to %d)", who, c->hla_n, HOT_MAX_HLA_BIG);
   if (c->hla_n > HOT_MAX_HLA_N && !c->hla_rows_big) return fail(HOT_ERR_INVALID, "%s: hla_n=%d needs hla_rows_big", who, c->hla_n);
   if (c->hla_r < 1 || c->hla_r > c->hla_n) return fail(HOT_ERR_INVALID, "%s: hla_r=%d outside [1, %d]", who, c->hla_r, c->hla_n);
+  if (c->streams < 0 || c->streams > 2) return fail(HOT_ERR_INVALID, "%s: streams=%d (0 = the library's rule, 1 or 2)", who, c->streams);
   const int bits[4] = {c->gx_bits, c->w_bits, c->gw_bits, c->act_bits};
   for (int i = 0; i < 4; ++i)
     if (bits[i] != 4 && bits[i] != 8) return fail(HOT_ERR_UNSUPPORTED, "%s: quantiser width %d (4 or 8)", who, bits[i]);
@@ -94,6 +94,18 @@ __global__ void clear3_kernel(uint32_t* p0, int n0, uint32_t* p1, int n1, uint32
   if (i < n2) p2[i] = 0u;
 }
 
+// One stream or two.  Forking and joining the side stream costs the host three event record / wait
+// pairs, about 60 us on top of the 23 us the ten launches take (measured); that is hidden only when
+// the kernels of the call run longer than it.  Calls with little arithmetic (both products together
+// below 30 GOP: ViT-B proj at 12608 tokens, 23 GOP, runs 75 us on one stream against 85 us with the
+// side stream; qkv, 70 GOP, 123 against 108) keep everything on the caller's stream.
+static int backward_streams(int64_t L, int64_t O, int64_t I, const hot_config* c) {
+  if (c->streams == 1 || c->streams == 2) return c->streams;
+  const double lp = (double)((L / c->hla_n) * c->hla_r);
+  const double ops = 2.0 * (double)O * (double)I * ((double)L + lp);
+  return ops < 3.0e10 ? 1 : 2;
+}
+
 static const int32_t* identity_rows() {
   struct Rows { int32_t v[HOT_MAX_HLA_N]; Rows() { for (int i = 0; i < HOT_MAX_HLA_N; ++i) v[i] = i; } };
   static const Rows rows;   // initialised once, thread-safe
@@ -108,6 +120,10 @@ extern "C" {
 
 const char* hot_last_error(void) { return g_err; }
 int hot_abi_version(void) { return HOT_ABI_VERSION; }
+int hot_backward_streams(int64_t L, int64_t O, int64_t I, const hot_config* cfg) {
+  if (check_cfg(cfg, "hot_backward_streams") || L <= 0 || O <= 0 || I <= 0) return 0;
+  return backward_streams(L, O, I, cfg);
+}
 int64_t hot_kpad(int64_t k) { return round_up(k, GEMM_KTILE); }
 
 int hot_gemm_splits(int64_t M, int64_t N, int64_t K, int bits) {
@@ -296,8 +312,7 @@ static int run_backward(const void* gy, const void* w, int dtype, const void* xq
   // beside the g_y statistics.
   std::unique_lock<std::mutex> side_guard(g_side_mutex, std::defer_lock);
   SideLane* side = nullptr;
-  static const bool sw_serial = [] { const char* v = getenv("HOT_SERIAL"); return v && *v == '1'; }();   // developer switch
-  if (!ev && !sw_serial) {
+  if (!ev && backward_streams(L, O, I, cfg) == 2) {
     side_guard.lock();
     side = side_lane_locked();
     if (!side) side_guard.unlock();

@@ -74,6 +74,7 @@ class HotOptions:
     gw_scale: int = SCALE_TENSOR
     act_scale: int = SCALE_TENSOR
     seed: int = 0
+    streams: int = 0      # launch order of the backward: 0 = the library's rule, 1 = one stream, 2 = with its side stream
 
     @property
     def hla_r(self) -> int:
@@ -121,6 +122,7 @@ class HotOptions:
         c.gx_scale, c.w_scale, c.gw_scale, c.act_scale = (_SCALE[self.gx_scale], _SCALE[self.w_scale],
                                                           _SCALE[self.gw_scale], _SCALE[self.act_scale])
         c.seed = int(self.seed) & 0xFFFFFFFFFFFFFFFF
+        c.streams = int(self.streams)
         return c
 
 
@@ -323,6 +325,11 @@ def linear_backward(gy: torch.Tensor, w: torch.Tensor, xq: torch.Tensor, sx: tor
     if timing:
         return gx, gw, [float(t) for t in times]
     return gx, gw
+
+
+def backward_streams(L: int, O: int, I: int, opt: HotOptions) -> int:
+    """1 or 2: the launch order linear_backward takes for this shape (hot_backward_streams)."""
+    return int(_lib.lib().hot_backward_streams(int(L), int(O), int(I), C.byref(opt.to_c())))
 
 
 def kpad_group(T: int, opt: HotOptions) -> int:

@@ -93,9 +93,18 @@ typedef struct hot_config {
                                   in the same kernels as smaller ones; from 256 on
                                   they take a two-level transform through an fp32
                                   workspace (launches only: capturable)          */
+  int32_t streams;  /* launch order of hot_linear_backward(_bias): 0 = the library's rule
+                       (hot_backward_streams), 1 = every kernel on the caller's stream, 2 =
+                       independent kernels also on the library's side stream (forked and joined by
+                       events).  The results do not depend on it.                               */
+  int32_t reserved; /* 0 */
 } hot_config;
 
 HOT_API const char* hot_last_error(void);
+/* 1 or 2: the launch order hot_linear_backward takes for this shape (cfg->streams when it is 1 or 2).
+ * Short calls, whose kernels take less time than the host needs for the event operations that fork
+ * and join the side stream, run on one stream; long ones overlap their independent kernels. */
+HOT_API int hot_backward_streams(int64_t L, int64_t O, int64_t I, const hot_config* cfg);
 HOT_API int hot_abi_version(void);
 
 /* Bytes of the leading dimension (row pitch) the library uses for a K-major

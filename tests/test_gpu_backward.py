@@ -501,13 +501,39 @@ def test_backward_errors(gpu):
         ops.abc_forward(x.to(gpu)[:100].contiguous(), opt)                               # L % n
 
 
-def test_backward_in_hip_graph(gpu):
-    """The whole call (main stream + the library's side stream, joined by events) is capturable;
-    every replay, with eager work in between, equals the eager result."""
+def test_backward_launch_orders_agree(gpu):
+    """hot_backward_streams: short calls run on the caller's stream, long ones fork the library's side
+    stream; cfg.streams overrides the rule; both orders give the same bits, bias gradient included."""
+    from dataclasses import replace
+    from hot_amd import ops
+    L, O, I = 1344, 384, 192
+    x, w, gy = make_case(L, O, I, seed=12, dtype=torch.bfloat16)
+    _, opt = both_configs(L)
+    assert ops.backward_streams(L, O, I, opt) == 1                                   # 0.3 GOP
+    assert ops.backward_streams(12608, 768, 768, opt) == 1 and ops.backward_streams(12608, 2304, 768, opt) == 2
+    assert ops.backward_streams(L, O, I, replace(opt, streams=2)) == 2
+    assert ops.backward_streams(12608, 3072, 768, replace(opt, streams=1)) == 1
+    with pytest.raises(ops.HotError, match="streams"):
+        ops.linear_backward(gy.to(gpu), w.to(gpu), *ops.abc_forward(x.to(gpu), opt), replace(opt, streams=3))
+    x, w, gy = x.to(gpu), w.to(gpu), gy.to(gpu)
+    xq, sx = ops.abc_forward(x, opt)
+    for variant in (dict(), dict(gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW, gw_round=orc.ROUND_STOCH, seed=5)):
+        one = ops.linear_backward(gy, w, xq, sx, replace(opt, streams=1, **variant), bias_grad=True)
+        two = ops.linear_backward(gy, w, xq, sx, replace(opt, streams=2, **variant), bias_grad=True)
+        for a, b in zip(one, two):
+            assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("streams", [1, 2])
+def test_backward_in_hip_graph(gpu, streams):
+    """The whole call -- on the caller's stream alone, or with the library's side stream forked and
+    joined by events -- is capturable; every replay, with eager work in between, equals the eager result."""
+    from dataclasses import replace
     from hot_amd import ops
     L, O, I = 1344, 384, 192
     x, w, gy = make_case(L, O, I, seed=11, dtype=torch.bfloat16)
     _, opt = both_configs(L)
+    opt = replace(opt, streams=streams)
     x, w, gy = x.to(gpu), w.to(gpu), gy.to(gpu)
     xq, sx = ops.abc_forward(x, opt)
     ws = torch.empty(1 << 26, dtype=torch.uint8, device=gpu)
