@@ -21,6 +21,8 @@
 // stream under graph capture records it like any other call.
 // This is the exactness path for large blocks, not a tuned one: the input is read with scalar loads
 // and the coefficients make a round trip through HBM in fp32.
+#include <string.h>
+
 #include <algorithm>
 #include <memory>
 
@@ -244,12 +246,55 @@ __global__ void big_clear_kernel(float* stat, float* colmax, int64_t C, int32_t*
   if (i < n) tab[i] = -1;
 }
 
-// A piece of the row table, carried in the kernel arguments (under the 4 KiB a launch may carry):
-// natural row row[i] of a block is the visit[i]-th kept row in natural order and goes to output
-// coefficient slot[i].
+// The row table, built by ONE launch whose arguments carry the kept rows by value: up to 2304 rows
+// of 13 bits each (3744 bytes of the 4 KiB a launch may carry; larger selections go in pieces of that
+// size).  Entry of natural row i: its output coefficient (the position of i in the caller's list) in
+// the low half, its visit number (the rank of i among the kept rows in natural order, which numbers
+// the elements of stochastic rounding) in the high half; -1 for dropped rows (written by the clear
+// kernel).  The rank is counted on the device: thread k compares its row with every row of the call.
+constexpr int TAB_ROWS = 2304;
+struct TabRows { uint32_t packed[(TAB_ROWS * 13 + 31) / 32]; int32_t count; };
+__device__ __host__ inline int tab_row_get(const uint32_t* packed, int i) {
+  const int bit = i * 13, w = bit >> 5, sh = bit & 31;
+  uint32_t v = packed[w] >> sh;
+  if (sh > 19) v |= packed[w + 1] << (32 - sh);
+  return (int)(v & 0x1FFFu);
+}
+inline void tab_row_put(uint32_t* packed, int i, int row) {
+  const int bit = i * 13, w = bit >> 5, sh = bit & 31;
+  packed[w] |= (uint32_t)row << sh;
+  if (sh > 19) packed[w + 1] |= (uint32_t)row >> (32 - sh);
+}
+__global__ void __launch_bounds__(256) big_table_kernel(int32_t* tab, const TabRows p) {
+  // every workgroup marks the kept rows in a bitmap of the block's n <= 8192 natural rows; the rank
+  // of a row is the number of marks below it
+  __shared__ uint32_t s_map[8192 / 32];
+  __shared__ uint32_t s_below[8192 / 32];
+  const int tid = threadIdx.x;
+  s_map[tid] = 0u;
+  __syncthreads();
+  for (int j = tid; j < p.count; j += 256) {
+    const int row = tab_row_get(p.packed, j);
+    atomicOr(&s_map[row >> 5], 1u << (row & 31));
+  }
+  __syncthreads();
+  {
+    // marks in the words before word `tid` (256 words: a serial sum per thread is short)
+    uint32_t acc = 0;
+    for (int w = 0; w < tid; ++w) acc += (uint32_t)__popc(s_map[w]);
+    s_below[tid] = acc;
+  }
+  __syncthreads();
+  const int k = blockIdx.x * 256 + tid;
+  if (k >= p.count) return;
+  const int row = tab_row_get(p.packed, k);
+  const int rank = (int)(s_below[row >> 5] + (uint32_t)__popc(s_map[row >> 5] & ((1u << (row & 31)) - 1u)));
+  tab[row] = k | (rank << 16);
+}
+// selections of more than TAB_ROWS rows: the host ranks, the rows travel with their visit numbers
 constexpr int TAB_PIECE = 512;
 struct TabPiece { uint16_t row[TAB_PIECE], visit[TAB_PIECE], slot[TAB_PIECE]; int32_t count; };
-__global__ void big_table_kernel(int32_t* tab, const TabPiece p) {
+__global__ void big_table_piece_kernel(int32_t* tab, const TabPiece p) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < p.count) tab[p.row[i]] = (int32_t)p.slot[i] | ((int32_t)p.visit[i] << 16);
 }
@@ -401,16 +446,24 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
   const int64_t nclr = std::max<int64_t>(std::max<int64_t>(C, n), (int64_t)(STAT_BYTES / 4));
   hipLaunchKernelGGL(big_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat, a.colmax, C,
                      (int32_t*)(ws + b.off_tab), n);
-  for (int v0 = 0; v0 < r; v0 += TAB_PIECE) {
-    TabPiece piece;
-    piece.count = std::min(TAB_PIECE, r - v0);
-    for (int i = 0; i < piece.count; ++i) {
-      const int32_t row = sorted[(size_t)(v0 + i)];
-      piece.row[i] = (uint16_t)row;
-      piece.visit[i] = (uint16_t)(v0 + i);
-      piece.slot[i] = (uint16_t)slot_of[(size_t)row];
+  if (r <= TAB_ROWS) {
+    TabRows tr;
+    memset(&tr, 0, sizeof(tr));
+    tr.count = r;
+    for (int k = 0; k < r; ++k) tab_row_put(tr.packed, k, rows[k]);
+    hipLaunchKernelGGL(big_table_kernel, dim3((unsigned)((r + 255) / 256)), dim3(256), 0, st, (int32_t*)(ws + b.off_tab), tr);
+  } else {
+    for (int v0 = 0; v0 < r; v0 += TAB_PIECE) {
+      TabPiece piece;
+      piece.count = std::min(TAB_PIECE, r - v0);
+      for (int i = 0; i < piece.count; ++i) {
+        const int32_t row = sorted[(size_t)(v0 + i)];
+        piece.row[i] = (uint16_t)row;
+        piece.visit[i] = (uint16_t)(v0 + i);
+        piece.slot[i] = (uint16_t)slot_of[(size_t)row];
+      }
+      hipLaunchKernelGGL(big_table_piece_kernel, dim3(TAB_PIECE / 256), dim3(256), 0, st, (int32_t*)(ws + b.off_tab), piece);
     }
-    hipLaunchKernelGGL(big_table_kernel, dim3(TAB_PIECE / 256), dim3(256), 0, st, (int32_t*)(ws + b.off_tab), piece);
   }
   if (int rc = check_launch("big_table_kernel")) return rc;
   const dim3 g1((unsigned)gx, (unsigned)(R / 64));
