@@ -563,9 +563,12 @@ def main():
                                 # kernels launched one after the other: [us, fraction of the 8 TB/s or 5 POP/s peak]
                                 "kernels_serial": {r["key"]: [r["us"], r["frac"]] for r in ltable}}
         # the same layer at the reference's own low-rank rule for 8192 tokens (utils/hadamard_matmul.py:209-226:
-        # one block of n = 8192, r = 2080 kept sequencies; the two-level token-wise path)
+        # one block of n = 8192, r = 2080 kept sequencies; the two-level token-wise path), the kept rows
+        # listed run by run as the layer lists them (hot_amd.quant_matmul.token_rule)
         try:
+            from hot_amd.hadamard_matmul import run_major
             rn, rrow = hla_rows(Ll)
+            rrow = run_major(rrow)
             ropt = ops.HotOptions(n_o=16, hla_n=int(rn), hla_rows=tuple(int(v) for v in rrow))
             del lbufs, lws
             rsec, rbufs, rws = step_time(lw, lsets, ropt, max(5, a.steps // 5), max(2, a.warmup // 5))

@@ -46,6 +46,11 @@ struct BigArgs {
   int32_t nk;          // coefficients of a 64-run that some kept row needs
   uint64_t kmask;      // bit k: coefficient k is one of them
   uint8_t klist[64];   // the nk set bits of kmask in increasing order
+  // run-major row lists only (big_stage2_runs_kernel): which runs keep needed coefficient index kc
+  // (bit j of keep[kc]: natural row 64 j + klist[kc] is kept), and the output coefficient of its first
+  // kept row (kbase[kc]; kbase[nk] = r): its other kept rows follow in run order
+  uint32_t keep[64][4];
+  uint16_t kbase[65];
   float* stat;         // [0] absmax, [1] step, [2] clip; the absmax slots from word 64
   float* colmax;       // per-channel absmax (ROW)
   double* partial;     // SAWB: 2 doubles per workgroup
@@ -176,6 +181,12 @@ __global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
     for (int j = 0; j < M; ++j) v[j] = 0.f;
   }
   fwht<M>(v);
+  // every coefficient is complete here: without this the compiler sinks the last butterfly stage into
+  // the conditional code below and holds both stages' registers (a third more than the block itself)
+  if constexpr (PASS == 1 || SAWB) {
+#pragma unroll
+    for (int j = 0; j < M; ++j) asm volatile("" : "+v"(v[j]));
+  }
 
   if constexpr (PASS == 0) {
     float cmax = 0.f;
@@ -236,6 +247,136 @@ __global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
       }
       a.tmp[(blk * a.r + slot) * a.C + c] = (int8_t)q;
     }
+  }
+}
+
+// Quantise pass for row lists in "run-major" order: the kept rows sorted by (row % 64, row / 64).  The
+// order of the kept coefficients along K is the caller's (slot = position in its list) and means
+// nothing to the product that consumes them, as long as both operands use the same; in this order
+// the coefficients that one coefficient index k of the 64-point stage yields -- what a thread of
+// this pass computes -- are neighbours along K, so a workgroup (64 channels x KG consecutive
+// needed indices, one per wave) owns ONE contiguous K run of every channel: the codes are staged
+// in LDS as [channel][run] and leave K-major, straight into the GEMM operand.  No [K, C]
+// intermediate with its 64-byte stores, no transpose kernel.  The workgroup of a block's last
+// index group also clears the row padding behind the last block.
+constexpr int KG = 4;
+template <int M, int ROUND, bool SAWB>
+__global__ void __launch_bounds__(64 * KG, 2) big_stage2_runs_kernel(const BigArgs a, int8_t* __restrict__ out, int64_t ld_out, int groups) {
+  __shared__ __align__(16) uint8_t img[64][KG * M + 16];
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int64_t c0 = (int64_t)blockIdx.x * 64, c = c0 + lane;
+  const bool active = c < a.C;
+  const int64_t blk = blockIdx.y / groups;
+  const int grp = (int)(blockIdx.y - blk * groups);
+  const int kc = grp * KG + wave;                      // this wave's needed coefficient index
+  const bool has_k = kc < a.nk;
+  const int qmax = (1 << (a.bits - 1)) - 1;
+  // the workgroup's K run within the block: the outputs of its coefficient indices, in list order
+  const int k_hi = (grp + 1) * KG < a.nk ? (grp + 1) * KG : a.nk;
+  const int run0 = a.kbase[grp * KG], run_len = a.kbase[k_hi] - run0;
+  float d = 1.f, clip = 0.f;
+  if (a.mode == HOT_SCALE_ROW) d = (active ? a.colmax[c] : 0.f) / (float)qmax + 1e-11f;
+  else if (a.mode == HOT_SCALE_TENSOR) d = a.stat[0] / (float)qmax + 1e-11f;
+  else { d = a.stat[1] + 1e-11f; clip = a.stat[2]; }
+  const float rcp = 1.0f / d;
+  if (has_k) {
+    float v[M];
+    if (active) {
+      const float* t = a.T + ((blk * M) * a.nk + kc) * a.C + c;
+#pragma unroll
+      for (int j = 0; j < M; ++j) v[j] = t[(int64_t)j * a.nk * a.C];
+    } else {
+#pragma unroll
+      for (int j = 0; j < M; ++j) v[j] = 0.f;
+    }
+    fwht<M>(v);
+    // every coefficient is complete here: without this the compiler sinks the last butterfly stage into
+    // the conditional code below and holds both stages' registers (a third more than the block itself)
+#pragma unroll
+    for (int j = 0; j < M; ++j) asm volatile("" : "+v"(v[j]));
+    // which runs keep this coefficient index: a bit mask in the kernel arguments, the same for every
+    // lane of the wave, so the walk below branches on scalar registers and a kept coefficient's place
+    // in the run is a running count (the list is run-major: this index's outputs are neighbours)
+    const int k = a.klist[kc];
+    int pos = __builtin_amdgcn_readfirstlane((int)a.kbase[kc] - run0);
+    uint32_t kw[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) kw[w] = __builtin_amdgcn_readfirstlane(a.keep[kc][w]);
+#pragma unroll
+    for (int j = 0; j < M; ++j) {
+      if (!((kw[j >> 5] >> (j & 31)) & 1u)) continue;
+      float x = v[j];
+      if constexpr (SAWB) x = fminf(fmaxf(x, -clip), clip);
+      int q;
+      if constexpr (ROUND == HOT_ROUND_NEAREST) {
+        q = (int)rint_div_fast(x, d, rcp);      // bit for bit rintf(x / d)
+      } else {
+        const int visit = a.tab[j * 64 + k] >> 16;
+        const uint64_t idx = ((uint64_t)c * (uint64_t)a.NB + (uint64_t)blk) * (uint64_t)a.rpad + (uint64_t)visit;
+        q = q_stoch_fix(x, rcp * 65536.0f, bits_of(idx, a.seed, a.stream), qmax);
+      }
+      img[lane][pos++] = (uint8_t)(q & 0xFF);
+    }
+  }
+  __syncthreads();
+  // flush: bytes [blk r + run0, + run_len) of every channel's row, dword by dword on the dwords of
+  // the destination (its first and last dword may belong to the run only in part)
+  const int nch = (int)((a.C - c0) < 64 ? (a.C - c0) : 64);
+  if (run_len > 0) {
+    const int64_t b0 = blk * a.r + run0, b1 = b0 + run_len;          // byte range within the row
+    const int64_t w0 = b0 >> 2, w1 = (b1 + 3) >> 2;                  // destination dwords [w0, w1)
+    const int nw = (int)(w1 - w0);
+    for (int i = tid; i < nch * nw; i += 64 * KG) {
+      const int rch = i / nw;
+      const int64_t w = w0 + (i - rch * nw);
+      int8_t* dst = out + (c0 + rch) * ld_out + w * 4;
+      const int off = (int)(w * 4 - b0);                              // position of the dword's first byte in the run
+      if (off >= 0 && off + 4 <= run_len) {
+        const uint8_t* src = &img[rch][off];
+        const uint32_t word = (uint32_t)src[0] | ((uint32_t)src[1] << 8) | ((uint32_t)src[2] << 16) | ((uint32_t)src[3] << 24);
+        *reinterpret_cast<uint32_t*>(dst) = word;
+      } else {
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          if (off + t >= 0 && off + t < run_len) dst[t] = (int8_t)img[rch][off + t];
+      }
+    }
+  }
+  if (blk == a.NB - 1 && grp == groups - 1) {
+    const int64_t k_end = a.NB * a.r;
+    const int pad = (int)(ld_out - k_end);
+    for (int i = tid; i < nch * pad; i += 64 * KG) {
+      const int rch = i / pad;
+      out[(c0 + rch) * ld_out + k_end + (i - rch * pad)] = 0;
+    }
+  }
+}
+
+template <int M>
+int launch_runs(const BigArgs& a, void* out, int64_t ld_out, hipStream_t st) {
+  const int groups = (a.nk + KG - 1) / KG;
+  const dim3 grid((unsigned)((a.C + 63) / 64), (unsigned)(a.NB * groups));
+  const bool sawb = a.mode == HOT_SCALE_SAWB, stoch = a.rounding == HOT_ROUND_STOCH;
+  if (stoch) {
+    if (sawb) hipLaunchKernelGGL((big_stage2_runs_kernel<M, 1, true>), grid, dim3(64 * KG), 0, st, a, (int8_t*)out, ld_out, groups);
+    else hipLaunchKernelGGL((big_stage2_runs_kernel<M, 1, false>), grid, dim3(64 * KG), 0, st, a, (int8_t*)out, ld_out, groups);
+  } else {
+    if (sawb) hipLaunchKernelGGL((big_stage2_runs_kernel<M, 0, true>), grid, dim3(64 * KG), 0, st, a, (int8_t*)out, ld_out, groups);
+    else hipLaunchKernelGGL((big_stage2_runs_kernel<M, 0, false>), grid, dim3(64 * KG), 0, st, a, (int8_t*)out, ld_out, groups);
+  }
+  return check_launch("big_stage2_runs_kernel");
+}
+
+int dispatch_runs(int m, const BigArgs& a, void* out, int64_t ld_out, hipStream_t st) {
+  switch (m) {
+    case 4: return launch_runs<4>(a, out, ld_out, st);
+    case 8: return launch_runs<8>(a, out, ld_out, st);
+    case 16: return launch_runs<16>(a, out, ld_out, st);
+    case 32: return launch_runs<32>(a, out, ld_out, st);
+    case 64: return launch_runs<64>(a, out, ld_out, st);
+    case 128: return launch_runs<128>(a, out, ld_out, st);
+    default: return fail(HOT_ERR_UNSUPPORTED, "hla: block size %d (64 m with m a power of two, 4 .. 128)", 64 * m);
   }
 }
 
@@ -490,6 +631,24 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
   if (int rc = dispatch_stage2(m, a, g2, 0, st)) return rc;
   hipLaunchKernelGGL(big_finalize_kernel, dim3(1), dim3(256), 0, st, a, (int64_t)gx * NB * a.nk, kout);
   if (after_stats) (void)hipEventRecord(after_stats, st);
+  // rows listed run-major (sorted by (row % 64, row / 64)): the quantise pass stores K-major itself
+  bool run_major = NB * ((a.nk + KG - 1) / KG) <= 65535;
+  for (int k = 1; k < r && run_major; ++k) {
+    const int prev = (rows[k - 1] & 63) * m + (rows[k - 1] >> 6), cur = (rows[k] & 63) * m + (rows[k] >> 6);
+    run_major = cur > prev;
+  }
+  if (run_major) {
+    memset(a.keep, 0, sizeof(a.keep));
+    memset(a.kbase, 0, sizeof(a.kbase));
+    int kc = -1, last_k = -1;
+    for (int i = 0; i < r; ++i) {
+      const int k = rows[i] & 63, j = rows[i] >> 6;
+      if (k != last_k) { ++kc; last_k = k; a.kbase[kc] = (uint16_t)i; }
+      a.keep[kc][j >> 5] |= 1u << (j & 31);
+    }
+    for (int q = kc + 1; q <= 64; ++q) a.kbase[q] = (uint16_t)r;
+    return dispatch_runs(m, a, codes_out, ld_out, st);
+  }
   if (int rc = dispatch_stage2(m, a, g2, 1, st)) return rc;
   const dim3 gt((unsigned)((ld_out + 63) / 64), (unsigned)((C + 63) / 64));
   hipLaunchKernelGGL(transpose_i8_kernel, gt, dim3(256), 0, st, a.tmp, kout, C, (int8_t*)codes_out, ld_out);

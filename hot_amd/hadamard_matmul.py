@@ -100,6 +100,15 @@ def hla_rows(size_m: int, percentile: float = 50) -> Tuple[int, np.ndarray]:
     return n, _hla_rows_cached(int(n), float(percentile))
 
 
+def run_major(rows) -> np.ndarray:
+    """The same kept rows listed by (row % 64, row // 64).  The order of the kept coefficients is the
+    order of the codes along K of both operands of the g_W product and does not show in its result; in
+    this order the coefficients that one coefficient index of the 64-point stage of the two-level
+    token-wise path yields are neighbours, and its quantise pass stores them K-major itself."""
+    rows = np.asarray(rows)
+    return rows[np.lexsort((rows // 64, rows % 64))]
+
+
 def paper_rows(n: int = 16, r: int = 8) -> Tuple[int, np.ndarray]:
     """The r lowest sequencies of an n-block (utils/analysis_calculator.py:174-175)."""
     return n, np.argsort(_sequency(n), kind="stable")[:r]

@@ -32,7 +32,7 @@ from torch.autograd.function import Function
 from . import args
 from . import ops
 from .hadamard_matmul import (Transform_Dict, biggest_power2_factor, biggest_power2_factor_max16, hla_rows,
-                              paper_rows)
+                              paper_rows, run_major)
 
 TD = Transform_Dict()
 
@@ -81,6 +81,10 @@ def token_rule(tokens: int):
     n, rows = hla_rows(tokens, args.vectorPercentile)
     if n > args.hla_max_block:
         n, rows = hla_rows(args.hla_max_block, args.vectorPercentile)
+    if n > 128:
+        # the two-level kernels store the codes themselves when the rows come run by run; the order along
+        # K is shared by the activation buffer and the gradient operand and cancels in their product
+        rows = run_major(rows)
     return n, rows
 
 

@@ -251,10 +251,15 @@ def test_llama_layers_full_size_reference_rule(gpu, O, I):
     widths.  Steps of the whole tensors, every code of the activation buffer and of (P g_y)^T, g_W and
     g_x on sampled rows and columns that touch every output tile."""
     from hot_amd import ops
+    from hot_amd.hadamard_matmul import run_major
     L = 8192
     x, w, gy, heavy = llama_inputs(L, O, I, seed=O + I + 1)
     ocfg = orc.HotConfig.python_rule(L)
     assert (ocfg.hla_n, len(ocfg.hla_rows)) == (8192, 2080)
+    if O == 11008:
+        # gate/up with the rows run by run, as the layers list them for large blocks (the K order of both
+        # g_W operands; g_W itself does not depend on it); down with the reference's sequency order
+        ocfg.hla_rows = tuple(int(v) for v in run_major(ocfg.hla_rows))
     opt = options_pair(ocfg)
     xd, wd, gyd = x.to(gpu), w.to(gpu), gy.to(gpu)
     xq, sx = ops.abc_forward(xd, opt)

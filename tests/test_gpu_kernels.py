@@ -502,6 +502,44 @@ def test_hla_tokenwise_large_blocks(gpu, n, L, C, scale, rounding, dtype):
     assert np.array_equal(got[:, :kout], q_ref) and not got[:, kout:].any()
 
 
+@pytest.mark.parametrize("n,L,C,scale,rounding,dtype", [
+    (256, 768, 200, "tensor", "nearest", torch.float32),          # three blocks, ragged channel strip, run lengths not multiples of 4
+    (256, 512, 64, "sawb", "stoch", torch.bfloat16),
+    (1024, 2048, 136, "row", "stoch", torch.float32),
+    (2048, 2048, 72, "tensor", "nearest", torch.float16),
+    (8192, 8192, 80, "tensor", "stoch", torch.bfloat16),
+])
+def test_hla_tokenwise_large_blocks_run_major(gpu, n, L, C, scale, rounding, dtype):
+    """The kept rows listed run by run (sorted by (row % 64, row // 64): hadamard_matmul.run_major, what the
+    layers pass for blocks above 128 tokens): the quantise pass of the two-level path then stores K-major
+    itself.  Codes in the caller's order, steps, zero padding and the numbering of stochastic rounding
+    (by natural row, whatever the order of the list) equal the one-pass oracle; the same rows in the
+    reference's sequency order give the same codes, permuted."""
+    from hot_amd import ops
+    from hot_amd.hadamard_matmul import run_major
+    _, rows_seq = orc.hla_rows(n)
+    rows = run_major(rows_seq)
+    assert sorted(rows.tolist()) == sorted(rows_seq.tolist()) and not np.array_equal(rows, rows_seq)
+    x = (torch.randn(L, C, generator=torch.Generator().manual_seed(n + C)) * 0.5).to(dtype)
+    mode = {"tensor": orc.SCALE_TENSOR, "row": orc.SCALE_ROW, "sawb": orc.SCALE_SAWB}[scale]
+    rnd = orc.ROUND_STOCH if rounding == "stoch" else orc.ROUND_NEAREST
+    tt = np.ascontiguousarray(orc.fwht_blocks_first(x.float().numpy(), n, rows).T)      # [C, L']
+    q_ref, s_ref = orc.quant(tt, 8, mode, rnd, seed=3, stream=orc.STREAM_GW,
+                             index=orc.colwise_rng_index(C, L // n, rows))
+    codes, s, kout = ops.hla_tokenwise(x.to(gpu), n, list(rows), bits=8, rounding=rounding, scale=scale, seed=3)
+    got = codes.cpu().numpy()
+    assert kout == tt.shape[1]
+    assert np.array_equal(s.cpu().numpy(), np.atleast_1d(s_ref).astype(np.float32).reshape(-1))
+    assert np.array_equal(got[:, :kout], q_ref) and not got[:, kout:].any()
+    # the sequency order: the general path (codes through the workspace and a transpose), same codes permuted
+    codes2, s2, _ = ops.hla_tokenwise(x.to(gpu), n, list(rows_seq), bits=8, rounding=rounding, scale=scale, seed=3)
+    pos = {int(v): i for i, v in enumerate(rows)}
+    perm = np.array([pos[int(v)] for v in rows_seq])
+    r = len(rows)
+    got2 = codes2.cpu().numpy()[:, :kout].reshape(C, L // n, r)
+    assert np.array_equal(got2, got[:, :kout].reshape(C, L // n, r)[:, :, perm]) and torch.equal(s, s2)
+
+
 @pytest.mark.parametrize("bits,rounding,dtype", [(8, "stoch", torch.bfloat16), (4, "nearest", torch.float32)])
 def test_hla_tokenwise_block128_any_selection(gpu, bits, rounding, dtype):
     """A 128-token block with a selection that is not the make_WHT one (table read at run time),
