@@ -27,6 +27,7 @@ Prints ONE JSON line.  Besides the contract fields it carries
   quantiser_grid the step over bits x rounding x step granularity x low-rank setting
   measure_py    the reference's latency harness (cuda_measure/measure.py) on the drop-in op
   vit_b16       whole-model backward with every layer swapped
+  forward_gemm  the plain bf16 forward product at the layer shapes: vendor library beside hot_gemm_bf16
 This run uses one GPU; --gpus above 1 is refused.
 """
 from __future__ import annotations
@@ -325,6 +326,29 @@ def layer_table(dev, steps=30, warmup=8):
             "rows": rows, "note": "%d steps after %d warm-ups, inputs rotated" % (steps, warmup)}
 
 
+def forward_gemm_table(dev):
+    """The plain bf16 linear layer y = x W^T + b (utils/quant_matmul.py:173-176) at the layer shapes:
+    torch's F.linear (the vendor library) beside hot_gemm_bf16, the same product through the data path
+    of this library's integer kernels.  Decides whether the forward product is worth owning (it would
+    have to be, for the activation buffer's statistics pass to move into its prologue)."""
+    import torch
+    import torch.nn.functional as F
+    from hot_amd import ops
+    rows = []
+    for name, L, O, I in (("vit_qkv", 12608, 2304, 768), ("vit_proj", 12608, 768, 768), ("vit_fc1", 12608, 3072, 768),
+                          ("vit_fc2", 12608, 768, 3072), ("llama_gate_up", 8192, 11008, 4096), ("llama_down", 8192, 4096, 11008)):
+        g = torch.Generator(device=dev).manual_seed(7)
+        x = torch.randn(L, I, device=dev, generator=g).bfloat16()
+        w = (torch.randn(O, I, device=dev, generator=g) * 0.03).bfloat16()
+        b = torch.randn(O, device=dev, generator=g).bfloat16()
+        vendor = _events(lambda: F.linear(x, w, b), 20, 5)
+        own = _events(lambda: ops.gemm_bf16(x, w, b), 20, 5)
+        rows.append([name, L, O, I, round(vendor, 1), round(own, 1), round(own / vendor, 2)])
+        del x, w, b
+    return {"columns": ["layer", "L", "O", "I", "vendor_us", "hot_gemm_bf16_us", "ratio"], "rows": rows,
+            "note": "bf16, bias added in the epilogue of both; 20 calls after 5 warm-ups"}
+
+
 def measure_py(dev, trials=100):
     """The reference's latency harness (cuda_measure/measure.py:35-80) on the drop-in op: L = 49 tokens,
     O = 3072, I = 768, lognormal(1, 0.1) inputs (numpy seed 2023), `trials` trials, medians.  As there:
@@ -580,7 +604,8 @@ def main():
             out["llama_gate_up_python_rule"] = {"error": repr(e)[:200]}
         del lw, lsets
     if not a.no_extras and not a.table_only:
-        for key, fn in (("layers", lambda: layer_table(dev)), ("measure_py", lambda: measure_py(dev))):
+        for key, fn in (("layers", lambda: layer_table(dev)), ("measure_py", lambda: measure_py(dev)),
+                        ("forward_gemm", lambda: forward_gemm_table(dev))):
             try:
                 out[key] = fn()
             except Exception as e:          # extras never cost the headline line

@@ -30,7 +30,7 @@ EXPORTS = (
     "hot_wq_colwise", "hot_colwise_workspace_bytes", "hot_gemm_i8", "hot_abc_workspace_bytes",
     "hot_abc_forward", "hot_backward_workspace_bytes", "hot_linear_backward", "hot_linear_backward_kernels",
     "hot_gemm_splits", "hot_hla_workspace_bytes", "hot_linear_backward_bias",
-    "hot_gemm_plan", "hot_gemm_workspace_bytes", "hot_gemm_i8_variant",
+    "hot_gemm_plan", "hot_gemm_workspace_bytes", "hot_gemm_i8_variant", "hot_gemm_bf16",
     "hot_hla_tokenwise_static", "hot_measure_ceilings",
     "hot_kpad_group", "hot_abc_batched_workspace_bytes", "hot_abc_forward_batched",
     "hot_backward_batched_workspace_bytes", "hot_linear_backward_batched", "hot_backward_batched_ranges",
@@ -103,6 +103,8 @@ def _declare(lib):
     lib.hot_gemm_i8_variant.restype = i32
     lib.hot_gemm_i8_variant.argtypes = [vp, i64, vp, i64, i32, i64, i64, i64, vp, i32, vp, fp, vp, i32, i64, vp,
                                         i32, vp, sz, vp]
+    lib.hot_gemm_bf16.restype = i32
+    lib.hot_gemm_bf16.argtypes = [vp, i64, vp, i64, i64, i64, i64, vp, vp, i32, i64, i32, vp]
     lib.hot_hla_tokenwise_static.restype = i32
     lib.hot_hla_tokenwise_static.argtypes = [vp, i32, i64, i64, i32, C.POINTER(C.c_int32), i32, i32, i32, u64, u32,
                                              i32, vp, i64, vp, vp]

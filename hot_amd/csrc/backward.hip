@@ -173,6 +173,11 @@ int hot_gemm_i8(const void* A, int64_t lda, const void* B, int64_t ldb, int bits
                       ldo, acc_out, (hipStream_t)hip_stream);
 }
 
+int hot_gemm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                  const void* bias, void* out, int out_dtype, int64_t ldo, int variant, void* hip_stream) {
+  return gemm_bf16_impl(A, lda, B, ldb, M, N, K, bias, out, out_dtype, ldo, (hipStream_t)hip_stream, variant);
+}
+
 int hot_gemm_plan(int64_t M, int64_t N, int64_t K, int bits, int64_t lda, int64_t ldb, size_t workspace_bytes) {
   return gemm_plan_impl(M, N, K, bits, lda, ldb, workspace_bytes);
 }

@@ -44,6 +44,7 @@ struct GemmArgs {
   int32_t a_per_row;
   void* out;
   int64_t ldo;
+  const void* bias;  // 16-bit floating operands only (BITS = 16): NULL or N elements of the output type, added per column
   int32_t* acc_out;
   int32_t tiles_m, tiles_n;
   int32_t group_m;   // tile rows per group of the launch order (tile_of)
@@ -135,6 +136,24 @@ __device__ __forceinline__ void load_row_scales(const GemmArgs& g, int64_t row_b
   }
 }
 
+// Output value of one accumulator register.  Integer codes: ((float(acc) * s_a) * s_b) * post_scale
+// (packed INT4 accumulates 256 x the product).  BITS = 16 (bf16 operands): the register holds the
+// fp32 sum itself, and `bias` (the column's bias, 0 without one) is added.
+template <int BITS>
+__device__ __forceinline__ float acc_value(int a, float sa, float sb, float post, float bias) {
+  if constexpr (BITS == 16) return __builtin_bit_cast(float, a) + bias;
+  if constexpr (BITS == 4) a >>= 8;
+  return (((float)a * sa) * sb) * post;
+}
+template <typename OutT> __device__ __forceinline__ float bias_at(const void* bias, int64_t col);
+template <> __device__ __forceinline__ float bias_at<float>(const void* bias, int64_t col) { return bias ? reinterpret_cast<const float*>(bias)[col] : 0.f; }
+template <> __device__ __forceinline__ float bias_at<bf16_t>(const void* bias, int64_t col) {
+  return bias ? as_f((uint32_t)reinterpret_cast<const uint16_t*>(bias)[col] << 16) : 0.f;
+}
+template <> __device__ __forceinline__ float bias_at<f16_t>(const void* bias, int64_t col) {
+  return bias ? (float)reinterpret_cast<const _Float16*>(bias)[col] : 0.f;
+}
+
 template <int WM, int WN, int BITS, typename OutT>
 __device__ __forceinline__ void gemm_epilogue(const v16i (&acc)[WM][WN], const GemmArgs& g, int64_t row_base,
                                               int64_t col_base, int lane, const float (&sa_row)[WM], float sb) {
@@ -152,25 +171,26 @@ __device__ __forceinline__ void gemm_epilogue(const v16i (&acc)[WM][WN], const G
         const int64_t col = col_base + j * 32 + 8 * q + 4 * half;
         if (col >= g.N) continue;
         int a[4];
+        float bv[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           a[t] = acc[i][j][4 * q + t];
-          if constexpr (BITS == 4) a[t] >>= 8;
+          if constexpr (BITS == 16) bv[t] = col + t < g.N ? bias_at<OutT>(g.bias, col + t) : 0.f;
         }
         if (g.acc_out) {
 #pragma unroll
           for (int t = 0; t < 4; ++t)
-            if (col + t < g.N) g.acc_out[row * g.N + col + t] = a[t];
+            if (col + t < g.N) g.acc_out[row * g.N + col + t] = BITS == 4 ? a[t] >> 8 : a[t];
         }
         if (g.vec_out && col + 3 < g.N) {
           typename Quad<OutT>::type v;
 #pragma unroll
-          for (int t = 0; t < 4; ++t) quad_set<OutT>(v, t, (((float)a[t] * sa) * sb) * g.post_scale);
+          for (int t = 0; t < 4; ++t) quad_set<OutT>(v, t, acc_value<BITS>(a[t], sa, sb, g.post_scale, bv[t]));
           *reinterpret_cast<typename Quad<OutT>::type*>(out + row * g.ldo + col) = v;
         } else {
 #pragma unroll
           for (int t = 0; t < 4; ++t)
-            if (col + t < g.N) store_scalar<OutT>(out + row * g.ldo + col + t, (((float)a[t] * sa) * sb) * g.post_scale);
+            if (col + t < g.N) store_scalar<OutT>(out + row * g.ldo + col + t, acc_value<BITS>(a[t], sa, sb, g.post_scale, bv[t]));
         }
       }
     }
@@ -313,9 +333,9 @@ __device__ __forceinline__ void gemm_epilogue_staged(const v16i (&acc)[WM][WN], 
         quad_t v;
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-          int a = acc[i][j][4 * q + t];
-          if constexpr (BITS == 4) a >>= 8;
-          quad_set<OutT>(v, t, (((float)a * sa) * sb) * g.post_scale);
+          float bv = 0.f;     // (the staged epilogue runs on whole tiles only: every column exists)
+          if constexpr (BITS == 16) bv = bias_at<OutT>(g.bias, col_base + j * 32 + 8 * q + 4 * half + t);
+          quad_set<OutT>(v, t, acc_value<BITS>(acc[i][j][4 * q + t], sa, sb, g.post_scale, bv));
         }
         *reinterpret_cast<quad_t*>(area + m * PITCH + (j * 32 + 8 * q + 4 * half) * (int)sizeof(OutT)) = v;
       }
@@ -634,6 +654,7 @@ gemm_i8_pipe_kernel(const GemmArgs g) {
 // spare KiB, so that every wave issues the same number of loads and one vmcnt serves all.
 // ---------------------------------------------------------------------------
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 
 template <int WM, int WN, int GM, int GN, int BITS, int S, int RB, typename OutT>
 __global__ void __launch_bounds__(G_THREADS) __attribute__((amdgpu_waves_per_eu(1, (WM * WN <= 8 ? 2 : 1))))
@@ -650,11 +671,11 @@ gemm_i8_slot_kernel(const GemmArgs g) {
   constexpr int RING_BYTES = S * STAGE_BYTES + (SPARE ? 1024 : 0);
   static_assert(S >= 2 && RING_BYTES <= 160 * 1024, "two or more LDS stages within 160 KiB");
   constexpr int NF = WM * WN;                       // accumulator fragments per wave
-  constexpr int NM = NF * (BITS == 8 ? 1 : 2);      // MFMAs (slots) per round
+  constexpr int NM = NF * (BITS == 4 ? 2 : 1);      // MFMAs (slots) per round
   constexpr int NR = WM + WN;                       // fragment reads per round
   constexpr int H = NM / 2;                         // slots per half round
   constexpr int DPS = (LPW + NM - 1) / NM;          // DMA instructions per slot of the refilling round
-  static_assert(NR <= H || BITS == 8, "the reads of a round fit the first half of the round before");
+  static_assert(NR <= H || BITS != 4, "the reads of a round fit the first half of the round before");
   __shared__ __attribute__((aligned(1024))) uint8_t ring[RING_BYTES];
 
   const int tid = threadIdx.x, lane = tid & 63;
@@ -663,12 +684,16 @@ gemm_i8_slot_kernel(const GemmArgs g) {
   int tm, tn;
   tile_of(g, (int)blockIdx.x, tm, tn);
   const int64_t row0 = (int64_t)tm * BM, col0 = (int64_t)tn * BN;
-  constexpr bool EARLY_SCALES = NF <= 4;
+  constexpr bool EARLY_SCALES = NF <= 4 && BITS != 16;
   float sa_row[WM];
   float sb = 0.f;
   if constexpr (EARLY_SCALES) {
     load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
     sb = g.scale_b[0];
+  }
+  if constexpr (BITS == 16) {
+#pragma unroll
+    for (int i = 0; i < WM; ++i) sa_row[i] = 1.f;
   }
 
   // LDS stage layout: rows of RB bytes = SPR slots of 16 bytes; logical slot s of row r sits at
@@ -749,7 +774,12 @@ gemm_i8_slot_kernel(const GemmArgs g) {
   // MFMA m of a round of parity p
   auto mfma_slot = [&](int p, int m) {
     const int mm = m % NF, i = mm / WN, j = mm % WN;
-    if constexpr (BITS == 8) {
+    if constexpr (BITS == 16) {
+      // bf16 operands: the same 16 bytes per lane are eight bf16 of K, the accumulator registers hold fp32
+      acc[i][j] = __builtin_bit_cast(v16i, __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                               __builtin_bit_cast(v8bf, fr[p][b_of(j)]), __builtin_bit_cast(v8bf, fr[p][a_of(i)]),
+                                               __builtin_bit_cast(v16f, acc[i][j]), 0, 0, 0));
+    } else if constexpr (BITS == 8) {
       acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fr[p][b_of(j)], fr[p][a_of(i)], acc[i][j], 0, 0, 0);
     } else {
       if (m < NF) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(lo[p][b_of(j)], lo[p][a_of(i)], acc[i][j], 0, 0, 0);
@@ -835,7 +865,7 @@ gemm_i8_slot_kernel(const GemmArgs g) {
   for (; kt0 + 2 * S - 1 < KT; kt0 += S) rotation(std::true_type{}, kt0);   // every tile inside has a tile kt + S
   for (; kt0 < KT; kt0 += S) rotation(std::false_type{}, kt0);
 
-  if constexpr (!EARLY_SCALES) {
+  if constexpr (!EARLY_SCALES && BITS != 16) {
     load_row_scales<WM>(g, row0 + wm * WM * 32, lane, sa_row);
     sb = g.scale_b[0];
   }
@@ -1320,7 +1350,7 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
   g.A = (const uint8_t*)A; g.B = (const uint8_t*)B; g.lda = lda; g.ldb = ldb; g.M = M; g.N = N;
   g.ktiles = (int)(kpad / G_BK);
   g.scale_a = scale_a; g.scale_b = scale_b; g.post_scale = post_scale; g.a_per_row = a_per_row;
-  g.out = out; g.ldo = ldo; g.acc_out = acc_out;
+  g.out = out; g.ldo = ldo; g.acc_out = acc_out; g.bias = nullptr;
   g.vec_out = ((ldo & 3) == 0 && ((uintptr_t)out & 15) == 0) ? 1 : 0;
   g.vec16 = (((uintptr_t)out & 15) == 0 && ((ldo * (out_dtype == HOT_F32 ? 4 : 2)) & 15) == 0) ? 1 : 0;
   g.splits = 1; g.partials = nullptr;
@@ -1334,6 +1364,54 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
     g.partials = (v4i*)split_ws;
   }
   return bits == 4 ? dispatch_out<4>(out_dtype, variant, g, st) : dispatch_out<8>(out_dtype, variant, g, st);
+}
+
+// out[M, N] = A[M, K] . B[N, K]^T (+ bias[N]) on bf16 operands, fp32 accumulation
+// (v_mfma_f32_32x32x16_bf16), through the data path of the slot-scheduled integer kernels: a lane's 16
+// bytes of a stage row are eight bf16 of K instead of sixteen codes, nothing else changes.  The plain
+// linear layer y = x W^T + b of the forward pass (utils/quant_matmul.py:173-176, F.linear), built to
+// measure this data path against the vendor library at the layer shapes.
+int gemm_bf16_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                   const void* bias, void* out, int out_dtype, int64_t ldo, hipStream_t st, int variant) {
+  const char* who = "hot_gemm_bf16";
+  if (!A || !B || !out) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
+  if (M < 0 || N < 0 || K <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape %lld x %lld x %lld", who, (long long)M, (long long)N, (long long)K);
+  if (K % G_BK) return fail(HOT_ERR_UNSUPPORTED, "%s: K=%lld must be a multiple of %d", who, (long long)K, G_BK);
+  if (lda < 2 * K || ldb < 2 * K || (lda & 15) || (ldb & 15))
+    return fail(HOT_ERR_INVALID, "%s: row pitches (%lld, %lld) are in bytes: multiples of 16, at least %lld", who, (long long)lda, (long long)ldb, (long long)(2 * K));
+  if (((uintptr_t)A & 15) || ((uintptr_t)B & 15)) return fail(HOT_ERR_INVALID, "%s: operands must be 16-byte aligned", who);
+  if (ldo < N) return fail(HOT_ERR_INVALID, "%s: ldo=%lld < N", who, (long long)ldo);
+  if (M * lda >= (1ll << 32) || N * ldb >= (1ll << 32)) return fail(HOT_ERR_UNSUPPORTED, "%s: operands of 4 GiB or more", who);
+  if (M == 0 || N == 0) return HOT_OK;
+  GemmArgs g;
+  g.A = (const uint8_t*)A; g.B = (const uint8_t*)B; g.lda = lda; g.ldb = ldb; g.M = M; g.N = N;
+  g.ktiles = (int)(K / G_BK);
+  g.scale_a = nullptr; g.scale_b = nullptr; g.post_scale = 1.0f; g.a_per_row = 0;
+  g.out = out; g.ldo = ldo; g.acc_out = nullptr; g.bias = bias;
+  g.vec_out = ((ldo & 3) == 0 && ((uintptr_t)out & 15) == 0) ? 1 : 0;
+  g.vec16 = (((uintptr_t)out & 15) == 0 && ((ldo * (out_dtype == HOT_F32 ? 4 : 2)) & 15) == 0) ? 1 : 0;
+  g.splits = 1; g.partials = nullptr;
+  g.groups = 0; g.group_stages = 0; g.gsplits = 1; g.gper = 0; g.gscale_a = nullptr; g.gscale_b = nullptr; g.gpart = nullptr; g.ldp = 0;
+  if (variant == HOT_GEMM_AUTO) {
+    // the 160 x 256 tile where it gives one balanced round (as for the integer products), else 256 x 256
+    // while it fills the chip, else 128 x 128
+    const int64_t t256 = ((M + 255) / 256) * ((N + 255) / 256);
+    const int64_t t160 = ((M + 159) / 160) * ((N + 255) / 256);
+    variant = (t160 <= 256 && t160 > t256) ? HOT_GEMM_SLOT_160X256 : (t256 >= 192 ? HOT_GEMM_SLOT_256 : HOT_GEMM_SLOT_128);
+  }
+#define HOT_BF16_CASE(OUT)                                                                                     \
+  switch (variant) {                                                                                           \
+    case HOT_GEMM_SLOT_256: return launch_gemm_slot<4, 4, 2, 2, 16, 2, 128, OUT>(g, st);                       \
+    case HOT_GEMM_SLOT_128: return launch_gemm_slot<2, 2, 2, 2, 16, 4, 128, OUT>(g, st);                       \
+    case HOT_GEMM_SLOT_160X256: return launch_gemm_slot<5, 2, 1, 4, 16, 2, 128, OUT>(g, st);                   \
+    default: return fail(HOT_ERR_UNSUPPORTED, "%s: kernel variant %d (the slot-scheduled kernels only)", who, variant); \
+  }
+  switch (out_dtype) {
+    case HOT_BF16: HOT_BF16_CASE(bf16_t)
+    case HOT_F32: HOT_BF16_CASE(float)
+    default: return fail(HOT_ERR_UNSUPPORTED, "%s: output type %d (bf16 or fp32)", who, out_dtype);
+  }
+#undef HOT_BF16_CASE
 }
 
 // INT8 product whose K dimension is `groups` samples of group_k codes each (a multiple of 128), every
@@ -1383,7 +1461,7 @@ int gemm_i8_grouped_impl(const void* A, int64_t lda, const void* B, int64_t ldb,
   g.A = (const uint8_t*)A; g.B = (const uint8_t*)B; g.lda = lda; g.ldb = ldb; g.M = M; g.N = N;
   g.ktiles = (int)(K / G_BK);
   g.scale_a = scale_a; g.scale_b = scale_b; g.post_scale = post_scale; g.a_per_row = a_per_row;
-  g.out = out; g.ldo = ldo; g.acc_out = nullptr;
+  g.out = out; g.ldo = ldo; g.acc_out = nullptr; g.bias = nullptr;
   g.vec_out = ((ldo & 3) == 0 && ((uintptr_t)out & 15) == 0) ? 1 : 0;
   g.vec16 = 0;
   g.splits = 1; g.partials = nullptr;

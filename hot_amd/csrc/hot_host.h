@@ -88,6 +88,8 @@ int gemm_i8_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int bit
                  int64_t K, const float* scale_a, int a_per_row, const float* scale_b, float post_scale,
                  void* out, int out_dtype, int64_t ldo, int32_t* acc_out, hipStream_t st, void* split_ws = nullptr,
                  size_t split_ws_bytes = 0, int variant = HOT_GEMM_AUTO);
+int gemm_bf16_impl(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t M, int64_t N, int64_t K,
+                   const void* bias, void* out, int out_dtype, int64_t ldo, hipStream_t st, int variant);
 // The hot_gemm_variant that gemm_i8_impl picks for a product when `ws_bytes` of workspace come with it.
 int gemm_plan_impl(int64_t M, int64_t N, int64_t K, int bits, int64_t lda, int64_t ldb, size_t ws_bytes);
 

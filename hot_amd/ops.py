@@ -222,6 +222,27 @@ def gemm_i8(a: torch.Tensor, b: torch.Tensor, k: int, bits: int, scale_a: torch.
     return (out, acc) if return_acc else out
 
 
+def gemm_bf16(a: torch.Tensor, b: torch.Tensor, bias: Optional[torch.Tensor] = None, out_dtype=torch.bfloat16,
+              variant: int = 0) -> torch.Tensor:
+    """out[M, N] = a[M, K] . b[N, K]^T (+ bias) on bf16 operands with fp32 accumulation (hot_gemm_bf16):
+    F.linear(a, b, bias) through the data path of the integer kernels.  K a multiple of 128."""
+    _need_gpu_2d(a, "A")
+    _need_gpu_2d(b, "B")
+    if a.dtype != torch.bfloat16 or b.dtype != torch.bfloat16:
+        raise RuntimeError("gemm_bf16 takes bf16 operands")
+    if a.stride(1) != 1 or b.stride(1) != 1 or a.shape[1] != b.shape[1]:
+        raise RuntimeError("gemm_bf16 takes K-major operands of one K")
+    M, K = a.shape
+    N = b.shape[0]
+    if bias is not None and (bias.dtype != out_dtype or bias.numel() != N or not bias.is_contiguous()):
+        raise RuntimeError("bias must hold N contiguous elements of the output type")
+    out = torch.empty((M, N), dtype=out_dtype, device=a.device)
+    _lib.check(_lib.lib().hot_gemm_bf16(a.data_ptr(), a.stride(0) * 2, b.data_ptr(), b.stride(0) * 2, M, N, K,
+                                        bias.data_ptr() if bias is not None else None, out.data_ptr(),
+                                        _DTYPES[out_dtype], N, int(variant), _stream()))
+    return out
+
+
 def _launch_stream(side: Optional["torch.cuda.Stream"]) -> int:
     return _stream() if side is None else side.cuda_stream
 

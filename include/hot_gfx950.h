@@ -189,6 +189,22 @@ HOT_API int hot_gemm_i8(const void* A, int64_t lda, const void* B, int64_t ldb, 
                 const float* scale_b, float post_scale, void* out, int out_dtype,
                 int64_t ldo, int32_t* acc_out, void* hip_stream);
 
+/*
+ * out[M, N] = A[M, K] . B[N, K]^T (+ bias[N]) on bf16 operands with fp32 accumulation: the plain
+ * linear layer of the forward pass, y = x W^T + b (utils/quant_matmul.py:173-176, F.linear), through
+ * the data path of the integer kernels (a lane's 16 bytes are eight bf16 of K).
+ *   A, B     device, bf16, K-major; row pitches lda, ldb in BYTES (multiples of 16, >= 2 K);
+ *            K a multiple of 128
+ *   bias     device, N elements of out_dtype, or NULL
+ *   out      device, [M, N] row-major of out_dtype (HOT_BF16 or HOT_F32), pitch ldo ELEMENTS
+ *   variant  HOT_GEMM_AUTO, HOT_GEMM_SLOT_128, HOT_GEMM_SLOT_256 or HOT_GEMM_SLOT_160X256
+ * The sums are added in the kernel's own order: the result equals the vendor library's to fp32
+ * rounding of a sum over K, not bit for bit.
+ */
+HOT_API int hot_gemm_bf16(const void* A, int64_t lda, const void* B, int64_t ldb, int64_t M, int64_t N,
+                  int64_t K, const void* bias, void* out, int out_dtype, int64_t ldo, int variant,
+                  void* hip_stream);
+
 /* Forward-side activation buffer: xq[I, hot_kpad(L')] = quant8(P x)^T, sx[1]. */
 HOT_API size_t hot_abc_workspace_bytes(int64_t L, int64_t I, const hot_config* cfg);
 HOT_API int hot_abc_forward(const void* x, int dtype, int64_t L, int64_t I, const hot_config* cfg,

@@ -461,6 +461,42 @@ def test_gemm_llama_products_sampled_rows_and_columns(gpu, bits, M, N, K, expect
     assert np.array_equal(out.cpu().numpy()[rows], dequant_ref(acc_rows, sa[rows], sb, 1 / 16))
 
 
+@pytest.mark.parametrize("M,N,K,bias,out_dtype", [
+    (200, 96, 128, True, torch.float32),        # ragged tiles, direct epilogue
+    (1000, 300, 384, False, torch.float32),     # 300 columns: four-wide stores across a ragged edge
+    (512, 512, 1024, True, torch.bfloat16),     # whole tiles: the LDS-staged epilogue
+    (12608, 768, 768, True, torch.bfloat16),    # ViT-B proj forward, the 160 x 256 tile
+])
+@pytest.mark.parametrize("variant", ["auto", "GEMM_SLOT_128", "GEMM_SLOT_256", "GEMM_SLOT_160X256"])
+def test_gemm_bf16_forward_product(gpu, M, N, K, bias, out_dtype, variant):
+    """hot_gemm_bf16 = x W^T + b (F.linear, utils/quant_matmul.py:173-176): bf16 operands are exact in
+    float64, so the float64 product is the reference; an fp32 sum over K terms in any order lies within
+    K 2^-24 sum|x w| of it (one rounding more for a bf16 output: 2^-8 relative)."""
+    from hot_amd import _lib, ops
+    g = torch.Generator().manual_seed(M + N + K)
+    x = torch.randn(M, K, generator=g).bfloat16()
+    w = (torch.randn(N, K, generator=g) * 0.05).bfloat16()
+    b = torch.randn(N, generator=g).to(out_dtype) if bias else None
+    v = 0 if variant == "auto" else getattr(_lib, variant)
+    y = ops.gemm_bf16(x.to(gpu), w.to(gpu), b.to(gpu) if bias else None, out_dtype=out_dtype, variant=v).cpu().double()
+    ref = x.double() @ w.double().T
+    mag = x.double().abs() @ w.double().abs().T
+    if bias:
+        ref = ref + b.double()
+        mag = mag + b.double().abs()
+    bound = K * 2.0 ** -24 * mag + (2.0 ** -8 * ref.abs() if out_dtype == torch.bfloat16 else 2.0 ** -23 * ref.abs())
+    assert torch.all((y - ref).abs() <= bound)
+
+
+def test_gemm_bf16_refuses_what_it_does_not_take(gpu):
+    from hot_amd import ops
+    x = torch.zeros(64, 100, device=gpu, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="multiple of 128"):
+        ops.gemm_bf16(x, x)
+    with pytest.raises(RuntimeError, match="bf16 operands"):
+        ops.gemm_bf16(x.float(), x.float())
+
+
 def test_gemm_splits_rule():
     """hot_gemm_splits: products with few output tiles and a long K are cut, others are not."""
     from hot_amd import _lib
