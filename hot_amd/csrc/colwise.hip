@@ -881,8 +881,8 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
                        bool stats_cleared, hipEvent_t after_stats, float* colsum_partial, int groups, int64_t kpad_group,
                        bool rowmajor) {
   if (!in || !codes_out || !scales_out || !rows) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
-  if (rowmajor && (groups > 1 || n > COL_MAX_N || scale_mode == HOT_SCALE_ROW || row16_absmax_out || colsum_partial))
-    return fail(HOT_ERR_UNSUPPORTED, "%s: the untransposed store takes token blocks up to %d, one step for the tensor, and no fused statistics", who, COL_MAX_N);
+  if (rowmajor && (groups > 1 || scale_mode == HOT_SCALE_ROW || row16_absmax_out || colsum_partial))
+    return fail(HOT_ERR_UNSUPPORTED, "%s: the untransposed store takes one step for the tensor and no fused statistics", who);
   if (R <= 0 || C <= 0) return fail(HOT_ERR_INVALID, "%s: bad shape R=%lld C=%lld", who, (long long)R, (long long)C);
   if (groups < 1) return fail(HOT_ERR_INVALID, "%s: %d sample groups", who, groups);
   if (groups > 1) {
@@ -893,7 +893,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
   }
   if (n > COL_MAX_N) {
     // blocks one thread cannot hold: the two-level path
-    if (store4) return fail(HOT_ERR_UNSUPPORTED, "%s: blocks above %d tokens have no packed-INT4 store", who, COL_MAX_N);
+    if (store4 && !rowmajor) return fail(HOT_ERR_UNSUPPORTED, "%s: blocks above %d tokens have no transposed packed-INT4 store", who, COL_MAX_N);
     if (R % n) return fail(HOT_ERR_INVALID, "%s: R=%lld is not a multiple of the block %d", who, (long long)R, n);
     if (r < 1 || r > n) return fail(HOT_ERR_INVALID, "%s: r=%d outside [1, %d]", who, r, n);
     if (bits != 4 && bits != 8) return fail(HOT_ERR_UNSUPPORTED, "%s: bits=%d (4 or 8)", who, bits);
@@ -910,7 +910,7 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
       }
     }
     return hla_big_impl(in, dtype, R, C, n, rows, r, bits, rounding, seed, rng_stream, scale_mode, codes_out, ld_out,
-                        scales_out, workspace, workspace_bytes, st, who, after_stats, row16_absmax_out);
+                        scales_out, workspace, workspace_bytes, st, who, after_stats, row16_absmax_out, rowmajor, store4);
   }
   if (n < 1 || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (a power of two)", who, n);
   if (R % n) return fail(HOT_ERR_INVALID, "%s: R=%lld is not a multiple of the block %d", who, (long long)R, n);

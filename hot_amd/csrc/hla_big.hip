@@ -39,7 +39,8 @@ constexpr size_t STAT_BYTES = 256 + STAT_SLOT_BYTES;   // [0] absmax, [1] step, 
 struct BigArgs {
   const void* in;
   float* T;            // [R, C] fp32 coefficients of the 64-point stage
-  int8_t* tmp;         // [Kout, C] codes before the transpose
+  int8_t* tmp;         // [Kout, tmp_ld] codes before the transpose (or the untransposed destination itself)
+  int64_t tmp_ld;
   const int32_t* tab;  // per natural row of a block: slot | visit << 16, or -1 when dropped
   int64_t R, C, NB;    // NB = R / n blocks
   int32_t n, r, rpad, bits, rounding, mode;
@@ -245,7 +246,7 @@ __global__ void __launch_bounds__(BT) big_stage2_kernel(const BigArgs a) {
         const uint64_t idx = ((uint64_t)c * (uint64_t)a.NB + (uint64_t)blk) * (uint64_t)a.rpad + (uint64_t)visit;
         q = q_stoch_fix(x, rcp * 65536.0f, bits_of(idx, a.seed, a.stream), qmax);
       }
-      a.tmp[(blk * a.r + slot) * a.C + c] = (int8_t)q;
+      a.tmp[(blk * a.r + slot) * a.tmp_ld + c] = (int8_t)q;
     }
   }
 }
@@ -489,6 +490,122 @@ __global__ void __launch_bounds__(256) transpose_i8_kernel(const int8_t* __restr
   }
 }
 
+// two channels to a byte, the even channel in bits 3:0 (the untransposed packed-INT4 operand)
+__global__ void __launch_bounds__(256) pack4_rows_kernel(const int8_t* __restrict__ tmp, int64_t K, int64_t C,
+                                                         int8_t* __restrict__ out, int64_t ld) {
+  const int64_t half = C / 2;
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= K * half) return;
+  const int64_t k = i / half, b = i - k * half;
+  const int lo = tmp[k * C + 2 * b], hi = tmp[k * C + 2 * b + 1];
+  out[k * ld + b] = (int8_t)((lo & 0xF) | ((hi & 0xF) << 4));
+}
+
+// ---- expansion P^T t of large blocks (the schemes that project g_y along the tokens for the g_x product,
+// utils/quant_matmul.py:334-337) ---------------------------------------------------------------------
+// H_n is symmetric, so P^T t = H_n z with z = the r coefficients at their natural rows and zeros
+// elsewhere, through the canonical butterflies (stages h = 1, 2, ..., n / 2 on the natural row index):
+// the stages below 64 act inside the runs of 64 consecutive rows (pass A, thread = channel, one run),
+// the stages from 64 up across the runs at a fixed position (pass B, thread = channel, one position),
+// with the fp32 intermediate [n, C] per block in the workspace.  Pass B scales by `post` (exact: 1 / n).
+struct ExpandBigArgs {
+  const float* t;      // [NB r, C]
+  float* U;            // [NB n, C]
+  void* out;           // [NB n, C]
+  const int32_t* tab;  // per natural row: slot | visit << 16, or -1
+  int64_t C;
+  int32_t r, m;
+  float post;
+};
+
+__global__ void __launch_bounds__(BT) expand_runs_kernel(const ExpandBigArgs a) {
+  const int64_t c = (int64_t)blockIdx.x * BT + threadIdx.x;
+  if (c >= a.C) return;
+  const int64_t blk = blockIdx.y / a.m;
+  const int j = (int)(blockIdx.y - blk * a.m);
+  float v[64];
+#pragma unroll
+  for (int k = 0; k < 64; ++k) {
+    const int32_t e = a.tab[j * 64 + k];               // the same for every thread: a scalar load and branch
+    v[k] = e >= 0 ? a.t[(blk * a.r + (e & 0xFFFF)) * a.C + c] : 0.f;
+  }
+  fwht<64>(v);
+  float* u = a.U + ((blk * a.m + j) * 64) * a.C + c;
+#pragma unroll
+  for (int k = 0; k < 64; ++k) u[(int64_t)k * a.C] = v[k];
+}
+
+template <int M, typename OutT>
+__global__ void __launch_bounds__(BT) expand_across_kernel(const ExpandBigArgs a) {
+  const int64_t c = (int64_t)blockIdx.x * BT + threadIdx.x;
+  if (c >= a.C) return;
+  const int64_t blk = blockIdx.y / 64;
+  const int k = (int)(blockIdx.y - blk * 64);
+  const int64_t base = ((blk * M) * 64 + k) * a.C + c;
+  float v[M];
+#pragma unroll
+  for (int j = 0; j < M; ++j) v[j] = a.U[base + (int64_t)j * 64 * a.C];
+  fwht<M>(v);
+  OutT* out = reinterpret_cast<OutT*>(a.out);
+#pragma unroll
+  for (int j = 0; j < M; ++j) store_scalar<OutT>(out + base + (int64_t)j * 64 * a.C, v[j] * a.post);
+}
+
+template <int M>
+int launch_expand_across(const ExpandBigArgs& a, dim3 grid, int out_dtype, hipStream_t st) {
+  switch (out_dtype) {
+    case HOT_F32: hipLaunchKernelGGL((expand_across_kernel<M, float>), grid, dim3(BT), 0, st, a); break;
+    case HOT_BF16: hipLaunchKernelGGL((expand_across_kernel<M, bf16_t>), grid, dim3(BT), 0, st, a); break;
+    case HOT_F16: hipLaunchKernelGGL((expand_across_kernel<M, f16_t>), grid, dim3(BT), 0, st, a); break;
+    default: return fail(HOT_ERR_INVALID, "hla_expand: bad out dtype %d", out_dtype);
+  }
+  return check_launch("expand_across_kernel");
+}
+
+__global__ void tab_clear_kernel(int32_t* tab, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) tab[i] = -1;
+}
+
+// Checks the row list and writes the table of a block (every entry: the clear kernel's -1 or a kept
+// row's slot | visit << 16) with launches alone.
+int build_row_table(int32_t* tab, int n, const int32_t* rows, int r, uint64_t* kmask_out, hipStream_t st, const char* who) {
+  std::unique_ptr<int32_t[]> slot_of(new int32_t[(size_t)n]);
+  for (int i = 0; i < n; ++i) slot_of[(size_t)i] = -1;
+  uint64_t kmask = 0;
+  for (int k = 0; k < r; ++k) {
+    if (rows[k] < 0 || rows[k] >= n) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d outside [0, %d)", who, k, rows[k], n);
+    if (slot_of[(size_t)rows[k]] != -1) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d listed twice", who, k, rows[k]);
+    slot_of[(size_t)rows[k]] = k;
+    kmask |= 1ull << (rows[k] & 63);
+  }
+  if (kmask_out) *kmask_out = kmask;
+  if (r <= TAB_ROWS) {
+    TabRows tr;
+    memset(&tr, 0, sizeof(tr));
+    tr.count = r;
+    for (int k = 0; k < r; ++k) tab_row_put(tr.packed, k, rows[k]);
+    hipLaunchKernelGGL(big_table_kernel, dim3((unsigned)((r + 255) / 256)), dim3(256), 0, st, tab, tr);
+  } else {
+    // rows in natural order: the visit number of a piece's entry i is its position in the sorted list
+    std::unique_ptr<int32_t[]> sorted(new int32_t[(size_t)r]);
+    for (int k = 0; k < r; ++k) sorted[(size_t)k] = rows[k];
+    std::sort(sorted.get(), sorted.get() + r);
+    for (int v0 = 0; v0 < r; v0 += TAB_PIECE) {
+      TabPiece piece;
+      piece.count = std::min(TAB_PIECE, r - v0);
+      for (int i = 0; i < piece.count; ++i) {
+        const int32_t row = sorted[(size_t)(v0 + i)];
+        piece.row[i] = (uint16_t)row;
+        piece.visit[i] = (uint16_t)(v0 + i);
+        piece.slot[i] = (uint16_t)slot_of[(size_t)row];
+      }
+      hipLaunchKernelGGL(big_table_piece_kernel, dim3(TAB_PIECE / 256), dim3(256), 0, st, tab, piece);
+    }
+  }
+  return check_launch("big_table_kernel");
+}
+
 template <int M>
 int launch_stage2(const BigArgs& a, dim3 grid, int pass, hipStream_t st) {
   const bool sawb = a.mode == HOT_SCALE_SAWB, stoch = a.rounding == HOT_ROUND_STOCH;
@@ -542,11 +659,14 @@ size_t hla_big_workspace_bytes_impl(int64_t R, int64_t C, int n, int r) {
 int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r, int bits,
                  int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_out,
                  float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st, const char* who,
-                 hipEvent_t after_stats, float* row16_absmax_out) {
+                 hipEvent_t after_stats, float* row16_absmax_out, bool rowmajor, int store4) {
   const int m = n / 64;
   if (n < 256 || n > 8192 || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (a power of two, 256 .. 8192)", who, n);
   const int64_t NB = R / n, kout = NB * r;
-  if (ld_out < kout || (ld_out & 15)) return fail(HOT_ERR_INVALID, "%s: ld_out=%lld must be a multiple of 16 and >= %lld", who, (long long)ld_out, (long long)kout);
+  if (!rowmajor && store4) return fail(HOT_ERR_UNSUPPORTED, "%s: blocks above 128 tokens have no transposed packed-INT4 store", who);
+  if (store4 && (C & 1)) return fail(HOT_ERR_UNSUPPORTED, "%s: packed INT4 output needs an even number of channels", who);
+  const int64_t row_bytes = rowmajor ? (store4 ? C / 2 : C) : kout;
+  if (ld_out < row_bytes || (ld_out & 15)) return fail(HOT_ERR_INVALID, "%s: ld_out=%lld must be a multiple of 16 and >= %lld", who, (long long)ld_out, (long long)row_bytes);
   const BigLayout b = big_layout(R, C, n, r);
   if (!workspace || workspace_bytes < b.total) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, b.total, workspace_bytes);
   if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
@@ -554,27 +674,17 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
   if (R / 64 > 65535 || (scale_mode == HOT_SCALE_SAWB && gx * NB * 64 > 65536))
     return fail(HOT_ERR_UNSUPPORTED, "%s: %lld blocks of %d tokens x %lld channels exceed the grid of the large-block path", who, (long long)NB, n, (long long)C);
 
-  // visit number of every kept row (rank among the kept rows in natural order) and the coefficients
-  // of a 64-run that the selection needs at all
-  std::unique_ptr<int32_t[]> slot_of(new int32_t[(size_t)n]);
-  std::unique_ptr<int32_t[]> sorted(new int32_t[(size_t)r]);
-  for (int i = 0; i < n; ++i) slot_of[(size_t)i] = -1;
-  uint64_t kmask = 0;
-  for (int k = 0; k < r; ++k) {
-    if (rows[k] < 0 || rows[k] >= n) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d outside [0, %d)", who, k, rows[k], n);
-    if (slot_of[(size_t)rows[k]] != -1) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d listed twice", who, k, rows[k]);
-    slot_of[(size_t)rows[k]] = k;
-    sorted[(size_t)k] = rows[k];
-    kmask |= 1ull << (rows[k] & 63);
-  }
-  std::sort(sorted.get(), sorted.get() + r);
-
   uint8_t* ws = (uint8_t*)workspace;
   BigArgs a;
   a.in = in; a.T = (float*)(ws + b.off_T); a.tmp = (int8_t*)(ws + b.off_tmp); a.tab = (const int32_t*)(ws + b.off_tab);
   a.R = R; a.C = C; a.NB = NB; a.n = n; a.r = r; a.rpad = r == 1 ? 1 : (r + 7) & ~7; a.bits = bits; a.rounding = rounding;
   a.mode = scale_mode; a.stat = (float*)ws; a.colmax = (float*)(ws + b.off_colmax);
   a.partial = (double*)(ws + b.off_partial); a.scales_out = scales_out; a.seed = seed; a.stream = rng_stream;
+  a.tmp_ld = C;
+  // the row table (and with it the check of the row list), after the clear kernel below
+  uint64_t kmask = 0;
+  for (int k = 0; k < r; ++k)
+    if (rows[k] >= 0 && rows[k] < n) kmask |= 1ull << (rows[k] & 63);
   a.kmask = kmask; a.nk = 0;
   for (int k = 0; k < 64; ++k) {
     a.klist[k] = 0;
@@ -587,26 +697,7 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
   const int64_t nclr = std::max<int64_t>(std::max<int64_t>(C, n), (int64_t)(STAT_BYTES / 4));
   hipLaunchKernelGGL(big_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat, a.colmax, C,
                      (int32_t*)(ws + b.off_tab), n);
-  if (r <= TAB_ROWS) {
-    TabRows tr;
-    memset(&tr, 0, sizeof(tr));
-    tr.count = r;
-    for (int k = 0; k < r; ++k) tab_row_put(tr.packed, k, rows[k]);
-    hipLaunchKernelGGL(big_table_kernel, dim3((unsigned)((r + 255) / 256)), dim3(256), 0, st, (int32_t*)(ws + b.off_tab), tr);
-  } else {
-    for (int v0 = 0; v0 < r; v0 += TAB_PIECE) {
-      TabPiece piece;
-      piece.count = std::min(TAB_PIECE, r - v0);
-      for (int i = 0; i < piece.count; ++i) {
-        const int32_t row = sorted[(size_t)(v0 + i)];
-        piece.row[i] = (uint16_t)row;
-        piece.visit[i] = (uint16_t)(v0 + i);
-        piece.slot[i] = (uint16_t)slot_of[(size_t)row];
-      }
-      hipLaunchKernelGGL(big_table_piece_kernel, dim3(TAB_PIECE / 256), dim3(256), 0, st, (int32_t*)(ws + b.off_tab), piece);
-    }
-  }
-  if (int rc = check_launch("big_table_kernel")) return rc;
+  if (int rc = build_row_table((int32_t*)(ws + b.off_tab), n, rows, r, nullptr, st, who)) return rc;
   const dim3 g1((unsigned)gx, (unsigned)(R / 64));
   a.row_absmax = row16_absmax_out;
   if (row16_absmax_out && (C % 16 || scale_mode == HOT_SCALE_SAWB))
@@ -631,6 +722,18 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
   if (int rc = dispatch_stage2(m, a, g2, 0, st)) return rc;
   hipLaunchKernelGGL(big_finalize_kernel, dim3(1), dim3(256), 0, st, a, (int64_t)gx * NB * a.nk, kout);
   if (after_stats) (void)hipEventRecord(after_stats, st);
+  if (rowmajor) {
+    // untransposed [NB r, C]: the quantise pass writes the destination itself (INT8), or its [Kout, C]
+    // scratch, which a second kernel packs two channels to a byte
+    if (!store4) { a.tmp = (int8_t*)codes_out; a.tmp_ld = ld_out; }
+    if (int rc = dispatch_stage2(m, a, g2, 1, st)) return rc;
+    if (store4) {
+      const int64_t items = kout * (C / 2);
+      hipLaunchKernelGGL(pack4_rows_kernel, dim3((unsigned)((items + 255) / 256)), dim3(256), 0, st, a.tmp, kout, C, (int8_t*)codes_out, ld_out);
+      return check_launch("pack4_rows_kernel");
+    }
+    return HOT_OK;
+  }
   // rows listed run-major (sorted by (row % 64, row / 64)): the quantise pass stores K-major itself
   bool run_major = NB * ((a.nk + KG - 1) / KG) <= 65535;
   for (int k = 1; k < r && run_major; ++k) {
@@ -653,6 +756,40 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
   const dim3 gt((unsigned)((ld_out + 63) / 64), (unsigned)((C + 63) / 64));
   hipLaunchKernelGGL(transpose_i8_kernel, gt, dim3(256), 0, st, a.tmp, kout, C, (int8_t*)codes_out, ld_out);
   return check_launch("transpose_i8_kernel");
+}
+
+size_t hla_expand_big_workspace_bytes_impl(int64_t nb, int64_t C, int n) {
+  return (size_t)round_up((int64_t)n * 4, 256) + (size_t)round_up(nb * n * C * 4, 256);
+}
+
+int hla_expand_big_impl(const float* t, int64_t nb, int64_t C, int n, const int32_t* rows, int r, float post, void* out,
+                        int out_dtype, void* workspace, size_t workspace_bytes, hipStream_t st) {
+  const char* who = "hla_expand";
+  const int m = n / 64;
+  if (n < 256 || n > 8192 || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block size %d (a power of two, 256 .. 8192)", who, n);
+  if (r < 1 || r > n) return fail(HOT_ERR_INVALID, "%s: r=%d outside [1, %d]", who, r, n);
+  if (nb * m > 65535 || nb * 64 > 65535) return fail(HOT_ERR_UNSUPPORTED, "%s: %lld blocks of %d tokens exceed the grid", who, (long long)nb, n);
+  const size_t need = hla_expand_big_workspace_bytes_impl(nb, C, n);
+  if (!workspace || workspace_bytes < need) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, need, workspace_bytes);
+  if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
+  int32_t* tab = (int32_t*)workspace;
+  ExpandBigArgs a;
+  a.t = t; a.U = (float*)((uint8_t*)workspace + round_up((int64_t)n * 4, 256)); a.out = out; a.tab = tab; a.C = C;
+  a.r = r; a.m = m; a.post = post;
+  hipLaunchKernelGGL(tab_clear_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, st, tab, n);
+  if (int rc = build_row_table(tab, n, rows, r, nullptr, st, who)) return rc;
+  const unsigned gx = (unsigned)((C + BT - 1) / BT);
+  hipLaunchKernelGGL(expand_runs_kernel, dim3(gx, (unsigned)(nb * m)), dim3(BT), 0, st, a);
+  if (int rc = check_launch("expand_runs_kernel")) return rc;
+  const dim3 g2(gx, (unsigned)(nb * 64));
+  switch (m) {
+    case 4: return launch_expand_across<4>(a, g2, out_dtype, st);
+    case 8: return launch_expand_across<8>(a, g2, out_dtype, st);
+    case 16: return launch_expand_across<16>(a, g2, out_dtype, st);
+    case 32: return launch_expand_across<32>(a, g2, out_dtype, st);
+    case 64: return launch_expand_across<64>(a, g2, out_dtype, st);
+    default: return launch_expand_across<128>(a, g2, out_dtype, st);
+  }
 }
 
 }  // namespace hot

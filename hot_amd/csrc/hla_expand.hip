@@ -5,8 +5,9 @@
 // their natural rows and zeros elsewhere: the same canonical butterflies as every other transform
 // here (adding an exact zero changes no bit), then one exact scaling by 1 / n.
 //
-// A thread owns one channel; its column of the block lives in LDS ([n][256] floats, the thread's
-// own bank column, so no thread ever touches another's values and no barrier is needed).  Kept for
+// A thread owns one channel; its column of the block lives in LDS ([n][threads] floats, the thread's
+// own bank column, so no thread ever touches another's values and no barrier is needed; 256 threads
+// up to n = 64, 128 at n = 128: 64 KiB either way).  Larger blocks: hla_expand_big_impl.  Kept for
 // completeness of the reference's scheme list, not tuned: memory-bound work done at LDS speed.
 #include <hip/hip_runtime.h>
 
@@ -17,8 +18,8 @@
 
 namespace hot {
 
-constexpr int EXP_MAX_N = 64;
-constexpr int EXP_THREADS = 256;
+constexpr int EXP_MAX_N = 128;
+constexpr int EXP_THREADS = 256;   // (at most; the launch may use fewer)
 
 struct ExpandArgs {
   const float* t;      // [nb r, C]
@@ -31,23 +32,23 @@ struct ExpandArgs {
 
 template <typename OutT>
 __global__ void __launch_bounds__(EXP_THREADS) hla_expand_kernel(const ExpandArgs a) {
-  extern __shared__ float col[];                      // [n][EXP_THREADS]
-  const int tid = threadIdx.x;
-  const int64_t c = (int64_t)blockIdx.x * EXP_THREADS + tid;
+  extern __shared__ float col[];                      // [n][threads]
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int64_t c = (int64_t)blockIdx.x * nt + tid;
   const int64_t blk = blockIdx.y;
   if (c >= a.C) return;                               // no barriers below: a thread may leave alone
-  for (int i = 0; i < a.n; ++i) col[i * EXP_THREADS + tid] = 0.f;
+  for (int i = 0; i < a.n; ++i) col[i * nt + tid] = 0.f;
   const float* src = a.t + blk * a.r * a.C + c;
-  for (int k = 0; k < a.r; ++k) col[a.row[k] * EXP_THREADS + tid] = src[(int64_t)k * a.C];
+  for (int k = 0; k < a.r; ++k) col[a.row[k] * nt + tid] = src[(int64_t)k * a.C];
   for (int h = 1; h < a.n; h <<= 1)
     for (int i = 0; i < a.n; ++i)
       if ((i & h) == 0) {
-        const float x = col[i * EXP_THREADS + tid], y = col[(i + h) * EXP_THREADS + tid];
-        col[i * EXP_THREADS + tid] = x + y;
-        col[(i + h) * EXP_THREADS + tid] = x - y;
+        const float x = col[i * nt + tid], y = col[(i + h) * nt + tid];
+        col[i * nt + tid] = x + y;
+        col[(i + h) * nt + tid] = x - y;
       }
   OutT* dst = reinterpret_cast<OutT*>(a.out) + blk * a.n * a.C + c;
-  for (int i = 0; i < a.n; ++i) store_scalar<OutT>(dst + (int64_t)i * a.C, col[i * EXP_THREADS + tid] * a.post);
+  for (int i = 0; i < a.n; ++i) store_scalar<OutT>(dst + (int64_t)i * a.C, col[i * nt + tid] * a.post);
 }
 
 int hla_expand_impl(const float* t, int64_t nb, int64_t C, int n, const int32_t* rows, int r, float post,
@@ -66,8 +67,9 @@ int hla_expand_impl(const float* t, int64_t nb, int64_t C, int n, const int32_t*
     seen[rows[k]] = true;
     a.row[k] = (int8_t)rows[k];
   }
-  const dim3 grid((unsigned)((C + EXP_THREADS - 1) / EXP_THREADS), (unsigned)nb);
-  const size_t lds = (size_t)n * EXP_THREADS * sizeof(float);          // 64 KiB at n = 64
+  const int nt = n > 64 ? 128 : EXP_THREADS;
+  const dim3 grid((unsigned)((C + nt - 1) / nt), (unsigned)nb);
+  const size_t lds = (size_t)n * nt * sizeof(float);                   // 64 KiB at n = 64 and at n = 128
   static std::once_flag once;
   static hipError_t attr_err = hipSuccess;
   std::call_once(once, [] {
@@ -77,9 +79,9 @@ int hla_expand_impl(const float* t, int64_t nb, int64_t C, int n, const int32_t*
   });
   if (attr_err != hipSuccess) return check_hip(attr_err, "hipFuncSetAttribute(hla_expand_kernel)");
   switch (out_dtype) {
-    case HOT_F32: hipLaunchKernelGGL(hla_expand_kernel<float>, grid, dim3(EXP_THREADS), lds, st, a); break;
-    case HOT_BF16: hipLaunchKernelGGL(hla_expand_kernel<bf16_t>, grid, dim3(EXP_THREADS), lds, st, a); break;
-    case HOT_F16: hipLaunchKernelGGL(hla_expand_kernel<f16_t>, grid, dim3(EXP_THREADS), lds, st, a); break;
+    case HOT_F32: hipLaunchKernelGGL(hla_expand_kernel<float>, grid, dim3(nt), lds, st, a); break;
+    case HOT_BF16: hipLaunchKernelGGL(hla_expand_kernel<bf16_t>, grid, dim3(nt), lds, st, a); break;
+    case HOT_F16: hipLaunchKernelGGL(hla_expand_kernel<f16_t>, grid, dim3(nt), lds, st, a); break;
     default: return fail(HOT_ERR_INVALID, "%s: bad out dtype %d", who, out_dtype);
   }
   return check_launch("hla_expand_kernel");

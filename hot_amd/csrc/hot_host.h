@@ -55,9 +55,13 @@ int colwise_quant_impl(const void* in, int dtype, int64_t R, int64_t C, int n, c
 // channels of a row are left alone: zero_pad_impl clears them), one step for the tensor.
 void zero_pad_impl(void* codes, int64_t rows, int64_t row_bytes, int64_t ld, hipStream_t st);
 // out[NB n, C] = (P^T t) * post for t [NB r, C] fp32: the kept coefficients go back to their natural rows of
-// every block and the block is transformed again (H is symmetric); n up to 64.
+// every block and the block is transformed again (H is symmetric); n up to 128.
 int hla_expand_impl(const float* t, int64_t nb, int64_t C, int n, const int32_t* rows, int r, float post,
                     void* out, int out_dtype, hipStream_t st);
+// The same for blocks of 256 .. 8192 tokens: two passes with the fp32 intermediate in the workspace.
+int hla_expand_big_impl(const float* t, int64_t nb, int64_t C, int n, const int32_t* rows, int r, float post, void* out,
+                        int out_dtype, void* workspace, size_t workspace_bytes, hipStream_t st);
+size_t hla_expand_big_workspace_bytes_impl(int64_t nb, int64_t C, int n);
 // With groups > 1 the R rows are `groups` samples of equal length, each quantised with steps of its own
 // (scales_out: [groups], or [groups][C] with per-channel steps); the codes of sample g take the bytes
 // [g * kpad_group, (g + 1) * kpad_group) of every output row, zero-filled behind the sample's codes.
@@ -77,7 +81,10 @@ size_t colwise_stats_bytes_impl(int64_t C);  // leading part of the workspace th
 int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r, int bits,
                  int rounding, uint64_t seed, uint32_t rng_stream, int scale_mode, void* codes_out, int64_t ld_out,
                  float* scales_out, void* workspace, size_t workspace_bytes, hipStream_t st, const char* who,
-                 hipEvent_t after_stats = nullptr, float* row16_absmax_out = nullptr);
+                 hipEvent_t after_stats = nullptr, float* row16_absmax_out = nullptr, bool rowmajor = false,
+                 int store4 = 0);
+// rowmajor: the codes are stored untransposed, [NB r, C] with ld_out bytes per coefficient row (store4:
+// two channels to a byte).
 // row16_absmax_out (STAT_SLOTS partial maxima, zero before the call; C a multiple of 16, absmax steps):
 // stage 1 also delivers the absmax of the row-wise 16-point Hadamard of the input.
 size_t hla_big_workspace_bytes_impl(int64_t R, int64_t C, int n, int r);

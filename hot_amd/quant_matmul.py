@@ -19,7 +19,6 @@ from __future__ import annotations
 from typing import Optional, Tuple
 
 import threading
-import warnings
 from dataclasses import replace
 
 import numpy as np
@@ -89,27 +88,17 @@ def token_rule(tokens: int):
 
 
 LOWRANK_GX_SCHEMES = ("low_rank", "gilr_gwh")
-LOWRANK_GX_MAX_BLOCK = 64
-_LOWRANK_CAP_WARNED: set = set()
 
 
 def gx_token_rule(tokens: int):
     """(n, rows) of the projection P along the tokens that the schemes "low_rank" and "gilr_gwh" apply to
     g_y for the g_x product (utils/quant_matmul.py:229-233; P is make_WHT of the token count, :356-362):
-    the low-rank rule of args.hla_rule with blocks of at most 64 tokens (the expansion pass holds a block
-    per thread)."""
+    the low-rank rule of args.hla_rule, blocks of up to args.hla_max_block tokens as for the g_W side."""
     if args.hla_rule == "paper":
         return (1, np.array([0])) if tokens % 16 else paper_rows(16, 8)
     n, rows = hla_rows(tokens, args.vectorPercentile)
-    cap = min(int(args.hla_max_block), LOWRANK_GX_MAX_BLOCK)
-    if n > cap:
-        if n > LOWRANK_GX_MAX_BLOCK and tokens not in _LOWRANK_CAP_WARNED:
-            _LOWRANK_CAP_WARNED.add(tokens)
-            warnings.warn("transform scheme %r at %d tokens: the reference's rule gives token blocks of %d for the g_x "
-                          "projection; the native expansion pass takes blocks up to %d, so g_x is projected with "
-                          "n = %d and differs numerically from the reference's" %
-                          (args.transform_scheme, tokens, n, LOWRANK_GX_MAX_BLOCK, cap), stacklevel=2)
-        n, rows = hla_rows(cap, args.vectorPercentile)
+    if n > args.hla_max_block:
+        n, rows = hla_rows(args.hla_max_block, args.vectorPercentile)
     return n, rows
 
 
@@ -306,28 +295,48 @@ class FLinearQ(Function):
             # g_x by an entry point of its own -- the projection along the tokens and its expansion
             # ("low_rank", "gilr_gwh"), or the logarithmic quantiser on g_y --, g_W as in "gih_gwlr" /
             # "hadamard": the token-wise kernel on g_y, then the INT8 product
-            what = "quantBWDGogi luq" if luq else "transform scheme %r" % args.transform_scheme
-            if go.dim() == 3 and args.batched_mode == "per_sample":
-                raise NotImplementedError("%s takes 2-D activations or batched_mode \"flatten\"" % what)
+            # 3-D activations with a step per sample (the reference's vmap over the batch,
+            # utils/quant_matmul.py:79-83): one pass per sample, sample b seeded with seed + b, the weight
+            # gradients of the samples added in fp32 in sample order
             if luq and args.transform_scheme in LOWRANK_GX_SCHEMES:
                 raise NotImplementedError("quantBWDGogi luq runs with the schemes gih_gwlr and hadamard")
             if not luq and opt.gx_scale != ops.SCALE_TENSOR:
                 raise NotImplementedError("transform scheme %r: the projected g_y takes one step for the tensor "
                                           "(quantBWDGogi int or stoch)" % args.transform_scheme)
-            go2 = _pad8(go.reshape(-1, go.shape[-1]))
-            if luq:
-                gx = ops.gx_luq(go2, wc, opt)
-            else:
-                n_gx, rows_gx = gx_token_rule(go2.shape[0])
-                gx = ops.gx_lowrank(go2, wc, replace(opt, hla_n=int(n_gx), hla_rows=tuple(int(v) for v in rows_gx)))
-            qgp, sgp, lp = ops.hla_tokenwise(go2, opt.hla_n, opt.hla_rows, bits=opt.gw_bits,
-                                             rounding="stoch" if opt.gw_round == ops.ROUND_STOCH else "nearest",
-                                             scale="row" if opt.gw_scale == ops.SCALE_ROW else "tensor",
-                                             seed=opt.seed, rng_stream=ops.STREAM_GW)
-            # both operands hold one code per byte whatever their widths (the token-wise kernel and the
-            # activation buffer never pack): an INT8 product, as in the fused path
-            grad_w = ops.gemm_i8(qgp, xq, lp, 8, sgp, sx, post_scale=1.0 / opt.hla_n, out_dtype=wc.dtype)
-            grad_input = gx[:, :I].reshape(ctx.x_shape)
+            per_sample = go.dim() == 3 and args.batched_mode == "per_sample"
+            samples = [go[b] for b in range(go.shape[0])] if per_sample else [go.reshape(-1, go.shape[-1])]
+            gxs, gw = [], None
+            for b, g in enumerate(samples):
+                opt_b = replace(opt, seed=opt.seed + b) if b else opt
+                go2 = _pad8(g)
+                if luq:
+                    gx = ops.gx_luq(go2, wc, opt_b)
+                else:
+                    n_gx, rows_gx = gx_token_rule(go2.shape[0])
+                    gx = ops.gx_lowrank(go2, wc, replace(opt_b, hla_n=int(n_gx), hla_rows=tuple(int(v) for v in rows_gx)))
+                qgp, sgp, lp = ops.hla_tokenwise(go2, opt.hla_n, opt.hla_rows, bits=opt.gw_bits,
+                                                 rounding="stoch" if opt.gw_round == ops.ROUND_STOCH else "nearest",
+                                                 scale="row" if opt.gw_scale == ops.SCALE_ROW else "tensor",
+                                                 seed=opt_b.seed, rng_stream=ops.STREAM_GW)
+                if not per_sample:
+                    xq_b, sx_b = xq, sx
+                elif ctx.batched:
+                    # the batched buffer keeps the samples side by side along K; the product reads whole
+                    # 128-code stages, so the sample's codes move to a zero-padded operand of their own
+                    kg = ops.kpad_group(go2.shape[0], opt)
+                    xq_b = torch.zeros((xq.shape[0], ops.kpad(lp)), dtype=xq.dtype, device=xq.device)
+                    xq_b[:, :lp] = xq[:, b * kg:b * kg + lp]
+                    sx_b = sx[b:b + 1]
+                else:
+                    xq_b, sx_b = xq[b], sx[b:b + 1]
+                # both operands hold one code per byte whatever their widths (the token-wise kernel and the
+                # activation buffer never pack): an INT8 product, as in the fused path
+                gw_b = ops.gemm_i8(qgp, xq_b, lp, 8, sgp, sx_b, post_scale=1.0 / opt.hla_n,
+                                   out_dtype=torch.float32 if per_sample else wc.dtype)
+                gw = gw_b if gw is None else gw + gw_b
+                gxs.append(gx[:, :I])
+            grad_w = gw.to(wc.dtype)
+            grad_input = torch.stack(gxs) if per_sample else gxs[0].reshape(ctx.x_shape)
         elif go.dim() == 3 and args.batched_mode == "per_sample" and ctx.batched:
             gx, grad_w = ops.linear_backward_batched(_pad8(go), wc, xq, sx, opt)
             grad_input = gx[..., :I]

@@ -810,6 +810,11 @@ def test_hq_linear_scheme_hadamard(gpu, fresh_args, L):
     (512, 256, 128, "paper", dict(w_scale=orc.SCALE_SAWB)),                       # n = 16, r = 8
     (200, 40, 24, "python", dict(gx_round=orc.ROUND_STOCH, seed=4)),              # n = 8, one ragged strip
     (49, 64, 32, "python", dict()),                                               # n = 1: nothing projected
+    (384, 96, 72, "python", dict()),                                              # n = 128, r = 36: the widest block one thread holds
+    (640, 64, 40, "python", dict(gx_bits=8, w_bits=8, gx_round=orc.ROUND_STOCH, seed=5)),   # n = 128, five blocks
+    (768, 64, 40, "python", dict()),                                              # n = 256, r = 136: the two-level path, packed INT4
+    (2048, 48, 264, "python", dict(gx_bits=8, w_bits=8)),                         # n = 2048, two channel strips of the expansion
+    (3072, 32, 24, "python", dict(gx_round=orc.ROUND_STOCH, seed=9)),             # n = 1024, three blocks, stochastic
 ])
 def test_gx_lowrank_matches_oracle(gpu, dtype, L, O, I, rule, variant):
     """g_x of the schemes "low_rank" / "gilr_gwh" (hot_gx_lowrank): the projected g_y stored untransposed,
@@ -830,13 +835,13 @@ def test_gx_lowrank_refuses_what_it_cannot_do(gpu):
     with pytest.raises(ops.HotError, match="one step for the tensor"):
         ops.gx_lowrank(gy.to(gpu), w.to(gpu), opt)
     n, rows = orc.hla_rows(128)
-    big = ops.HotOptions(hla_n=n, hla_rows=tuple(int(v) for v in rows))
-    with pytest.raises(ops.HotError, match="token blocks up to 64"):
-        ops.gx_lowrank(gy.to(gpu), w.to(gpu), big)
+    odd = ops.HotOptions(hla_n=n, hla_rows=tuple(int(v) for v in rows))
+    with pytest.raises(ops.HotError, match="not a multiple of hla_n"):
+        ops.gx_lowrank(gy[:192].to(gpu), w.to(gpu), odd)
 
 
 @pytest.mark.parametrize("scheme", ["low_rank", "gilr_gwh"])
-@pytest.mark.parametrize("L", [448, 200])
+@pytest.mark.parametrize("L", [448, 200, 384, 512])
 def test_hq_linear_lowrank_gx_schemes(gpu, fresh_args, scheme, L):
     """transform_scheme "low_rank" (utils/quant_matmul.py:184-185,231-232,263-264,296-297,334-335) and
     "gilr_gwh" (:186-187,233-234,265-266,298-299,336-338) through HQ_Linear: g_x by projection along the
@@ -851,7 +856,7 @@ def test_hq_linear_lowrank_gx_schemes(gpu, fresh_args, scheme, L):
     gy = torch.randn(L, O, device=gpu) * 1e-3
     lin(x).backward(gy)
     xn, gyn, wn = x.detach().cpu().numpy(), gy.cpu().numpy(), lin.weight.detach().cpu().numpy()
-    n_lr, rows_lr = orc.hla_rows(L)                                      # 64 / 36 at 448, 8 / 5 at 200
+    n_lr, rows_lr = orc.hla_rows(L)                      # 64 / 36 at 448, 8 / 5 at 200, 128 / 36 at 384, 512 / 136 at 512
     cfg_gx = orc.HotConfig(hla_n=n_lr, hla_rows=tuple(int(v) for v in rows_lr))
     if scheme == "low_rank":
         cfg_gw = cfg_gx
@@ -932,9 +937,45 @@ def test_hq_linear_with_luq_on_the_gx_path(gpu, fresh_args):
     xq_ref, sx_ref = orc.abc_forward(xn, ocfg)
     assert np.array_equal(x.grad.cpu().numpy(), orc.gx_luq(gyn, wn, ocfg).g_x)
     assert np.array_equal(lin.weight.grad.cpu().numpy(), orc.linear_backward(gyn, wn, xq_ref, sx_ref, ocfg).g_w)
+
+
+@pytest.mark.parametrize("path,T", [("luq", 64), ("luq", 197), ("low_rank", 64), ("gilr_gwh", 48), ("low_rank", 256)])
+def test_hq_linear_3d_per_sample_on_the_separate_gx_paths(gpu, fresh_args, path, T):
+    """3-D activations with a step per sample (the reference's vmap over the batch,
+    utils/quant_matmul.py:79-83,118-122) through quantBWDGogi = "luq" and the schemes that project g_y
+    along the tokens: every sample is the 2-D case of its own tokens, sample b seeded with seed + b,
+    the weight gradients added in fp32 in sample order.  Against the oracle, sample by sample."""
+    from hot_amd.quant_matmul import HQ_Linear
+    B, I, O = 3, 96, 128
     fresh_args.batched_mode = "per_sample"
-    with pytest.raises(NotImplementedError):
-        lin(torch.randn(2, 64, I, device=gpu, requires_grad=True)).sum().backward()
+    if path == "luq":
+        fresh_args.quantBWDGogi = "luq"
+    else:
+        fresh_args.transform_scheme = path
+    torch.manual_seed(T)
+    lin = HQ_Linear(I, O, bias=False).to(gpu)
+    x = torch.randn(B, T, I, device=gpu, requires_grad=True)
+    gy = torch.randn(B, T, O, device=gpu) * 1e-3 * (10.0 ** torch.arange(B, device=gpu).float().view(B, 1, 1))
+    step = fresh_args.sr_step
+    lin(x).backward(gy)
+    wn = lin.weight.detach().cpu().numpy()
+    seed = (int(fresh_args.sr_seed) << 20) + step
+    n_lr, rows_lr = orc.hla_rows(T)
+    gxs, gw = [], None
+    for b in range(B):
+        cfg_gx = orc.HotConfig(hla_n=n_lr, hla_rows=tuple(int(v) for v in rows_lr), seed=seed + b)
+        if path == "gilr_gwh":
+            n16 = orc.pow2_factor_max16(T)
+            cfg_gw = orc.HotConfig(hla_n=n16, hla_rows=tuple(range(n16)), seed=seed + b)
+        else:
+            cfg_gw = cfg_gx
+        xn, gyn = x[b].detach().cpu().numpy(), gy[b].cpu().numpy()
+        xq_ref, sx_ref = orc.abc_forward(xn, cfg_gw)
+        gw_b = orc.linear_backward(gyn, wn, xq_ref, sx_ref, cfg_gw).g_w
+        gw = gw_b if gw is None else (gw + gw_b).astype(np.float32)
+        gxs.append(orc.gx_luq(gyn, wn, cfg_gx).g_x if path == "luq" else orc.gx_lowrank(gyn, wn, cfg_gx).g_x)
+    assert np.array_equal(x.grad.cpu().numpy(), np.stack(gxs))
+    assert np.array_equal(lin.weight.grad.cpu().numpy(), gw)
 
 
 def test_hq_linear_under_autocast_matches_the_inline_buffer_write(gpu, fresh_args):
