@@ -35,6 +35,7 @@ EXPORTS = (
     "hot_kpad_group", "hot_abc_batched_workspace_bytes", "hot_abc_forward_batched",
     "hot_backward_batched_workspace_bytes", "hot_linear_backward_batched", "hot_backward_batched_ranges",
     "hot_gx_lowrank_workspace_bytes", "hot_gx_lowrank", "hot_gx_luq_workspace_bytes", "hot_gx_luq",
+    "hot_gw_luq_workspace_bytes", "hot_gw_luq",
 )
 
 
@@ -124,6 +125,10 @@ def _declare(lib):
     lib.hot_gx_luq_workspace_bytes.argtypes = [i64, i64, i64, cfgp]
     lib.hot_gx_luq.restype = i32
     lib.hot_gx_luq.argtypes = [vp, vp, i32, i64, i64, i64, cfgp, vp, i32, vp, sz, vp]
+    lib.hot_gw_luq_workspace_bytes.restype = sz
+    lib.hot_gw_luq_workspace_bytes.argtypes = [i64, i64, i64, cfgp]
+    lib.hot_gw_luq.restype = i32
+    lib.hot_gw_luq.argtypes = [vp, i32, vp, vp, i64, i64, i64, cfgp, vp, i32, vp, sz, vp]
     lib.hot_backward_batched_ranges.restype = i32
     lib.hot_backward_batched_ranges.argtypes = [i64, i64, i64, i64, cfgp]
     lib.hot_linear_backward_batched.restype = i32

@@ -624,6 +624,78 @@ int hot_gx_luq(const void* gy, const void* w, int dtype, int64_t L, int64_t O, i
                       1.0f / (float)cfg->n_o, gx, out_dtype, I, nullptr, st);
 }
 
+// ---- g_W with the logarithmic quantiser on the projected g_y ------------------------------------------
+// quantBWDGogw = "luq", or luq_quantizer picked for a layer's g_W under quantAuto (utils/quant_matmul.py:
+// 296-301, 307-314, 322-324): g_W = (luq((P g_y)^T) . q(P x)) s s_x / n.  The projection is computed
+// unquantised in fp32 ([O, L'], rows padded with zeros to a multiple of 8: a zero draws code 0), the
+// quantiser runs on its rows (element e = o K8 + k draws the uniforms 2 e, 2 e + 1 of stream 5), and the
+// two planes of the codes (q = 16 a + b) meet the INT8 activation buffer in two products whose integer
+// sums a last kernel combines: 16 acc_a + acc_b is the exact sum of q x.  Kept for completeness.
+
+struct GwLuqLayout {
+  int64_t lp, k8, kp;
+  size_t off_slots, off_sg, off_proj, off_codes, off_acca, off_accb, total;
+};
+
+static GwLuqLayout gw_luq_layout(int64_t L, int64_t O, int64_t I, const hot_config* c) {
+  GwLuqLayout b;
+  b.lp = (L / c->hla_n) * c->hla_r;
+  b.k8 = round_up(b.lp, 8);
+  b.kp = round_up(b.lp, GEMM_KTILE);
+  size_t o = 0;
+  b.off_slots = o; o += STAT_SLOT_BYTES;
+  b.off_sg = o;    o += 256;
+  b.off_proj = o;  o += align256((size_t)O * b.k8 * 4);
+  b.off_codes = o; o += align256((size_t)O * 2 * b.kp);
+  b.off_acca = o;  o += align256((size_t)O * I * 4);
+  b.off_accb = o;  o += align256((size_t)O * I * 4);
+  b.total = o;
+  return b;
+}
+
+static int check_gw_luq(const hot_config* cfg, int64_t L, int64_t O, int64_t I, const char* who) {
+  if (int e = check_cfg(cfg, who)) return e;
+  if (L <= 0 || O <= 0 || I <= 0 || I % 8) return fail(HOT_ERR_INVALID, "%s: L=%lld, O=%lld and I=%lld must be positive, I a multiple of 8", who, (long long)L, (long long)O, (long long)I);
+  if (cfg->hla_n > 128) return fail(HOT_ERR_UNSUPPORTED, "%s: token blocks up to 128 (the projection pass holds a block per thread)", who);
+  if (L % cfg->hla_n) return fail(HOT_ERR_INVALID, "%s: L=%lld is not a multiple of hla_n=%d", who, (long long)L, cfg->hla_n);
+  if (cfg->gw_bits != 4) return fail(HOT_ERR_UNSUPPORTED, "%s: the logarithmic quantiser runs at 4 bits (gw_bits)", who);
+  if ((L / cfg->hla_n) * cfg->hla_r > 16384) return fail(HOT_ERR_UNSUPPORTED, "%s: more than 16384 coefficients per channel overflow the int32 sums", who);
+  return HOT_OK;
+}
+
+size_t hot_gw_luq_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_config* cfg) {
+  if (check_gw_luq(cfg, L, O, I, "hot_gw_luq_workspace_bytes")) return 0;
+  return gw_luq_layout(L, O, I, cfg).total;
+}
+
+int hot_gw_luq(const void* gy, int dtype, const void* xq, const float* sx, int64_t L, int64_t O, int64_t I,
+               const hot_config* cfg, void* gw, int out_dtype, void* workspace, size_t workspace_bytes, void* hip_stream) {
+  const char* who = "hot_gw_luq";
+  if (int e = check_gw_luq(cfg, L, O, I, who)) return e;
+  if (!gy || !xq || !sx || !gw) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
+  const GwLuqLayout b = gw_luq_layout(L, O, I, cfg);
+  if (!workspace || workspace_bytes < b.total) return fail(HOT_ERR_WORKSPACE, "%s: workspace of %zu bytes needed, %zu given", who, b.total, workspace_bytes);
+  if ((uintptr_t)workspace & 255) return fail(HOT_ERR_INVALID, "%s: workspace must be 256-byte aligned", who);
+  hipStream_t st = (hipStream_t)hip_stream;
+  uint8_t* ws = (uint8_t*)workspace;
+  float* sg = (float*)(ws + b.off_sg);
+  float* proj = (float*)(ws + b.off_proj);
+  int8_t* codes = (int8_t*)(ws + b.off_codes);
+  int32_t* acc_a = (int32_t*)(ws + b.off_acca);
+  int32_t* acc_b = (int32_t*)(ws + b.off_accb);
+  int rc = hla_project_impl(gy, dtype, L, O, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, proj, b.k8, st);
+  if (rc) return rc;
+  rc = hq_luq_impl(proj, HOT_F32, O, b.k8, 1, cfg->gw_bits, cfg->seed, codes, b.kp, sg, ws + b.off_slots, STAT_SLOT_BYTES, st,
+                   HOT_STREAM_LUQ_GW);
+  if (rc) return rc;
+  const float post = 1.0f / (float)cfg->hla_n;
+  rc = gemm_i8_impl(codes, 2 * b.kp, xq, b.kp, 8, O, I, b.lp, sg, 0, sx, post, gw, out_dtype, I, acc_a, st);
+  if (rc) return rc;
+  rc = gemm_i8_impl(codes + b.kp, 2 * b.kp, xq, b.kp, 8, O, I, b.lp, sg, 0, sx, post, gw, out_dtype, I, acc_b, st);
+  if (rc) return rc;
+  return luq_combine_impl(acc_a, acc_b, O, I, sg, sx, post, gw, out_dtype, st);
+}
+
 // ---- 3-D activations: one set of steps per sample --------------------------------------------------
 // The reference vmaps its quantisers over the batch dimension of [B, T, C] tensors
 // (utils/quant_matmul.py:33-37,102-106,118-122), applies the token-wise transform inside each sample

@@ -87,4 +87,106 @@ int hla_expand_impl(const float* t, int64_t nb, int64_t C, int n, const int32_t*
   return check_launch("hla_expand_kernel");
 }
 
+// ---- the projection itself, unquantised (the operand of the logarithmic quantiser on the g_W side:
+// luq_quantizer(lowering_matmul_back(P, g_y).mT), utils/quant_matmul.py:296-301,307-314) ---------------
+// Same ownership as the expansion: a thread holds its channel's block in its own LDS column, runs the
+// canonical butterflies and writes the r kept coefficients to its channel's row of the transposed
+// fp32 output.  Kept for completeness, not tuned.
+struct ProjectArgs {
+  const void* in;      // [nb n, C]
+  float* out;          // [C, ld]
+  int64_t nb, C, ld;
+  int32_t n, r;
+  int8_t row[EXP_MAX_N];
+};
+
+template <typename T> __device__ __forceinline__ float load_as_f32(const void* p, int64_t i);
+template <> __device__ __forceinline__ float load_as_f32<float>(const void* p, int64_t i) { return reinterpret_cast<const float*>(p)[i]; }
+template <> __device__ __forceinline__ float load_as_f32<bf16_t>(const void* p, int64_t i) {
+  return as_f((uint32_t)reinterpret_cast<const uint16_t*>(p)[i] << 16);
+}
+template <> __device__ __forceinline__ float load_as_f32<f16_t>(const void* p, int64_t i) { return (float)reinterpret_cast<const _Float16*>(p)[i]; }
+
+template <typename T>
+__global__ void __launch_bounds__(EXP_THREADS) hla_project_kernel(const ProjectArgs a) {
+  extern __shared__ float col[];                      // [n][threads]
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int64_t c = (int64_t)blockIdx.x * nt + tid;
+  const int64_t blk = blockIdx.y;
+  if (c >= a.C) return;                               // no barriers below
+  for (int i = 0; i < a.n; ++i) col[i * nt + tid] = load_as_f32<T>(a.in, (blk * a.n + i) * a.C + c);
+  for (int h = 1; h < a.n; h <<= 1)
+    for (int i = 0; i < a.n; ++i)
+      if ((i & h) == 0) {
+        const float x = col[i * nt + tid], y = col[(i + h) * nt + tid];
+        col[i * nt + tid] = x + y;
+        col[(i + h) * nt + tid] = x - y;
+      }
+  float* dst = a.out + c * a.ld + blk * a.r;
+  for (int k = 0; k < a.r; ++k) dst[k] = col[a.row[k] * nt + tid];
+  if (blk == a.nb - 1)
+    for (int64_t k = a.nb * a.r; k < a.ld; ++k) a.out[c * a.ld + k] = 0.f;
+}
+
+int hla_project_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r, float* out,
+                     int64_t ld, hipStream_t st) {
+  const char* who = "hla_project";
+  if (!in || !out || !rows) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
+  if (n < 1 || n > EXP_MAX_N || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block %d (a power of two up to %d)", who, n, EXP_MAX_N);
+  if (R <= 0 || C <= 0 || R % n) return fail(HOT_ERR_INVALID, "%s: %lld rows are not whole blocks of %d", who, (long long)R, n);
+  if (r < 1 || r > n) return fail(HOT_ERR_INVALID, "%s: r=%d outside [1, %d]", who, r, n);
+  const int64_t nb = R / n;
+  if (nb > 65535) return fail(HOT_ERR_UNSUPPORTED, "%s: more than 65535 token blocks", who);
+  if (ld < nb * r) return fail(HOT_ERR_INVALID, "%s: ld=%lld < %lld coefficients", who, (long long)ld, (long long)(nb * r));
+  ProjectArgs a;
+  a.in = in; a.out = out; a.nb = nb; a.C = C; a.ld = ld; a.n = n; a.r = r;
+  bool seen[EXP_MAX_N] = {};
+  for (int k = 0; k < r; ++k) {
+    if (rows[k] < 0 || rows[k] >= n || seen[rows[k]]) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d out of range or listed twice", who, k, rows[k]);
+    seen[rows[k]] = true;
+    a.row[k] = (int8_t)rows[k];
+  }
+  const int nt = n > 64 ? 128 : EXP_THREADS;
+  const dim3 grid((unsigned)((C + nt - 1) / nt), (unsigned)nb);
+  const size_t lds = (size_t)n * nt * sizeof(float);
+  static std::once_flag once;
+  static hipError_t attr_err = hipSuccess;
+  std::call_once(once, [] {
+    attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&hla_project_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    if (attr_err == hipSuccess) attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&hla_project_kernel<bf16_t>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+    if (attr_err == hipSuccess) attr_err = hipFuncSetAttribute(reinterpret_cast<const void*>(&hla_project_kernel<f16_t>), hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+  });
+  if (attr_err != hipSuccess) return check_hip(attr_err, "hipFuncSetAttribute(hla_project_kernel)");
+  switch (dtype) {
+    case HOT_F32: hipLaunchKernelGGL(hla_project_kernel<float>, grid, dim3(nt), lds, st, a); break;
+    case HOT_BF16: hipLaunchKernelGGL(hla_project_kernel<bf16_t>, grid, dim3(nt), lds, st, a); break;
+    case HOT_F16: hipLaunchKernelGGL(hla_project_kernel<f16_t>, grid, dim3(nt), lds, st, a); break;
+    default: return fail(HOT_ERR_INVALID, "%s: bad dtype %d", who, dtype);
+  }
+  return check_launch("hla_project_kernel");
+}
+
+template <typename OutT>
+__global__ void __launch_bounds__(256) luq_combine_kernel(const int32_t* __restrict__ acc_a, const int32_t* __restrict__ acc_b,
+                                                          int64_t count, const float* __restrict__ s_a,
+                                                          const float* __restrict__ s_b, float post, OutT* __restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= count) return;
+  const int32_t acc = 16 * acc_a[i] + acc_b[i];
+  store_scalar<OutT>(out + i, (((float)acc * s_a[0]) * s_b[0]) * post);
+}
+
+int luq_combine_impl(const int32_t* acc_a, const int32_t* acc_b, int64_t M, int64_t N, const float* s_a, const float* s_b,
+                     float post, void* out, int out_dtype, hipStream_t st) {
+  const int64_t count = M * N;
+  const dim3 grid((unsigned)((count + 255) / 256));
+  switch (out_dtype) {
+    case HOT_F32: hipLaunchKernelGGL(luq_combine_kernel<float>, grid, dim3(256), 0, st, acc_a, acc_b, count, s_a, s_b, post, (float*)out); break;
+    case HOT_BF16: hipLaunchKernelGGL(luq_combine_kernel<bf16_t>, grid, dim3(256), 0, st, acc_a, acc_b, count, s_a, s_b, post, (bf16_t*)out); break;
+    case HOT_F16: hipLaunchKernelGGL(luq_combine_kernel<f16_t>, grid, dim3(256), 0, st, acc_a, acc_b, count, s_a, s_b, post, (f16_t*)out); break;
+    default: return fail(HOT_ERR_INVALID, "luq_combine: bad out dtype %d", out_dtype);
+  }
+  return check_launch("luq_combine_kernel");
+}
+
 }  // namespace hot

@@ -41,7 +41,17 @@ int hq_rowwise_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int 
 // Logarithmic quantiser of the row-wise transformed tensor (luq_quantizer_BWD): codes 0 / +-2^j split as
 // 16 a + b into two planes of kp bytes per row ([M, 2 kp]), one step; the workspace holds STAT_SLOT_BYTES.
 int hq_luq_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, uint64_t seed, void* codes_out,
-                int64_t kp, float* scale_out, void* workspace, size_t workspace_bytes, hipStream_t st);
+                int64_t kp, float* scale_out, void* workspace, size_t workspace_bytes, hipStream_t st,
+                uint32_t rng_stream = 4);
+// RNG streams of the logarithmic quantiser: its operand of the g_x product, of the g_W product
+constexpr uint32_t HOT_STREAM_LUQ = 4, HOT_STREAM_LUQ_GW = 5;
+// Unquantised token-wise projection, transposed: out[c][blk r + k] = (P in)[blk r + k][c] in fp32, ld
+// floats per channel (the tail [NB r, ld) cleared); blocks up to 128 tokens.
+int hla_project_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r, float* out,
+                     int64_t ld, hipStream_t st);
+// out = ((float(16 acc_a + acc_b) * s_a[0]) * s_b[0]) * post on [M, N] int32 sums
+int luq_combine_impl(const int32_t* acc_a, const int32_t* acc_b, int64_t M, int64_t N, const float* s_a, const float* s_b,
+                     float post, void* out, int out_dtype, hipStream_t st);
 // [rows, 2 kp] = [16 w | w] from INT8-stored codes w [rows, kp] with |w| <= 8
 int luq_pair_impl(const void* qw, int64_t rows, int64_t kp, void* out, hipStream_t st);
 

@@ -277,7 +277,8 @@ __global__ void hq_group_quant_kernel(const T* __restrict__ in, int64_t chunks_p
 // q = 16 a + b and stored in two planes of a row, a in bytes [0, Kp) and b in bytes [Kp, 2 Kp); the other
 // operand carries 16 w in its first plane and w in its second, so one INT8 product over 2 Kp codes
 // is the exact sum of q w.  Element e draws the uniforms 2 e and 2 e + 1 of the stream.
-constexpr uint32_t LUQ_STREAM = 4;
+constexpr uint32_t LUQ_STREAM = 4;      // the g_y operand of the g_x product
+constexpr uint32_t LUQ_GW_STREAM = 5;   // the projected g_y operand of the g_W product
 
 __device__ __forceinline__ int luq_code(float x, float s, float u1, float u2) {
 #pragma clang fp contract(off)
@@ -320,7 +321,7 @@ __global__ void hq_posmax_kernel(const T* __restrict__ in, int64_t nchunks, floa
 template <typename T, int N>
 __global__ void hq_luq_kernel(const T* __restrict__ in, int64_t nchunks, int64_t nch_row, int64_t ld, int64_t kp,
                               const float* __restrict__ slots, float inv_levels, int8_t* __restrict__ codes,
-                              float* __restrict__ scale_out, uint64_t seed, int nrt) {
+                              float* __restrict__ scale_out, uint64_t seed, uint32_t rng_stream, int nrt) {
   const int lane = threadIdx.x & 63;
   const float s = stat_slots_max(slots, lane) * inv_levels;       // a power of two: exact
   if (blockIdx.x == 0 && threadIdx.x == 0) *scale_out = s;
@@ -330,8 +331,8 @@ __global__ void hq_luq_kernel(const T* __restrict__ in, int64_t nchunks, int64_t
     load_chunk<T>(in + ch * EPL, x);
     fwht_lanes<N>(x, lane, nrt);
     float u[2 * EPL];
-    sr_uniform8((uint64_t)ch * 2, seed, LUQ_STREAM, u);          // uniforms 16 ch .. 16 ch + 15
-    sr_uniform8((uint64_t)ch * 2 + 1, seed, LUQ_STREAM, u + EPL);
+    sr_uniform8((uint64_t)ch * 2, seed, rng_stream, u);          // uniforms 16 ch .. 16 ch + 15
+    sr_uniform8((uint64_t)ch * 2 + 1, seed, rng_stream, u + EPL);
     uint32_t hi0 = 0, hi1 = 0, lo0 = 0, lo1 = 0;
 #pragma unroll
     for (int j = 0; j < EPL; ++j) {
@@ -487,7 +488,7 @@ static int dispatch_n(int n, int bits, int rounding, int scale_mode, const void*
 
 template <typename T, int N>
 static int launch_luq(const void* in, int64_t M, int64_t K, int bits, void* codes, int64_t ld, int64_t kp, float* scale,
-                      float* slots, uint64_t seed, hipStream_t st, int nrt) {
+                      float* slots, uint64_t seed, uint32_t rng_stream, hipStream_t st, int nrt) {
   const int64_t nch = M * K / EPL;
   int64_t blocks = (nch + 255) / 256;
   if (blocks > 256 * 16) blocks = 256 * 16;
@@ -496,23 +497,23 @@ static int launch_luq(const void* in, int64_t M, int64_t K, int bits, void* code
   hipLaunchKernelGGL(fill_u32_kernel, dim3(2), dim3(256), 0, st, (uint32_t*)slots, 0u, (int)(STAT_SLOT_BYTES / 4));
   hipLaunchKernelGGL((hq_posmax_kernel<T, N>), dim3((unsigned)blocks), dim3(256), 0, st, (const T*)in, nch, slots, nrt);
   hipLaunchKernelGGL((hq_luq_kernel<T, N>), dim3((unsigned)blocks), dim3(256), 0, st, (const T*)in, nch, K / EPL, ld, kp,
-                     slots, 1.0f / (float)(1 << lev), (int8_t*)codes, scale, seed, nrt);
+                     slots, 1.0f / (float)(1 << lev), (int8_t*)codes, scale, seed, rng_stream, nrt);
   return check_launch("hq_luq_kernel");
 }
 
 template <typename T>
 static int dispatch_luq(int n, const void* in, int64_t M, int64_t K, int bits, void* codes, int64_t ld, int64_t kp,
-                        float* scale, float* slots, uint64_t seed, hipStream_t st) {
+                        float* scale, float* slots, uint64_t seed, uint32_t rng_stream, hipStream_t st) {
   switch (n) {
-    case 1: case 2: case 4: case 8: return launch_luq<T, 8>(in, M, K, bits, codes, ld, kp, scale, slots, seed, st, n);
-    case 16: return launch_luq<T, 16>(in, M, K, bits, codes, ld, kp, scale, slots, seed, st, n);
-    case 32: return launch_luq<T, 32>(in, M, K, bits, codes, ld, kp, scale, slots, seed, st, n);
-    default: return launch_luq<T, 64>(in, M, K, bits, codes, ld, kp, scale, slots, seed, st, n);
+    case 1: case 2: case 4: case 8: return launch_luq<T, 8>(in, M, K, bits, codes, ld, kp, scale, slots, seed, rng_stream, st, n);
+    case 16: return launch_luq<T, 16>(in, M, K, bits, codes, ld, kp, scale, slots, seed, rng_stream, st, n);
+    case 32: return launch_luq<T, 32>(in, M, K, bits, codes, ld, kp, scale, slots, seed, rng_stream, st, n);
+    default: return launch_luq<T, 64>(in, M, K, bits, codes, ld, kp, scale, slots, seed, rng_stream, st, n);
   }
 }
 
 int hq_luq_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits, uint64_t seed, void* codes_out,
-                int64_t kp, float* scale_out, void* workspace, size_t workspace_bytes, hipStream_t st) {
+                int64_t kp, float* scale_out, void* workspace, size_t workspace_bytes, hipStream_t st, uint32_t rng_stream) {
   const char* who = "hq_luq";
   if (!in || !codes_out || !scale_out) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
   if (M <= 0 || K <= 0 || K % 8) return fail(HOT_ERR_INVALID, "%s: bad shape M=%lld K=%lld (K a multiple of 8)", who, (long long)M, (long long)K);
@@ -525,9 +526,9 @@ int hq_luq_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits
   zero_pad_impl(codes_out, M, K, 2 * kp, st);
   float* slots = (float*)workspace;
   switch (dtype) {
-    case HOT_F32: return dispatch_luq<float>(n, in, M, K, bits, codes_out, 2 * kp, kp, scale_out, slots, seed, st);
-    case HOT_BF16: return dispatch_luq<bf16_t>(n, in, M, K, bits, codes_out, 2 * kp, kp, scale_out, slots, seed, st);
-    case HOT_F16: return dispatch_luq<f16_t>(n, in, M, K, bits, codes_out, 2 * kp, kp, scale_out, slots, seed, st);
+    case HOT_F32: return dispatch_luq<float>(n, in, M, K, bits, codes_out, 2 * kp, kp, scale_out, slots, seed, rng_stream, st);
+    case HOT_BF16: return dispatch_luq<bf16_t>(n, in, M, K, bits, codes_out, 2 * kp, kp, scale_out, slots, seed, rng_stream, st);
+    case HOT_F16: return dispatch_luq<f16_t>(n, in, M, K, bits, codes_out, 2 * kp, kp, scale_out, slots, seed, rng_stream, st);
     default: return fail(HOT_ERR_INVALID, "%s: bad dtype %d", who, dtype);
   }
 }

@@ -455,6 +455,29 @@ def gx_luq(gy: torch.Tensor, w: torch.Tensor, opt: HotOptions, out_dtype=None) -
     return gx
 
 
+def gw_luq(gy: torch.Tensor, xq: torch.Tensor, sx: torch.Tensor, opt: HotOptions, out_dtype=None) -> torch.Tensor:
+    """g_W [O, I] with the logarithmic quantiser on the projected g_y (hot_gw_luq; quantBWDGogw = "luq" or
+    luq_quantizer picked for g_W under quantAuto): opt.hla_n / hla_rows, gw_bits = 4 and opt.seed are read;
+    xq [I, kpad(L')] / sx [1] as abc_forward writes them."""
+    _need_gpu_2d(gy, "Go")
+    _need_gpu_2d(xq, "xq")
+    L, O = gy.shape
+    I = xq.shape[0]
+    lp = (L // opt.hla_n) * opt.hla_r
+    if xq.dtype != torch.int8 or xq.stride(0) != kpad(lp) or xq.stride(1) != 1:
+        raise RuntimeError("xq must be the [I, kpad(L')] INT8 buffer of abc_forward")
+    out_dtype = out_dtype or gy.dtype
+    cfg = opt.to_c()
+    need = _lib.lib().hot_gw_luq_workspace_bytes(L, O, I, C.byref(cfg))
+    if need == 0:
+        raise HotError("bad configuration: %s" % _lib.lib().hot_last_error().decode())
+    ws = _ws(need, gy.device)
+    gw = torch.empty((O, I), dtype=out_dtype, device=gy.device)
+    _lib.check(_lib.lib().hot_gw_luq(gy.data_ptr(), _dt(gy), xq.data_ptr(), sx.data_ptr(), L, O, I, C.byref(cfg),
+                                     gw.data_ptr(), _DTYPES[out_dtype], ws.data_ptr(), ws.numel(), _stream()))
+    return gw
+
+
 def measure_ceilings(device=None):
     """(copy GB/s, INT8 MFMA TOP/s) of this box from the library's two plain ceiling kernels."""
     device = device or torch.device("cuda", torch.cuda.current_device())

@@ -41,8 +41,9 @@ _QUANT_SCHEMES = {
     "stoch_quantizer": (ops.ROUND_STOCH, ops.SCALE_TENSOR),
     "norm_quantizer": (ops.ROUND_STOCH, ops.SCALE_ROW),
     "sawb_quantizer": (ops.ROUND_NEAREST, ops.SCALE_SAWB),
-    # the logarithmic quantiser has an entry point of its own for the g_x product (ops.gx_luq, see
-    # gx_uses_luq); the pair below only fills the option fields that entry point does not read
+    # the logarithmic quantiser has entry points of its own (ops.gx_luq for the g_x product, see
+    # gx_uses_luq; ops.gw_luq for the g_W product, see gw_uses_luq); the pair below only fills the option
+    # fields those entry points do not read
     "luq_quantizer": (ops.ROUND_STOCH, ops.SCALE_TENSOR),
 }
 _FLAG_SCHEMES = {"int": "int_quantizer", "stoch": "stoch_quantizer", "nq": "norm_quantizer",
@@ -55,6 +56,14 @@ def gx_uses_luq(layer_name: str = " ") -> bool:
     if args.quantAuto and len(args.layer_quant_dict) > 0:
         return args.layer_quant_dict.get(layer_name + "_gx") == "luq_quantizer"
     return args.quantBWDGogi == "luq"
+
+
+def gw_uses_luq(layer_name: str = " ") -> bool:
+    """True when the quantiser of the projected g_y of the g_W product is luq_quantizer
+    (args.quantBWDGogw == "luq", or the layer's "_gw" entry under quantAuto; utils/quant_matmul.py:307-314)."""
+    if args.quantAuto and len(args.layer_quant_dict) > 0:
+        return args.layer_quant_dict.get(layer_name + "_gw") == "luq_quantizer"
+    return args.quantBWDGogw == "luq"
 
 
 def _scheme(flag: str, what: str, allowed) -> Tuple[int, int]:
@@ -152,11 +161,9 @@ def _options_uncached(tokens: int, layer_name: str, out_features: int) -> ops.Ho
         gx_round, gx_scale = _QUANT_SCHEMES[args.layer_quant_dict[layer_name + "_gx"]]
         gw_round, gw_scale = _QUANT_SCHEMES[args.layer_quant_dict[layer_name + "_gw"]]
         gw_bits = args.GogiQuantBit
-        if args.layer_quant_dict[layer_name + "_gw"] == "luq_quantizer":
-            raise NotImplementedError("the logarithmic quantiser runs on the g_x product only (its codes are no INT8 grid)")
     else:
         gx_round, gx_scale = _scheme(args.quantBWDGogi, "GradHo", ("int", "stoch", "nq", "luq"))
-        gw_round, gw_scale = _scheme(args.quantBWDGogw, "GradHb", ("int", "stoch", "nq"))
+        gw_round, gw_scale = _scheme(args.quantBWDGogw, "GradHb", ("int", "stoch", "nq", "luq"))
     w_round, w_scale = _scheme(args.quantBWDWgt, "Weight", ("int", "stoch", "sawb"))
     act_round, act_scale = _scheme(args.quantBWDAct, "Activation", ("int", "stoch", "sawb"))
     return ops.HotOptions(
@@ -291,10 +298,12 @@ class FLinearQ(Function):
         if go.dtype != wc.dtype:
             go = go.to(wc.dtype)
         luq = gx_uses_luq(ctx.name)
-        if args.transform_scheme in LOWRANK_GX_SCHEMES or luq:
+        luq_gw = gw_uses_luq(ctx.name)
+        if args.transform_scheme in LOWRANK_GX_SCHEMES or luq or luq_gw:
             # g_x by an entry point of its own -- the projection along the tokens and its expansion
             # ("low_rank", "gilr_gwh"), or the logarithmic quantiser on g_y --, g_W as in "gih_gwlr" /
-            # "hadamard": the token-wise kernel on g_y, then the INT8 product
+            # "hadamard": the token-wise kernel on g_y, then the INT8 product; or, with the logarithmic
+            # quantiser on the projected g_y, ops.gw_luq
             # 3-D activations with a step per sample (the reference's vmap over the batch,
             # utils/quant_matmul.py:79-83): one pass per sample, sample b seeded with seed + b, the weight
             # gradients of the samples added in fp32 in sample order
@@ -309,15 +318,7 @@ class FLinearQ(Function):
             for b, g in enumerate(samples):
                 opt_b = replace(opt, seed=opt.seed + b) if b else opt
                 go2 = _pad8(g)
-                if luq:
-                    gx = ops.gx_luq(go2, wc, opt_b)
-                else:
-                    n_gx, rows_gx = gx_token_rule(go2.shape[0])
-                    gx = ops.gx_lowrank(go2, wc, replace(opt_b, hla_n=int(n_gx), hla_rows=tuple(int(v) for v in rows_gx)))
-                qgp, sgp, lp = ops.hla_tokenwise(go2, opt.hla_n, opt.hla_rows, bits=opt.gw_bits,
-                                                 rounding="stoch" if opt.gw_round == ops.ROUND_STOCH else "nearest",
-                                                 scale="row" if opt.gw_scale == ops.SCALE_ROW else "tensor",
-                                                 seed=opt_b.seed, rng_stream=ops.STREAM_GW)
+                lp = (go2.shape[0] // opt.hla_n) * opt.hla_r
                 if not per_sample:
                     xq_b, sx_b = xq, sx
                 elif ctx.batched:
@@ -329,10 +330,26 @@ class FLinearQ(Function):
                     sx_b = sx[b:b + 1]
                 else:
                     xq_b, sx_b = xq[b], sx[b:b + 1]
-                # both operands hold one code per byte whatever their widths (the token-wise kernel and the
-                # activation buffer never pack): an INT8 product, as in the fused path
-                gw_b = ops.gemm_i8(qgp, xq_b, lp, 8, sgp, sx_b, post_scale=1.0 / opt.hla_n,
-                                   out_dtype=torch.float32 if per_sample else wc.dtype)
+                if luq:
+                    gx = ops.gx_luq(go2, wc, opt_b)
+                elif args.transform_scheme in LOWRANK_GX_SCHEMES:
+                    n_gx, rows_gx = gx_token_rule(go2.shape[0])
+                    gx = ops.gx_lowrank(go2, wc, replace(opt_b, hla_n=int(n_gx), hla_rows=tuple(int(v) for v in rows_gx)))
+                else:
+                    # the usual g_x, from the fused call (its g_W, by the quantiser the option fields
+                    # name for the logarithmic one, is dropped)
+                    gx = ops.linear_backward(go2, wc, xq_b, sx_b, opt_b)[0]
+                gw_dtype = torch.float32 if per_sample else wc.dtype
+                if luq_gw:
+                    gw_b = ops.gw_luq(go2, xq_b, sx_b, opt_b, out_dtype=gw_dtype)
+                else:
+                    qgp, sgp, lp = ops.hla_tokenwise(go2, opt.hla_n, opt.hla_rows, bits=opt.gw_bits,
+                                                     rounding="stoch" if opt.gw_round == ops.ROUND_STOCH else "nearest",
+                                                     scale="row" if opt.gw_scale == ops.SCALE_ROW else "tensor",
+                                                     seed=opt_b.seed, rng_stream=ops.STREAM_GW)
+                    # both operands hold one code per byte whatever their widths (the token-wise kernel and
+                    # the activation buffer never pack): an INT8 product, as in the fused path
+                    gw_b = ops.gemm_i8(qgp, xq_b, lp, 8, sgp, sx_b, post_scale=1.0 / opt.hla_n, out_dtype=gw_dtype)
                 gw = gw_b if gw is None else gw + gw_b
                 gxs.append(gx[:, :I])
             grad_w = gw.to(wc.dtype)

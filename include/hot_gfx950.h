@@ -319,6 +319,19 @@ HOT_API int hot_gx_luq(const void* gy, const void* w, int dtype, int64_t L, int6
                size_t workspace_bytes, void* hip_stream);
 
 /*
+ * g_W with the logarithmic quantiser on the projected g_y (quantBWDGogw = "luq", or luq_quantizer
+ * picked for a layer's g_W under quantAuto, utils/quant_matmul.py:296-301,307-314,322-324):
+ * g_W[O, I] = (luq((P g_y)^T) . xq^T) s sx / hla_n, xq / sx as written by hot_abc_forward
+ * ([I, hot_kpad(L')] INT8 codes, one step).  gw_bits = 4, token blocks up to 128.  Element
+ * e = o K8 + k of the projected tensor [O, L'] (K8 = L' rounded up to 8) draws the uniforms 2 e and
+ * 2 e + 1 of Philox stream 5 under cfg->seed; codes saturate at +-2^10 as in hot_gx_luq.
+ */
+HOT_API size_t hot_gw_luq_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_config* cfg);
+HOT_API int hot_gw_luq(const void* gy, int dtype, const void* xq, const float* sx, int64_t L, int64_t O,
+               int64_t I, const hot_config* cfg, void* gw, int out_dtype, void* workspace,
+               size_t workspace_bytes, void* hip_stream);
+
+/*
  * Number of K ranges into which the GEMMs inside hot_linear_backward cut a product of
  * M x N outputs over K codes of `bits` bits (1 = one kernel; more = a kernel per range
  * writing int32 partial tiles to the workspace, then a reduce kernel).  Products with

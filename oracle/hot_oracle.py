@@ -598,6 +598,28 @@ def gx_luq(g_y: np.ndarray, w: np.ndarray, cfg: HotConfig, max_exp: Optional[int
     return tr
 
 
+STREAM_LUQ_GW = 5  # the logarithmic quantiser on the projected g_y of the g_W product
+
+
+def gw_luq(g_y: np.ndarray, xq: np.ndarray, sx: np.ndarray, cfg: HotConfig,
+           max_exp: Optional[int] = LUQ_PRODUCT_MAX_EXP) -> np.ndarray:
+    """grad_weight with the logarithmic quantiser on the projected g_y (quantBWDGogw = "luq", or
+    luq_quantizer picked for a layer's g_W under quantAuto; utils/quant_matmul.py:296-301 g_y <- (P g_y)^T
+    [O, L'], :307-314 luq_quantizer at cfg.gw_bits, :322-324 (q . xq) s s_x, :339-346 / n).  xq [L', I]
+    and sx as abc_forward returns them.  Element e = o K8 + k of the projected tensor, K8 = L' rounded up
+    to a multiple of 8 (the kernel's rows are padded with zeros, which draw code 0), takes the uniforms
+    2 e and 2 e + 1 of stream STREAM_LUQ_GW.  Codes saturate at +-2^max_exp as in gx_luq."""
+    g_y = np.asarray(g_y, dtype=F32)
+    rows = np.asarray(cfg.hla_rows)
+    Gt = np.ascontiguousarray(fwht_blocks_first(g_y, cfg.hla_n, rows).T)                  # [O, L']
+    O, lp = Gt.shape
+    k8 = -(-lp // 8) * 8
+    index = np.arange(O, dtype=np.int64)[:, None] * k8 + np.arange(lp, dtype=np.int64)[None, :]
+    q, s = luq_quant(Gt, cfg.gw_bits, cfg.seed, stream=STREAM_LUQ_GW, index=index, max_exp=max_exp)
+    acc = int_gemm_nt(q, np.asarray(xq).T)
+    return (((acc.astype(F32) * s[0]).astype(F32) * F32(np.asarray(sx).reshape(-1)[0])).astype(F32) / F32(cfg.hla_n)).astype(F32)
+
+
 def stoch_round_mantissa(x: np.ndarray) -> np.ndarray:
     """The reference CUDA op's pseudo-stochastic rounding
     (HLQ_backward_kernel.cu:19-36), kept only to characterise its bias; the

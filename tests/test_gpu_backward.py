@@ -939,6 +939,67 @@ def test_hq_linear_with_luq_on_the_gx_path(gpu, fresh_args):
     assert np.array_equal(lin.weight.grad.cpu().numpy(), orc.linear_backward(gyn, wn, xq_ref, sx_ref, ocfg).g_w)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("L,O,I,rule,variant", [
+    (448, 192, 160, "python", dict(seed=1)),                       # n = 64, r = 36
+    (1576, 80, 264, "python", dict(seed=2, act_bits=4)),            # n = 8: L' is no multiple of 8, rows padded
+    (512, 256, 128, "paper", dict(seed=3)),                        # n = 16, r = 8
+    (197, 40, 24, "python", dict(seed=4)),                         # n = 1: nothing projected, 197 -> 200 per row
+    (4096, 768, 512, "python", dict(seed=5)),
+])
+def test_gw_luq_matches_oracle(gpu, dtype, L, O, I, rule, variant):
+    """g_W with the logarithmic quantiser on the projected g_y (hot_gw_luq): the projection in fp32 by
+    the canonical butterflies, codes 0 / +-2^j as two INT8 planes against the activation buffer, the
+    integer sums combined: bit for bit the oracle (same uniforms, same float operations)."""
+    from hot_amd import ops
+    x, w, gy = make_case(L, O, I, seed=L + O, dtype=dtype)
+    ocfg, opt = both_configs(L, rule=rule, gw_bits=4, **variant)
+    xq, sx = ops.abc_forward(x.to(gpu), opt)
+    xq_ref, sx_ref = orc.abc_forward(x.float().numpy(), ocfg)
+    gw = ops.gw_luq(gy.to(gpu), xq, sx, opt)
+    ref = orc.gw_luq(gy.float().numpy(), xq_ref, sx_ref, ocfg)
+    assert gw.dtype == dtype and tuple(gw.shape) == (O, I)
+    assert torch.equal(gw.cpu(), torch.from_numpy(ref).to(dtype))
+
+
+def test_gw_luq_refuses_what_it_cannot_do(gpu):
+    from hot_amd import ops
+    x, w, gy = make_case(256, 64, 32, seed=0)
+    _, opt = both_configs(256)
+    xq, sx = ops.abc_forward(x.to(gpu), opt)
+    with pytest.raises(ops.HotError, match="4 bits"):
+        ops.gw_luq(gy.to(gpu), xq, sx, opt)                        # gw_bits = 8
+
+
+@pytest.mark.parametrize("how", ["flag", "auto"])
+def test_hq_linear_with_luq_on_the_gw_path(gpu, fresh_args, how):
+    """quantBWDGogw = "luq" at GogwQuantBit = 4, and luq_quantizer picked for both products of a layer
+    under quantAuto (where the g_W branch reads GogiQuantBit, utils/quant_matmul.py:307-308): g_W through
+    hot_gw_luq, g_x by the fused call or hot_gx_luq.  Bit-exact against the oracle."""
+    from hot_amd.quant_matmul import HQ_Linear
+    L, I, O = 448, 96, 128
+    torch.manual_seed(6)
+    lin = HQ_Linear(I, O, bias=False).to(gpu)
+    lin.layer_name = "blk.fc"
+    if how == "flag":
+        fresh_args.quantBWDGogw = "luq"
+        fresh_args.GogwQuantBit = 4
+    else:
+        fresh_args.quantAuto = True
+        fresh_args.layer_quant_dict = {"blk.fc_gx": "luq_quantizer", "blk.fc_gw": "luq_quantizer"}
+    x = torch.randn(L, I, device=gpu, requires_grad=True)
+    gy = torch.randn(L, O, device=gpu) * 1e-3
+    step = fresh_args.sr_step
+    lin(x).backward(gy)
+    xn, gyn, wn = x.detach().cpu().numpy(), gy.cpu().numpy(), lin.weight.detach().cpu().numpy()
+    seed = (int(fresh_args.sr_seed) << 20) + step
+    ocfg, _ = both_configs(L, seed=seed, gw_bits=4, gw_round=orc.ROUND_STOCH)
+    xq_ref, sx_ref = orc.abc_forward(xn, ocfg)
+    assert np.array_equal(lin.weight.grad.cpu().numpy(), orc.gw_luq(gyn, xq_ref, sx_ref, ocfg))
+    gx_ref = orc.gx_luq(gyn, wn, ocfg).g_x if how == "auto" else orc.linear_backward(gyn, wn, xq_ref, sx_ref, ocfg).g_x
+    assert np.array_equal(x.grad.cpu().numpy(), gx_ref)
+
+
 @pytest.mark.parametrize("path,T", [("luq", 64), ("luq", 197), ("low_rank", 64), ("gilr_gwh", 48), ("low_rank", 256)])
 def test_hq_linear_3d_per_sample_on_the_separate_gx_paths(gpu, fresh_args, path, T):
     """3-D activations with a step per sample (the reference's vmap over the batch,

@@ -111,10 +111,11 @@ def test_options_follow_args(fresh_args):
     a.quantBWDGogi = "luq"                          # an entry point of its own for the g_x product
     from hot_amd.quant_matmul import gx_uses_luq
     assert gx_uses_luq() and options_for(64).gx_bits == 4
-    a.quantBWDGogw = "luq"                          # not for the g_W product
-    with pytest.raises(NotImplementedError):
-        options_for(64)
+    a.quantBWDGogw = "luq"                          # and one for the g_W product
+    from hot_amd.quant_matmul import gw_uses_luq
+    assert gw_uses_luq() and options_for(64).gw_round == ops.ROUND_STOCH
     a.quantBWDGogw = "int"
+    assert not gw_uses_luq()
     a.quantBWDGogi = "int"
     assert not gx_uses_luq()
     a.transform_scheme = "hadamard"                 # block Hadamard along the tokens, nothing dropped
@@ -125,7 +126,11 @@ def test_options_follow_args(fresh_args):
     from hot_amd.quant_matmul import gx_token_rule
     o = options_for(12608)
     assert (o.hla_n, o.hla_r) == (64, 36)
-    assert gx_token_rule(8192)[0] == 64 and len(gx_token_rule(8192)[1]) == 36    # blocks of at most 64 tokens
+    assert gx_token_rule(8192)[0] == 8192 and len(gx_token_rule(8192)[1]) == 2080    # the reference's own rule
+    assert gx_token_rule(25216)[0] == 128 and len(gx_token_rule(25216)[1]) == 36
+    a.hla_max_block = 64
+    assert gx_token_rule(8192)[0] == 64 and len(gx_token_rule(8192)[1]) == 36
+    a.hla_max_block = 8192
     a.transform_scheme = "gilr_gwh"                 # g_W side as hadamard
     o = options_for(12608)
     assert (o.hla_n, o.hla_r) == (16, 16)

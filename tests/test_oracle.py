@@ -8,6 +8,7 @@ import itertools
 import os
 
 import numpy as np
+from dataclasses import replace
 import pytest
 import scipy.linalg
 
@@ -609,6 +610,39 @@ def test_luq_saturation_of_the_product_form():
     assert np.abs(tr_h.qG).max() == 1024 and np.abs(tr_f.qG).max() > 1024
     keep = np.ones(32, bool); keep[3] = False
     assert np.array_equal(tr_h.g_x[keep], tr_f.g_x[keep])
+
+
+def test_gw_luq_mean_is_the_product_with_the_dequantised_buffer():
+    """gw_luq = (luq((P g_y)^T) . xq^T) s s_x / n: the quantiser is unbiased, so the mean over seeds
+    converges on ((P g_y)^T . (xq s_x)^T) / n, a plain float product of the projection (computed here from
+    the explicit matrix P, not from the butterflies) with the dequantised buffer.  A transposed operand,
+    a dropped step or the wrong divisor misses it by far more than the sampling error; the rows are
+    padded (L' = 21 -> 24), which moves the element numbers only."""
+    rng = np.random.default_rng(8)
+    L, O, I = 56, 24, 16
+    gy = (rng.standard_normal((L, O)) * 1e-3).astype(np.float32)
+    x = rng.standard_normal((L, I)).astype(np.float32)
+    n, rows = orc.hla_rows(L)
+    lp = (L // n) * len(rows)
+    assert (n, lp) == (8, 21)
+    cfg = orc.HotConfig(hla_n=n, hla_rows=tuple(int(v) for v in rows), gw_bits=4)
+    xq, sx = orc.abc_forward(x, cfg)
+    P = np.kron(np.eye(L // n), orc.make_WHT(n).astype(np.float64))                    # [L', L]
+    target = (P @ gy.astype(np.float64)).T @ (xq.astype(np.float64) * float(sx[0])) / n
+    N = 300
+    acc = np.zeros_like(target)
+    for seed in range(N):
+        acc += orc.gw_luq(gy, xq, sx, replace(cfg, seed=seed))
+    assert np.linalg.norm(acc / N - target) / np.linalg.norm(target) < 0.05
+    one = orc.gw_luq(gy, xq, sx, cfg)
+    assert one.shape == (O, I) and one.dtype == np.float32
+    assert np.linalg.norm(one - target) / np.linalg.norm(target) > 0.05                # a single draw is coarse
+    # element numbering: padded rows, stream 5 -- a different stream or the unpadded numbering draws other codes
+    Gt = np.ascontiguousarray(orc.fwht_blocks_first(gy, n, np.asarray(rows)).T)
+    idx = np.arange(O)[:, None] * 24 + np.arange(lp)[None, :]
+    q, s = orc.luq_quant(Gt, 4, 0, stream=orc.STREAM_LUQ_GW, index=idx, max_exp=10)
+    ref = ((orc.int_gemm_nt(q, xq.T).astype(np.float32) * s[0]) * sx[0]) / np.float32(n)
+    assert np.array_equal(orc.gw_luq(gy, xq, sx, replace(cfg, seed=0)), ref.astype(np.float32))
 
 
 def test_gx_luq_close_to_the_plain_product():
