@@ -28,6 +28,7 @@ Prints ONE JSON line.  Besides the contract fields it carries
   measure_py    the reference's latency harness (cuda_measure/measure.py) on the drop-in op
   vit_b16       whole-model backward with every layer swapped
   forward_gemm  the plain bf16 forward product at the layer shapes: vendor library beside hot_gemm_bf16
+  schemes       the layer's backward under every transform scheme / quantiser family the native path runs
 This run uses one GPU; --gpus above 1 is refused.
 """
 from __future__ import annotations
@@ -349,6 +350,39 @@ def forward_gemm_table(dev):
             "note": "bf16, bias added in the epilogue of both; 20 calls after 5 warm-ups"}
 
 
+def scheme_table(dev):
+    """The layer's backward through autograd (HQ_Linear, ViT-B fc1, bf16, 2-D tokens) under every transform
+    scheme and quantiser family the native path runs: the fused call for gih_gwlr / hadamard, the separate
+    g_x entry points for the schemes that project g_y along the tokens and for the logarithmic quantiser
+    (kept for completeness of the reference's scheme list, not tuned)."""
+    import torch
+    from hot_amd import args
+    from hot_amd.quant_matmul import HQ_Linear
+    L, O, I = 12608, 3072, 768
+    saved = {k: getattr(args, k) for k in dir(args) if not k.startswith("_") and not callable(getattr(args, k))}
+    rows = []
+    try:
+        for label, recipe in (("gih_gwlr int", dict()), ("gih_gwlr stoch per-token", dict(gx="nq", gw="nq")),
+                              ("hadamard", dict(scheme="hadamard")), ("low_rank", dict(scheme="low_rank")),
+                              ("gilr_gwh", dict(scheme="gilr_gwh")), ("gih_gwlr luq g_x", dict(gx="luq")),
+                              ("gih_gwlr luq g_W", dict(gw="luq", gw_bits=4))):
+            args.hot_recipe(**recipe)
+            torch.manual_seed(0)
+            lin = HQ_Linear(I, O, bias=False).to(dev).to(torch.bfloat16)
+            x = torch.randn(L, I, device=dev, dtype=torch.bfloat16, requires_grad=True)
+            gy = (torch.randn(L, O, device=dev) * 1e-3).to(torch.bfloat16)
+            y = lin(x)
+            us = _events(lambda: torch.autograd.grad(y, (x, lin.weight), gy, retain_graph=True), 20, 10)
+            rows.append([label, round(us, 1)])
+            del lin, x, gy, y
+            torch.cuda.empty_cache()
+    finally:
+        for k, v in saved.items():
+            setattr(args, k, v)
+    return {"columns": ["scheme / quantisers", "backward_us"], "rows": rows,
+            "note": "L=12608 O=3072 I=768 bf16; 20 backward passes of one saved forward after 10 warm-ups"}
+
+
 def measure_py(dev, trials=100):
     """The reference's latency harness (cuda_measure/measure.py:35-80) on the drop-in op: L = 49 tokens,
     O = 3072, I = 768, lognormal(1, 0.1) inputs (numpy seed 2023), `trials` trials, medians.  As there:
@@ -605,7 +639,7 @@ def main():
         del lw, lsets
     if not a.no_extras and not a.table_only:
         for key, fn in (("layers", lambda: layer_table(dev)), ("measure_py", lambda: measure_py(dev)),
-                        ("forward_gemm", lambda: forward_gemm_table(dev))):
+                        ("forward_gemm", lambda: forward_gemm_table(dev)), ("schemes", lambda: scheme_table(dev))):
             try:
                 out[key] = fn()
             except Exception as e:          # extras never cost the headline line
