@@ -29,6 +29,7 @@ Prints ONE JSON line.  Besides the contract fields it carries
   vit_b16       whole-model backward with every layer swapped
   forward_gemm  the plain bf16 forward product at the layer shapes: vendor library beside hot_gemm_bf16
   schemes       the layer's backward under every transform scheme / quantiser family the native path runs
+  host_cost     host microseconds of one backward call (C entry point, Python op), one- and two-stream order
 This run uses one GPU; --gpus above 1 is refused.
 """
 from __future__ import annotations
@@ -76,13 +77,13 @@ def make_layer(L, O, I, dtype, dev, nsets, seed=0):
     return w, sets
 
 
-def profiled_traffic():
-    """HBM bytes per launch of the kernels of the step at the bench workload, as the committed counter
-    summary gives them (profiles/hot_linear_backward_vit_b_fc1_bf16.hbm_traffic.txt: lines
-    `traffic_bytes <kernel key> <bytes>` and `measured_at <commit>`), or (None, None) when the summary
-    is absent or carries no such lines.  The figures belong to the commit named there: kernels changed
-    since then are listed without traffic."""
-    path = os.path.join(ROOT, "profiles", "hot_linear_backward_vit_b_fc1_bf16.hbm_traffic.txt")
+def profiled_traffic(workload="vit_b_fc1"):
+    """HBM bytes per launch of the kernels of the step at a workload ("vit_b_fc1", "llama_gate_up"), as
+    the committed counter summary gives them (profiles/hot_linear_backward_<workload>_bf16.hbm_traffic.txt:
+    lines `traffic_bytes <kernel key> <bytes>` and `measured_at <commit>`), or (None, None) when the
+    summary is absent or carries no such lines.  The figures belong to the commit named there: kernels
+    changed since then are listed without traffic."""
+    path = os.path.join(ROOT, "profiles", "hot_linear_backward_%s_bf16.hbm_traffic.txt" % workload)
     table, commit = {}, None
     try:
         for line in open(path):
@@ -383,6 +384,55 @@ def scheme_table(dev):
             "note": "L=12608 O=3072 I=768 bf16; 20 backward passes of one saved forward after 10 warm-ups"}
 
 
+def host_cost(dev, calls=300):
+    """Host time of one backward call: the C entry point through ctypes with prepared arguments, and
+    ops.linear_backward, at a shape whose kernels are short (64 tokens, O = I = 64), issued back to back
+    without waiting for the GPU, in the one-stream order (what the library picks for short calls) and
+    with the two-stream order forced (three event record / wait pairs more)."""
+    import ctypes as C
+    import time
+    import torch
+    from hot_amd import _lib, ops
+    from hot_amd.hadamard_matmul import hla_rows
+    L, O, I = 64, 64, 64
+    n, rows = hla_rows(L)
+    w, sets = make_layer(L, O, I, torch.bfloat16, dev, nsets=2, seed=5)
+    out = {}
+    for label, streams in (("one_stream", 1), ("two_streams", 2)):
+        opt = ops.HotOptions(n_o=16, hla_n=int(n), hla_rows=tuple(int(v) for v in rows), streams=streams)
+        bufs = [ops.abc_forward(x, opt) for (x, _) in sets]
+        cfg = opt.to_c()
+        need = _lib.lib().hot_backward_workspace_bytes(L, O, I, C.byref(cfg))
+        ws = torch.empty(need, dtype=torch.uint8, device=dev)
+        gx = torch.empty((L, I), dtype=torch.bfloat16, device=dev)
+        gw = torch.empty((O, I), dtype=torch.bfloat16, device=dev)
+        st = torch.cuda.current_stream().cuda_stream
+        fn = _lib.lib().hot_linear_backward
+
+        def c_call(i):
+            gy = sets[i % 2][1]
+            xq, sx = bufs[i % 2]
+            fn(gy.data_ptr(), w.data_ptr(), 1, xq.data_ptr(), sx.data_ptr(), L, O, I, C.byref(cfg), gx.data_ptr(),
+               gw.data_ptr(), 1, ws.data_ptr(), ws.numel(), None, st)
+
+        def py_call(i):
+            xq, sx = bufs[i % 2]
+            ops.linear_backward(sets[i % 2][1], w, xq, sx, opt)
+
+        for name, call in (("c_call_us", c_call), ("python_call_us", py_call)):
+            for i in range(30):
+                call(i)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(calls):
+                call(i)
+            t1 = time.perf_counter()
+            torch.cuda.synchronize()
+            out.setdefault(name, {})[label] = round((t1 - t0) / calls * 1e6, 1)
+    out["note"] = "%d calls issued back to back, wall time of the issuing loop per call (the GPU drains afterwards)" % calls
+    return out
+
+
 def measure_py(dev, trials=100):
     """The reference's latency harness (cuda_measure/measure.py:35-80) on the drop-in op: L = 49 tokens,
     O = 3072, I = 768, lognormal(1, 0.1) inputs (numpy seed 2023), `trials` trials, medians.  As there:
@@ -516,6 +566,8 @@ def main():
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run three 512 MiB device-to-device copies (a kernel of known traffic, for scaling "
                          "the FETCH_SIZE / WRITE_SIZE counters of a profiler run)")
+    ap.add_argument("--python-rule", action="store_true",
+                    help="with --llama-table: the reference's own low-rank rule (n = 8192, r = 2080), the step only")
     ap.add_argument("--llama-table", action="store_true",
                     help="only the per-kernel pass at the Llama-7B gate/up shape (kernels launched one after the "
                          "other), printed as one JSON line; for profiling runs of that shape")
@@ -544,12 +596,20 @@ def main():
 
     if a.llama_table:
         Ll, Ol, Il = 8192, 11008, 4096
-        pn, prow = paper_rows(16, 8)
+        if a.python_rule:
+            # the reference's own rule for 8192 tokens (one block of 8192, 2080 rows kept, listed run by
+            # run as the layer lists them): the two-level token-wise path, which has no per-kernel pass
+            from hot_amd.hadamard_matmul import run_major
+            pn, prow = hla_rows(Ll)
+            prow = run_major(prow)
+        else:
+            pn, prow = paper_rows(16, 8)
         lopt = ops.HotOptions(n_o=16, hla_n=int(pn), hla_rows=tuple(int(v) for v in prow))
         lw, lsets = make_layer(Ll, Ol, Il, torch.bfloat16, dev, nsets=2, seed=1)
         lsec, lbufs, lws = step_time(lw, lsets, lopt, a.steps, a.warmup)
-        ltable = kernel_table(lw, lsets, lbufs, lopt, lws, iters=6, warm=2)
-        print(json.dumps({"workload": "Llama-7B gate/up linear backward (L=8192, O=11008, I=4096), bf16, HLA n=16 r=8",
+        ltable = None if a.python_rule else kernel_table(lw, lsets, lbufs, lopt, lws, iters=6, warm=2)
+        print(json.dumps({"workload": "Llama-7B gate/up linear backward (L=8192, O=11008, I=4096), bf16, HLA n=%d r=%d"
+                                      % (lopt.hla_n, lopt.hla_r),
                           "us_per_layer": round(lsec * 1e6, 1), "steps": a.steps, "warmup": a.warmup,
                           "kernels_serial": ltable}))
         return
@@ -615,11 +675,15 @@ def main():
         lopt = ops.HotOptions(n_o=16, hla_n=int(pn), hla_rows=tuple(int(v) for v in prow))
         lw, lsets = make_layer(Ll, Ol, Il, torch.bfloat16, dev, nsets=2, seed=1)
         lsec, lbufs, lws = step_time(lw, lsets, lopt, max(5, a.steps // 5), max(2, a.warmup // 5))
-        ltable = kernel_table(lw, lsets, lbufs, lopt, lws, iters=6, warm=2)
+        ltraffic, ltraffic_commit = profiled_traffic("llama_gate_up")
+        ltable = kernel_table(lw, lsets, lbufs, lopt, lws, iters=6, warm=2, traffic=ltraffic)
         out["llama_gate_up"] = {"us_per_layer": round(lsec * 1e6, 1), "L": Ll, "O": Ol, "I": Il,
                                 "hla": "n=16 r=8", "int8_tops": round((2.0 * Ll * Ol * Il + 2.0 * Ol * Il * (Ll // 2)) / lsec / 1e12, 1),
-                                # kernels launched one after the other: [us, fraction of the 8 TB/s or 5 POP/s peak]
-                                "kernels_serial": {r["key"]: [r["us"], r["frac"]] for r in ltable}}
+                                # kernels launched one after the other: [us, fraction of the 8 TB/s or 5 POP/s
+                                # peak, HBM bytes per launch from the committed counter summary or null]
+                                "kernels_serial": {r["key"]: [r["us"], r["frac"], r["traffic"]] for r in ltable},
+                                "traffic_source": ("profiles/hot_linear_backward_llama_gate_up_bf16.hbm_traffic.txt at commit %s"
+                                                   % ltraffic_commit) if ltraffic else None}
         # the same layer at the reference's own low-rank rule for 8192 tokens (utils/hadamard_matmul.py:209-226:
         # one block of n = 8192, r = 2080 kept sequencies; the two-level token-wise path), the kept rows
         # listed run by run as the layer lists them (hot_amd.quant_matmul.token_rule)
@@ -639,7 +703,7 @@ def main():
         del lw, lsets
     if not a.no_extras and not a.table_only:
         for key, fn in (("layers", lambda: layer_table(dev)), ("measure_py", lambda: measure_py(dev)),
-                        ("forward_gemm", lambda: forward_gemm_table(dev)), ("schemes", lambda: scheme_table(dev))):
+                        ("forward_gemm", lambda: forward_gemm_table(dev)), ("schemes", lambda: scheme_table(dev)), ("host_cost", lambda: host_cost(dev))):
             try:
                 out[key] = fn()
             except Exception as e:          # extras never cost the headline line
