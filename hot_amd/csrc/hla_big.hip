@@ -276,10 +276,21 @@ __global__ void __launch_bounds__(64 * KG, 2) big_stage2_runs_kernel(const BigAr
   // the workgroup's K run within the block: the outputs of its coefficient indices, in list order
   const int k_hi = (grp + 1) * KG < a.nk ? (grp + 1) * KG : a.nk;
   const int run0 = a.kbase[grp * KG], run_len = a.kbase[k_hi] - run0;
+  // absmax steps come straight from the statistic (no finalize kernel in between); the workgroups of
+  // the first block and index group publish them
   float d = 1.f, clip = 0.f;
-  if (a.mode == HOT_SCALE_ROW) d = (active ? a.colmax[c] : 0.f) / (float)qmax + 1e-11f;
-  else if (a.mode == HOT_SCALE_TENSOR) d = a.stat[0] / (float)qmax + 1e-11f;
-  else { d = a.stat[1] + 1e-11f; clip = a.stat[2]; }
+  if (a.mode == HOT_SCALE_ROW) {
+    const float sc = (active ? a.colmax[c] : 0.f) / (float)qmax;
+    d = sc + 1e-11f;
+    if (active && blockIdx.y == 0 && wave == 0) a.scales_out[c] = sc;
+  } else if (a.mode == HOT_SCALE_TENSOR) {
+    const float sc = stat_slots_max(a.stat + 64, lane) / (float)qmax;
+    d = sc + 1e-11f;
+    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) a.scales_out[0] = sc;
+  } else {
+    d = a.stat[1] + 1e-11f;
+    clip = a.stat[2];
+  }
   const float rcp = 1.0f / d;
   if (has_k) {
     float v[M];
@@ -432,6 +443,37 @@ __global__ void __launch_bounds__(256) big_table_kernel(int32_t* tab, const TabR
   const int row = tab_row_get(p.packed, k);
   const int rank = (int)(s_below[row >> 5] + (uint32_t)__popc(s_map[row >> 5] & ((1u << (row & 31)) - 1u)));
   tab[row] = k | (rank << 16);
+}
+// Clear and table in one launch (selections of up to TAB_ROWS rows): every workgroup marks the kept
+// rows in its own LDS bitmap; thread i of the grid clears word i of the statistics and of the
+// per-channel maxima, writes -1 for natural row i when it is dropped, and the entry of the i-th row of
+// the caller's list.  Dropped and kept rows are disjoint, so the two writes never meet.
+__global__ void __launch_bounds__(256) big_prepare_kernel(float* stat, float* colmax, int64_t C, int32_t* tab, int n, const TabRows p) {
+  __shared__ uint32_t s_map[8192 / 32];
+  __shared__ uint32_t s_below[8192 / 32];
+  const int tid = threadIdx.x;
+  s_map[tid] = 0u;
+  __syncthreads();
+  for (int j = tid; j < p.count; j += 256) {
+    const int row = tab_row_get(p.packed, j);
+    atomicOr(&s_map[row >> 5], 1u << (row & 31));
+  }
+  __syncthreads();
+  {
+    uint32_t acc = 0;
+    for (int w = 0; w < tid; ++w) acc += (uint32_t)__popc(s_map[w]);
+    s_below[tid] = acc;
+  }
+  __syncthreads();
+  const int64_t i = (int64_t)blockIdx.x * 256 + tid;
+  if (i < (int64_t)(STAT_BYTES / 4)) stat[i] = 0.f;
+  if (i < C) colmax[i] = 0.f;
+  if (i < n && !((s_map[i >> 5] >> (i & 31)) & 1u)) tab[i] = -1;
+  if (i < p.count) {
+    const int row = tab_row_get(p.packed, (int)i);
+    const int rank = (int)(s_below[row >> 5] + (uint32_t)__popc(s_map[row >> 5] & ((1u << (row & 31)) - 1u)));
+    tab[row] = (int)i | (rank << 16);
+  }
 }
 // selections of more than TAB_ROWS rows: the host ranks, the rows travel with their visit numbers
 constexpr int TAB_PIECE = 512;
@@ -695,9 +737,26 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
   // statistics and table cleared, then the table written piece by piece (rows in natural order, so
   // the visit number of a piece's entry i is its position in the sorted list)
   const int64_t nclr = std::max<int64_t>(std::max<int64_t>(C, n), (int64_t)(STAT_BYTES / 4));
-  hipLaunchKernelGGL(big_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat, a.colmax, C,
-                     (int32_t*)(ws + b.off_tab), n);
-  if (int rc = build_row_table((int32_t*)(ws + b.off_tab), n, rows, r, nullptr, st, who)) return rc;
+  if (r <= TAB_ROWS) {
+    // the row list is checked here, the table written by the clear launch itself
+    std::unique_ptr<uint8_t[]> seen(new uint8_t[(size_t)n]());
+    TabRows tr;
+    memset(&tr, 0, sizeof(tr));
+    tr.count = r;
+    for (int k = 0; k < r; ++k) {
+      if (rows[k] < 0 || rows[k] >= n) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d outside [0, %d)", who, k, rows[k], n);
+      if (seen[(size_t)rows[k]]) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d listed twice", who, k, rows[k]);
+      seen[(size_t)rows[k]] = 1;
+      tab_row_put(tr.packed, k, rows[k]);
+    }
+    hipLaunchKernelGGL(big_prepare_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat, a.colmax, C,
+                       (int32_t*)(ws + b.off_tab), n, tr);
+    if (int rc = check_launch("big_prepare_kernel")) return rc;
+  } else {
+    hipLaunchKernelGGL(big_clear_kernel, dim3((unsigned)((nclr + 255) / 256)), dim3(256), 0, st, a.stat, a.colmax, C,
+                       (int32_t*)(ws + b.off_tab), n);
+    if (int rc = build_row_table((int32_t*)(ws + b.off_tab), n, rows, r, nullptr, st, who)) return rc;
+  }
   const dim3 g1((unsigned)gx, (unsigned)(R / 64));
   a.row_absmax = row16_absmax_out;
   if (row16_absmax_out && (C % 16 || scale_mode == HOT_SCALE_SAWB))
@@ -720,7 +779,15 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
   if (int rc = check_launch("big_stage1_kernel")) return rc;
   const dim3 g2((unsigned)gx, (unsigned)(NB * a.nk));
   if (int rc = dispatch_stage2(m, a, g2, 0, st)) return rc;
-  hipLaunchKernelGGL(big_finalize_kernel, dim3(1), dim3(256), 0, st, a, (int64_t)gx * NB * a.nk, kout);
+  // rows listed run-major (sorted by (row % 64, row / 64)): the quantise pass stores K-major itself
+  bool run_major = !rowmajor && NB * ((a.nk + KG - 1) / KG) <= 65535;
+  for (int k = 1; k < r && run_major; ++k) {
+    const int prev = (rows[k - 1] & 63) * m + (rows[k - 1] >> 6), cur = (rows[k] & 63) * m + (rows[k] >> 6);
+    run_major = cur > prev;
+  }
+  // (with absmax steps the run-major quantise pass reads the statistic itself and publishes the steps)
+  if (!(run_major && scale_mode != HOT_SCALE_SAWB))
+    hipLaunchKernelGGL(big_finalize_kernel, dim3(1), dim3(256), 0, st, a, (int64_t)gx * NB * a.nk, kout);
   if (after_stats) (void)hipEventRecord(after_stats, st);
   if (rowmajor) {
     // untransposed [NB r, C]: the quantise pass writes the destination itself (INT8), or its [Kout, C]
@@ -733,12 +800,6 @@ int hla_big_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const i
       return check_launch("pack4_rows_kernel");
     }
     return HOT_OK;
-  }
-  // rows listed run-major (sorted by (row % 64, row / 64)): the quantise pass stores K-major itself
-  bool run_major = NB * ((a.nk + KG - 1) / KG) <= 65535;
-  for (int k = 1; k < r && run_major; ++k) {
-    const int prev = (rows[k - 1] & 63) * m + (rows[k - 1] >> 6), cur = (rows[k] & 63) * m + (rows[k] >> 6);
-    run_major = cur > prev;
   }
   if (run_major) {
     memset(a.keep, 0, sizeof(a.keep));
