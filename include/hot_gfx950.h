@@ -30,6 +30,14 @@
  *   hot_linear_backward  backward_cuda (HLQ_backward_kernel.cu:457-737) with
  *                        the numerics of FLinearQ.backward, scheme gih_gwlr
  *                        (utils/quant_matmul.py:215-348)
+ *   hot_*_batched        the same two on [B, T, C] tensors with the quantisers
+ *                        vmapped over the batch (utils/quant_matmul.py:33-37,
+ *                        102-106,118-122)
+ *   hot_gx_lowrank       the g_x side of the schemes low_rank / gilr_gwh
+ *                        (utils/quant_matmul.py:229-234,263-266,334-338)
+ *   hot_gx_luq, hot_gw_luq   luq_quantizer on the g_y operand of either product
+ *                        (utils/quant_matmul.py:58-83,250-253,307-314)
+ *   hot_gemm_bf16        F.linear of the forward pass (utils/quant_matmul.py:173-176)
  */
 #ifndef HOT_GFX950_H
 #define HOT_GFX950_H
