@@ -100,7 +100,8 @@ def profiled_traffic(workload="vit_b_fc1"):
 GEMM_VARIANT_NAMES = {1: "gemm_i8_pipe_kernel<128x128, 3 stages>", 2: "gemm_i8_pipe_kernel<128x128, 4 stages>",
                       3: "gemm_i8_pipe_kernel<256x256, 4 stages>", 4: "gemm_i8_kernel<128x128, register-staged>",
                       5: "gemm_i8_pipe_kernel<128x128, split K>", 6: "gemm_i8_slot_kernel<256x256>",
-                      7: "gemm_i8_slot_kernel<128x128>", 8: "gemm_i8_slot_kernel<160x256>"}
+                      7: "gemm_i8_slot_kernel<128x128>", 8: "gemm_i8_slot_kernel<160x256>",
+                      9: "gemm_i8_slot_kernel<96x128>", 10: "gemm_i8_slot_kernel<64x128>", 11: "gemm_i8_slot_kernel<32x128>"}
 
 
 def gemm_kernel_name(M, N, K, bits, with_ws=False):

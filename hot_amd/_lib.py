@@ -22,7 +22,7 @@ SCALE_TENSOR, SCALE_ROW, SCALE_SAWB = 0, 1, 2
 STREAM_GX, STREAM_GW, STREAM_W, STREAM_ACT = 0, 1, 2, 3
 # enum hot_gemm_variant
 (GEMM_AUTO, GEMM_DMA_128_S3, GEMM_DMA_128_S4, GEMM_DMA_256_S4, GEMM_REG_128, GEMM_DMA_128_SPLITK, GEMM_SLOT_256,
- GEMM_SLOT_128, GEMM_SLOT_160X256) = range(9)
+ GEMM_SLOT_128, GEMM_SLOT_160X256, GEMM_SLOT_96X128, GEMM_SLOT_64X128, GEMM_SLOT_32X128) = range(12)
 HOT_STATIC_MAX_CHANNELS = 16384
 
 EXPORTS = (

@@ -675,6 +675,7 @@ gemm_i8_slot_kernel(const GemmArgs g) {
   constexpr int NR = WM + WN;                       // fragment reads per round
   constexpr int H = NM / 2;                         // slots per half round
   constexpr int DPS = (LPW + NM - 1) / NM;          // DMA instructions per slot of the refilling round
+  constexpr int RPSL = (NR + NM - 1) / NM;          // fragment reads per slot (1 unless NR > NM)
   static_assert(NR <= H || BITS != 4, "the reads of a round fit the first half of the round before");
   __shared__ __attribute__((aligned(1024))) uint8_t ring[RING_BYTES];
 
@@ -840,10 +841,15 @@ gemm_i8_slot_kernel(const GemmArgs g) {
           for (int i = m * DPS; i < (m + 1) * DPS && i < LPW; ++i)
             if (refill) dma_one(CUR, kt + S, i);
         }
-        if constexpr (m < NR) {
-          if constexpr (!LAST) read_frag(cur, r + 1, m);
-          else if (more) read_frag(nxt, 0, m);
-        }
+        // fragment reads of the next round: one per slot from the first slot on, or, when a wave owns
+        // fewer MFMAs than fragments (tiles of one fragment row or column per wave), RPSL per slot
+        static_for<RPSL>([&](auto tc) {
+          constexpr int t = m * RPSL + decltype(tc)::value;
+          if constexpr (t < NR) {
+            if constexpr (!LAST) read_frag(cur, r + 1, t);
+            else if (more) read_frag(nxt, 0, t);
+          }
+        });
         if constexpr (BITS == 4) {
           if constexpr (m < H) expand_hi(p, m * EPS_, (m + 1) * EPS_);
           else if (!LAST || more) expand_lo(p ^ 1, (m - H) * EPS_, (m - H + 1) * EPS_);
@@ -1281,6 +1287,17 @@ int gemm_plan_impl(int64_t M, int64_t N, int64_t K, int bits, int64_t lda, int64
   const int64_t big = ((M + 255) / 256) * ((N + 255) / 256);
   const int64_t mid = ((M + 159) / 160) * ((N + 255) / 256);
   const double k = (double)kpad;   // codes along K
+  if (bits == 8 && rows128 && kpad >= 1024 && tiles <= 256) {
+    // an INT8 product that leaves CUs idle at 128 x 128: the shortest tile (32, 64 or 96 rows of A against
+    // 128 of B) that still gives every tile a CU of its own.  Measured at K = 7092 against 128 x 128
+    // (and the split-K pair): 3072 x 768 25.5 against 29.3 us, 2304 x 768 20.3 / 27.2, 768 x 768 15.4 / 25.2
+    // (21.2), 768 x 3072 24.1 / 28.3; a second round of tiles costs more than the longer tile.
+    const int64_t tn = (N + 127) / 128;
+    if (((M + 31) / 32) * tn <= 256) return HOT_GEMM_SLOT_32X128;
+    if (((M + 63) / 64) * tn <= 256) return HOT_GEMM_SLOT_64X128;
+    if (((M + 95) / 96) * tn <= 256) return HOT_GEMM_SLOT_96X128;
+    return HOT_GEMM_SLOT_128;
+  }
   const GemmSplit sp = gemm_split_plan(M, N, K, bits);
   if (sp.splits > 1 && ws_bytes >= sp.ws_bytes && !(rows128 && tiles >= 96)) return HOT_GEMM_DMA_128_SPLITK;
   if (tiles <= 256) return (rows128 && kpad >= 1024) ? HOT_GEMM_SLOT_128 : HOT_GEMM_DMA_128_S4;
@@ -1310,6 +1327,15 @@ static int launch_variant(int variant, GemmArgs& g, hipStream_t st) {
     case HOT_GEMM_SLOT_256: return launch_gemm_slot<4, 4, 2, 2, BITS, 2, 128, OutT>(g, st);
     case HOT_GEMM_SLOT_128: return launch_gemm_slot<2, 2, 2, 2, BITS, 4, 128, OutT>(g, st);
     case HOT_GEMM_SLOT_160X256: return launch_gemm_slot<5, 2, 1, 4, BITS, 2, 128, OutT>(g, st);
+    case HOT_GEMM_SLOT_96X128:
+      if constexpr (BITS == 8) return launch_gemm_slot<3, 1, 1, 4, 8, 4, 128, OutT>(g, st);
+      else return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: the 96 x 128 kernel takes INT8 codes");
+    case HOT_GEMM_SLOT_64X128:
+      if constexpr (BITS == 8) return launch_gemm_slot<2, 1, 1, 4, 8, 4, 128, OutT>(g, st);
+      else return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: the 64 x 128 kernel takes INT8 codes");
+    case HOT_GEMM_SLOT_32X128:
+      if constexpr (BITS == 8) return launch_gemm_slot<1, 1, 1, 4, 8, 4, 128, OutT>(g, st);
+      else return fail(HOT_ERR_UNSUPPORTED, "hot_gemm_i8: the 32 x 128 kernel takes INT8 codes");
     default: return fail(HOT_ERR_INVALID, "hot_gemm_i8: unknown kernel variant %d", variant);
   }
 }

@@ -370,7 +370,10 @@ enum hot_gemm_variant {
   HOT_GEMM_SLOT_256 = 6,       /* 256 x 256 tiles, two stages                                   */
   HOT_GEMM_SLOT_128 = 7,       /* 128 x 128 tiles, four stages, one workgroup per CU            */
   HOT_GEMM_SLOT_160X256 = 8,   /* 160 x 256 tiles (four waves side by side), two stages         */
-  HOT_GEMM_VARIANTS = 9
+  HOT_GEMM_SLOT_96X128 = 9,    /* 96 x 128 tiles (four waves side by side), four stages, INT8   */
+  HOT_GEMM_SLOT_64X128 = 10,   /* 64 x 128 tiles (four waves side by side), four stages, INT8   */
+  HOT_GEMM_SLOT_32X128 = 11,   /* 32 x 128 tiles (four waves side by side), four stages, INT8   */
+  HOT_GEMM_VARIANTS = 12
 };
 /* The variant hot_gemm_i8 (workspace_bytes = 0) or a GEMM inside hot_linear_backward
  * (workspace_bytes = what the call can spare) runs for this product; lda, ldb in bytes. */

@@ -370,6 +370,10 @@ VARIANT_CASES = [
     ("GEMM_SLOT_128", 4, 1, 1, 200), ("GEMM_SLOT_128", 8, 384, 256, 7092),
     ("GEMM_SLOT_160X256", 8, 700, 530, 600), ("GEMM_SLOT_160X256", 4, 700, 530, 1000), ("GEMM_SLOT_160X256", 4, 161, 257, 2304),
     ("GEMM_SLOT_160X256", 8, 159, 255, 128), ("GEMM_SLOT_160X256", 4, 1600, 768, 3072),
+    # one fragment column per wave: more fragment reads than MFMAs per round (several reads per slot); INT8 only
+    ("GEMM_SLOT_96X128", 8, 700, 530, 600), ("GEMM_SLOT_96X128", 8, 97, 129, 128), ("GEMM_SLOT_96X128", 8, 384, 256, 7092),
+    ("GEMM_SLOT_96X128", 8, 960, 768, 1000),
+    ("GEMM_SLOT_64X128", 8, 700, 530, 600), ("GEMM_SLOT_64X128", 8, 65, 127, 256), ("GEMM_SLOT_64X128", 8, 384, 256, 7092),
 ]
 
 
@@ -404,7 +408,9 @@ def test_gemm_every_variant_exact(gpu, name, bits, M, N, K):
     (4, 4000, 4090, 8320, "GEMM_DMA_256_S4"),      # rows of 4160 bytes: not whole 128-byte lines
     (4, 5000, 6600, 192, "GEMM_DMA_128_S3"),       # short K: many small tiles, three workgroups per CU
     (8, 5000, 6600, 192, "GEMM_DMA_128_S4"),
-    (8, 384, 256, 4000, "GEMM_SLOT_128"),          # few tiles, no workspace: one deep-ring workgroup per tile
+    (8, 384, 256, 4000, "GEMM_SLOT_32X128"),       # few tiles: the shortest tile, 24 workgroups instead of 6
+    (8, 3000, 800, 4000, "GEMM_SLOT_96X128"),      # 168 tiles of 128 x 128, 224 of 96 x 128, 329 of 64 x 128
+    (8, 4096, 1024, 1024, "GEMM_SLOT_128"),        # 256 tiles: nothing shorter keeps one round
     (4, 384, 256, 4200, "GEMM_DMA_128_S4"),        # the same with rows of 2112 bytes
     (4, 12608, 768, 3072, "GEMM_SLOT_160X256"),    # ViT-B fc1 g_x: one balanced round of 237 tiles
 ])
@@ -501,12 +507,13 @@ def test_gemm_splits_rule():
     """hot_gemm_splits: products with few output tiles and a long K are cut, others are not."""
     from hot_amd import _lib
     f = _lib.lib().hot_gemm_splits
-    assert f(3072, 768, 7092, 8) == 1          # ViT-B fc1 g_W: 144 tiles, one deep-ring workgroup each
-    assert f(768, 768, 7092, 8) == 7           # ViT-B proj g_W: 36 tiles, 112 stages in 7 ranges of 16
+    assert f(3072, 768, 7092, 8) == 1          # ViT-B fc1 g_W: 192 tiles of 96 x 128, one deep-ring workgroup each
+    assert f(768, 768, 7092, 8) == 1           # ViT-B proj g_W: 144 tiles of 32 x 128 instead of 36 tiles in 7 K ranges
+    assert f(768, 768, 7092, 4) == 3           # the INT4 form of that product: 36 tiles, K cut into 3 ranges
     assert f(12608, 768, 3072, 4) == 1         # ViT-B fc1 g_x: 594 tiles
     assert f(11008, 4096, 4096, 8) == 1
     assert f(256, 256, 128, 8) == 1            # short K
-    assert f(256, 256, 2304, 8) == 2
+    assert f(256, 256, 2304, 8) == 1           # INT8, 4 tiles of 128 x 128: 16 tiles of 32 x 128, unsplit
     assert _lib.lib().hot_gemm_workspace_bytes(256, 256, 2304, 8) == 4 * 2 * 128 * 128 * 4
 
 

@@ -241,10 +241,14 @@ def test_library_argument_checks_need_no_gpu():
     # the variant query and the named-variant entry point validate before they touch anything
     assert lib.hot_gemm_plan(12608, 768, 3072, 4, 1536, 1536, 0) == _lib.GEMM_SLOT_160X256
     assert lib.hot_gemm_plan(12608, 768, 2304, 4, 1152, 1152, 0) == _lib.GEMM_DMA_128_S3
-    assert lib.hot_gemm_plan(3072, 768, 7092, 8, 7168, 7168, 0) == _lib.GEMM_SLOT_128
-    assert lib.hot_gemm_plan(3072, 768, 7092, 8, 7168, 7168, 1 << 30) == _lib.GEMM_SLOT_128     # 144 tiles: unsplit
-    assert lib.hot_gemm_plan(768, 768, 7092, 8, 7168, 7168, 1 << 30) == _lib.GEMM_DMA_128_SPLITK # 36 tiles
-    assert lib.hot_gemm_plan(768, 768, 7092, 8, 7168, 7168, 0) == _lib.GEMM_SLOT_128
+    # INT8 products with room to spare at 128 x 128 take the shortest tile that keeps one round (ViT-B g_W products)
+    assert lib.hot_gemm_plan(3072, 768, 7092, 8, 7168, 7168, 0) == _lib.GEMM_SLOT_96X128        # fc1: 192 tiles
+    assert lib.hot_gemm_plan(3072, 768, 7092, 8, 7168, 7168, 1 << 30) == _lib.GEMM_SLOT_96X128  # a workspace changes nothing
+    assert lib.hot_gemm_plan(2304, 768, 7092, 8, 7168, 7168, 0) == _lib.GEMM_SLOT_64X128        # qkv: 216 tiles
+    assert lib.hot_gemm_plan(768, 768, 7092, 8, 7168, 7168, 1 << 30) == _lib.GEMM_SLOT_32X128   # proj: 144 tiles, no split
+    assert lib.hot_gemm_plan(768, 3072, 7092, 8, 7168, 7168, 0) == _lib.GEMM_SLOT_96X128        # fc2: 192 tiles
+    assert lib.hot_gemm_plan(4096, 1024, 7092, 8, 7168, 7168, 0) == _lib.GEMM_SLOT_128          # 256 tiles: nothing shorter fits
+    assert lib.hot_gemm_plan(768, 768, 7092, 4, 3584, 3584, 1 << 30) == _lib.GEMM_DMA_128_SPLITK # INT4: 36 tiles, split K
     assert lib.hot_gemm_plan(8192, 4096, 11008, 4, 5504, 5504, 0) == _lib.GEMM_SLOT_256
     assert lib.hot_gemm_plan(8192, 4096, 11136, 4, 5568, 5568, 0) == _lib.GEMM_DMA_256_S4     # rows of 43.5 lines
     assert lib.hot_gemm_plan(1 << 20, 128, 8192, 8, 8192, 8192, 0) == _lib.GEMM_REG_128     # A is 8 GiB
