@@ -483,7 +483,7 @@ int hot_linear_backward_bias(const void* gy, const void* w, int dtype, const voi
 
 struct LowrankLayout {
   int64_t lp, ld_g, ld_w;
-  size_t off_colg, off_colw, off_sg, off_sw, off_qg, off_qw, off_t, off_exp, colg_bytes, exp_bytes, total;
+  size_t off_colg, off_colw, off_sg, off_sw, off_qg, off_qw, off_t, off_exp, off_proj, colg_bytes, exp_bytes, total;
 };
 
 static LowrankLayout lowrank_layout(int64_t L, int64_t O, int64_t I, const hot_config* c) {
@@ -498,12 +498,15 @@ static LowrankLayout lowrank_layout(int64_t L, int64_t O, int64_t I, const hot_c
   b.exp_bytes = c->hla_n > 128 ? hla_expand_big_workspace_bytes_impl(L / c->hla_n, I, c->hla_n) : 0;
   b.off_colg = o; o += align256(b.colg_bytes);
   b.off_colw = o; o += align256(colwise_workspace_bytes_impl(I));
-  b.off_sg = o;   o += 256;
+  // a step per coefficient row (gx_scale ROW): lp steps, and the unquantised projection [L', O] in fp32
+  const bool per_row = c->gx_scale == HOT_SCALE_ROW;
+  b.off_sg = o;   o += per_row ? align256((size_t)b.lp * 4) : 256;
   b.off_sw = o;   o += 256;
   b.off_qg = o;   o += align256((size_t)b.lp * b.ld_g);
   b.off_qw = o;   o += align256((size_t)I * b.ld_w);
   b.off_t = o;    o += align256((size_t)b.lp * (size_t)I * 4);
   b.off_exp = o;  o += align256(b.exp_bytes);
+  b.off_proj = o; o += per_row ? align256((size_t)b.lp * (size_t)O * 4) : 0;
   b.total = o;
   return b;
 }
@@ -513,7 +516,8 @@ static int check_lowrank(const hot_config* cfg, int64_t L, int64_t O, int64_t I,
   if (L <= 0 || O <= 0 || I <= 0 || O % 8 || I % 8) return fail(HOT_ERR_INVALID, "%s: L=%lld, O=%lld and I=%lld must be positive, O and I multiples of 8", who, (long long)L, (long long)O, (long long)I);
   if (L % cfg->hla_n) return fail(HOT_ERR_INVALID, "%s: L=%lld is not a multiple of hla_n=%d", who, (long long)L, cfg->hla_n);
   if (cfg->gx_bits != cfg->w_bits) return fail(HOT_ERR_UNSUPPORTED, "%s: gx_bits (%d) and w_bits (%d) must match", who, cfg->gx_bits, cfg->w_bits);
-  if (cfg->gx_scale != HOT_SCALE_TENSOR) return fail(HOT_ERR_UNSUPPORTED, "%s: the projected g_y takes one step for the tensor (a step per coefficient row or per channel has no place in the product's epilogue)", who);
+  if (cfg->gx_scale == HOT_SCALE_SAWB) return fail(HOT_ERR_UNSUPPORTED, "%s: the projected g_y takes absmax steps (one for the tensor or one per coefficient row)", who);
+  if (cfg->gx_scale == HOT_SCALE_ROW && cfg->hla_n > 128) return fail(HOT_ERR_UNSUPPORTED, "%s: a step per coefficient row takes token blocks up to 128", who);
   if (cfg->w_scale == HOT_SCALE_ROW) return fail(HOT_ERR_UNSUPPORTED, "%s: W uses one step per tensor", who);
   return HOT_OK;
 }
@@ -538,9 +542,21 @@ int hot_gx_lowrank(const void* gy, const void* w, int dtype, int64_t L, int64_t 
   float* sw = (float*)(ws + b.off_sw);
   const int bits = cfg->gx_bits;
   // q(P g_y), untransposed [L', O]; the K padding of every row is cleared apart
-  int rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, bits, cfg->gx_round, cfg->seed,
-                              HOT_STREAM_GX, HOT_SCALE_TENSOR, ws + b.off_qg, b.ld_g, bits == 4, sg, ws + b.off_colg,
-                              b.colg_bytes, st, who, nullptr, false, nullptr, nullptr, 1, 0, true);
+  int rc;
+  const bool per_row = cfg->gx_scale == HOT_SCALE_ROW;
+  if (per_row) {
+    // a step per coefficient row (norm_quantizer on [L', O], utils/quant_matmul.py:19-37,244-255): the
+    // projection unquantised in fp32, then the row-wise quantiser without a transform (elements numbered
+    // row-major for stochastic rounding)
+    float* proj = (float*)(ws + b.off_proj);
+    rc = hla_project_impl(gy, dtype, L, O, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, proj, O, st, true);
+    if (!rc) rc = hq_rowwise_impl(proj, HOT_F32, b.lp, O, 1, bits, cfg->gx_round, cfg->seed, HOT_STREAM_GX, HOT_SCALE_ROW,
+                                  ws + b.off_qg, b.ld_g, sg, nullptr, 0, st);
+  } else {
+    rc = colwise_quant_impl(gy, dtype, L, O, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, bits, cfg->gx_round, cfg->seed,
+                            HOT_STREAM_GX, HOT_SCALE_TENSOR, ws + b.off_qg, b.ld_g, bits == 4, sg, ws + b.off_colg,
+                            b.colg_bytes, st, who, nullptr, false, nullptr, nullptr, 1, 0, true);
+  }
   if (rc) return rc;
   zero_pad_impl(ws + b.off_qg, b.lp, O * bits / 8, b.ld_g, st);
   // q(W), stored [I, O]: blocks of one row, nothing transformed
@@ -549,7 +565,7 @@ int hot_gx_lowrank(const void* gy, const void* w, int dtype, int64_t L, int64_t 
                           colwise_workspace_bytes_impl(I), st, who);
   if (rc) return rc;
   float* t = (float*)(ws + b.off_t);
-  rc = gemm_i8_impl(ws + b.off_qg, b.ld_g, ws + b.off_qw, b.ld_w, bits, b.lp, I, O, sg, 0, sw, 1.0f, t, HOT_F32, I, nullptr, st);
+  rc = gemm_i8_impl(ws + b.off_qg, b.ld_g, ws + b.off_qw, b.ld_w, bits, b.lp, I, O, sg, per_row ? 1 : 0, sw, 1.0f, t, HOT_F32, I, nullptr, st);
   if (rc) return rc;
   if (cfg->hla_n > 128)
     return hla_expand_big_impl(t, L / cfg->hla_n, I, cfg->hla_n, cfg_rows(cfg), cfg->hla_r, 1.0f / (float)cfg->hla_n, gx,

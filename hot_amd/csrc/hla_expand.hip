@@ -94,9 +94,9 @@ int hla_expand_impl(const float* t, int64_t nb, int64_t C, int n, const int32_t*
 // fp32 output.  Kept for completeness, not tuned.
 struct ProjectArgs {
   const void* in;      // [nb n, C]
-  float* out;          // [C, ld]
+  float* out;          // [C, ld] (transposed) or [nb r, ld] (row-major)
   int64_t nb, C, ld;
-  int32_t n, r;
+  int32_t n, r, rowmajor;
   int8_t row[EXP_MAX_N];
 };
 
@@ -122,6 +122,11 @@ __global__ void __launch_bounds__(EXP_THREADS) hla_project_kernel(const ProjectA
         col[i * nt + tid] = x + y;
         col[(i + h) * nt + tid] = x - y;
       }
+  if (a.rowmajor) {
+    float* dst = a.out + blk * a.r * a.ld + c;
+    for (int k = 0; k < a.r; ++k) dst[(int64_t)k * a.ld] = col[a.row[k] * nt + tid];
+    return;
+  }
   float* dst = a.out + c * a.ld + blk * a.r;
   for (int k = 0; k < a.r; ++k) dst[k] = col[a.row[k] * nt + tid];
   if (blk == a.nb - 1)
@@ -129,7 +134,7 @@ __global__ void __launch_bounds__(EXP_THREADS) hla_project_kernel(const ProjectA
 }
 
 int hla_project_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r, float* out,
-                     int64_t ld, hipStream_t st) {
+                     int64_t ld, hipStream_t st, bool rowmajor) {
   const char* who = "hla_project";
   if (!in || !out || !rows) return fail(HOT_ERR_INVALID, "%s: null pointer", who);
   if (n < 1 || n > EXP_MAX_N || (n & (n - 1))) return fail(HOT_ERR_UNSUPPORTED, "%s: block %d (a power of two up to %d)", who, n, EXP_MAX_N);
@@ -137,9 +142,9 @@ int hla_project_impl(const void* in, int dtype, int64_t R, int64_t C, int n, con
   if (r < 1 || r > n) return fail(HOT_ERR_INVALID, "%s: r=%d outside [1, %d]", who, r, n);
   const int64_t nb = R / n;
   if (nb > 65535) return fail(HOT_ERR_UNSUPPORTED, "%s: more than 65535 token blocks", who);
-  if (ld < nb * r) return fail(HOT_ERR_INVALID, "%s: ld=%lld < %lld coefficients", who, (long long)ld, (long long)(nb * r));
+  if (ld < (rowmajor ? C : nb * r)) return fail(HOT_ERR_INVALID, "%s: ld=%lld too short", who, (long long)ld);
   ProjectArgs a;
-  a.in = in; a.out = out; a.nb = nb; a.C = C; a.ld = ld; a.n = n; a.r = r;
+  a.in = in; a.out = out; a.nb = nb; a.C = C; a.ld = ld; a.n = n; a.r = r; a.rowmajor = rowmajor ? 1 : 0;
   bool seen[EXP_MAX_N] = {};
   for (int k = 0; k < r; ++k) {
     if (rows[k] < 0 || rows[k] >= n || seen[rows[k]]) return fail(HOT_ERR_INVALID, "%s: rows[%d]=%d out of range or listed twice", who, k, rows[k]);

@@ -46,9 +46,10 @@ int hq_luq_impl(const void* in, int dtype, int64_t M, int64_t K, int n, int bits
 // RNG streams of the logarithmic quantiser: its operand of the g_x product, of the g_W product
 constexpr uint32_t HOT_STREAM_LUQ = 4, HOT_STREAM_LUQ_GW = 5;
 // Unquantised token-wise projection, transposed: out[c][blk r + k] = (P in)[blk r + k][c] in fp32, ld
-// floats per channel (the tail [NB r, ld) cleared); blocks up to 128 tokens.
+// floats per channel (the tail [NB r, ld) cleared); or row-major: out[blk r + k][c], ld floats per
+// coefficient row.  Blocks up to 128 tokens.
 int hla_project_impl(const void* in, int dtype, int64_t R, int64_t C, int n, const int32_t* rows, int r, float* out,
-                     int64_t ld, hipStream_t st);
+                     int64_t ld, hipStream_t st, bool rowmajor = false);
 // out = ((float(16 acc_a + acc_b) * s_a[0]) * s_b[0]) * post on [M, N] int32 sums
 int luq_combine_impl(const int32_t* acc_a, const int32_t* acc_b, int64_t M, int64_t N, const float* s_a, const float* s_b,
                      float post, void* out, int out_dtype, hipStream_t st);

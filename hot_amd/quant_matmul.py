@@ -309,9 +309,6 @@ class FLinearQ(Function):
             # gradients of the samples added in fp32 in sample order
             if luq and args.transform_scheme in LOWRANK_GX_SCHEMES:
                 raise NotImplementedError("quantBWDGogi luq runs with the schemes gih_gwlr and hadamard")
-            if not luq and opt.gx_scale != ops.SCALE_TENSOR:
-                raise NotImplementedError("transform scheme %r: the projected g_y takes one step for the tensor "
-                                          "(quantBWDGogi int or stoch)" % args.transform_scheme)
             per_sample = go.dim() == 3 and args.batched_mode == "per_sample"
             samples = [go[b] for b in range(go.shape[0])] if per_sample else [go.reshape(-1, go.shape[-1])]
             gxs, gw = [], None

@@ -296,11 +296,15 @@ HOT_API int hot_linear_backward_batched(const void* gy, const void* w, int dtype
  * (utils/quant_matmul.py, transform_scheme "low_rank" and "gilr_gwh": :229-233 g_y <- P g_y,
  * :263-266 W untransformed, :288-290 the product and its two steps, :334-337 P^T (.) / n):
  *   g_x [L, I] = P^T ( q(P g_y) [L', O] . q(W) [O, I] ) s_g s_w / hla_n.
- * cfg->hla_n / hla_rows describe P (blocks up to 64 tokens), gx_bits / gx_round the quantiser of
- * P g_y (one step for the tensor), w_bits (= gx_bits) / w_round / w_scale that of W.  The g_W side
- * of those schemes is the g_W side of hot_linear_backward with the matching token-wise selection
- * (hot_hla_tokenwise + hot_gemm_i8).  Four kernels on `hip_stream`, kept for completeness of the
- * reference's scheme list.
+ * cfg->hla_n / hla_rows (hla_rows_big above 64) describe P: blocks up to 128 tokens in one pass,
+ * 256 .. 8192 through the two-level path in both directions (fp32 intermediates in the workspace).
+ * gx_bits / gx_round / gx_scale are the quantiser of P g_y: HOT_SCALE_TENSOR (one step; elements of
+ * stochastic rounding numbered as hot_hla_tokenwise numbers them) or HOT_SCALE_ROW (one step per
+ * coefficient row of [L', O], as norm_quantizer gives them; blocks up to 128 tokens; elements
+ * numbered row-major).  w_bits (= gx_bits) / w_round / w_scale are the quantiser of W.  The g_W
+ * side of those schemes is the g_W side of hot_linear_backward with the matching token-wise
+ * selection (hot_hla_tokenwise + hot_gemm_i8).  Four to eight kernels on `hip_stream`, kept for
+ * completeness of the reference's scheme list.
  */
 HOT_API size_t hot_gx_lowrank_workspace_bytes(int64_t L, int64_t O, int64_t I, const hot_config* cfg);
 HOT_API int hot_gx_lowrank(const void* gy, const void* w, int dtype, int64_t L, int64_t O, int64_t I,

@@ -521,12 +521,17 @@ def gx_lowrank(g_y: np.ndarray, w: np.ndarray, cfg: HotConfig) -> BackwardTrace:
     rows = np.asarray(cfg.hla_rows)
     tr = BackwardTrace()
     Gp = fwht_blocks_first(g_y, cfg.hla_n, rows)                                        # [L', O]
-    tr.qG, tr.sG = quant(Gp, cfg.gx_bits, SCALE_TENSOR, cfg.gx_round, cfg.seed, STREAM_GX,
-                         index=colwise_rng_index(O, L // cfg.hla_n, rows).T)
+    if cfg.gx_scale == SCALE_ROW:
+        # a step per coefficient row (norm_quantizer on [L', O], :19-37): elements numbered row-major
+        tr.qG, tr.sG = quant(Gp, cfg.gx_bits, SCALE_ROW, cfg.gx_round, cfg.seed, STREAM_GX)
+    else:
+        tr.qG, tr.sG = quant(Gp, cfg.gx_bits, SCALE_TENSOR, cfg.gx_round, cfg.seed, STREAM_GX,
+                             index=colwise_rng_index(O, L // cfg.hla_n, rows).T)
     tr.qW, tr.sW = quant(w, cfg.w_bits, cfg.w_scale, cfg.w_round, cfg.seed, STREAM_W,
                          index=colwise_rng_index(w.shape[1], w.shape[0], np.arange(1)).T)
     tr.acc_x = int_gemm_nt(tr.qG, tr.qW.T)                                              # [L', I]
-    t = ((tr.acc_x.astype(F32) * tr.sG[0]).astype(F32) * tr.sW[0]).astype(F32)
+    sg = tr.sG[:, None] if cfg.gx_scale == SCALE_ROW else tr.sG[0]
+    t = ((tr.acc_x.astype(F32) * sg).astype(F32) * tr.sW[0]).astype(F32)
     tr.g_x = (hla_expand(t, cfg.hla_n, rows) / F32(cfg.hla_n)).astype(F32)
     return tr
 

@@ -34,10 +34,10 @@ def make_case(L, O, I, seed=0, dtype=torch.float32, outliers=True):
     return x.to(dtype), w.to(dtype), gy.to(dtype)
 
 
-def both_configs(L, rule="python", **kw):
+def both_configs(L, rule="python", max_block=64, **kw):
     from hot_amd import ops
     ocfg = orc.HotConfig.python_rule(L, **kw) if rule == "python" else orc.HotConfig.paper(16, 8, **kw)
-    if ocfg.hla_n > 64:
+    if ocfg.hla_n > max_block:
         n, rows = orc.hla_rows(64)
         ocfg.hla_n, ocfg.hla_rows = n, tuple(int(v) for v in rows)
     opt = ops.HotOptions(n_o=ocfg.n_o, hla_n=ocfg.hla_n, hla_rows=ocfg.hla_rows, gx_bits=ocfg.gx_bits,
@@ -815,13 +815,18 @@ def test_hq_linear_scheme_hadamard(gpu, fresh_args, L):
     (768, 64, 40, "python", dict()),                                              # n = 256, r = 136: the two-level path, packed INT4
     (2048, 48, 264, "python", dict(gx_bits=8, w_bits=8)),                         # n = 2048, two channel strips of the expansion
     (3072, 32, 24, "python", dict(gx_round=orc.ROUND_STOCH, seed=9)),             # n = 1024, three blocks, stochastic
+    # a step per coefficient row of P g_y (norm_quantizer, the canonical recipe's g_y quantiser)
+    (448, 192, 160, "python", dict(gx_scale=orc.SCALE_ROW, gx_round=orc.ROUND_STOCH, seed=6)),
+    (384, 96, 72, "python", dict(gx_scale=orc.SCALE_ROW, gx_bits=8, w_bits=8)),    # n = 128
+    (512, 256, 128, "paper", dict(gx_scale=orc.SCALE_ROW, gx_round=orc.ROUND_STOCH, w_scale=orc.SCALE_SAWB, seed=2)),
 ])
 def test_gx_lowrank_matches_oracle(gpu, dtype, L, O, I, rule, variant):
     """g_x of the schemes "low_rank" / "gilr_gwh" (hot_gx_lowrank): the projected g_y stored untransposed,
     W quantised without a transform, the product in fp32 and the expansion pass, bit for bit the oracle."""
     from hot_amd import ops
     x, w, gy = make_case(L, O, I, seed=L + I, dtype=dtype)
-    ocfg, opt = both_configs(L, rule=rule, **variant)
+    ocfg, opt = both_configs(L, rule=rule, max_block=8192, **variant)
+    assert ocfg.hla_n == (16 if rule == "paper" else orc.hla_rows(L)[0])
     gx = ops.gx_lowrank(gy.to(gpu), w.to(gpu), opt)
     tr = orc.gx_lowrank(gy.float().numpy(), w.float().numpy(), ocfg)
     assert gx.dtype == dtype and tuple(gx.shape) == (L, I)
@@ -831,9 +836,13 @@ def test_gx_lowrank_matches_oracle(gpu, dtype, L, O, I, rule, variant):
 def test_gx_lowrank_refuses_what_it_cannot_do(gpu):
     from hot_amd import ops
     x, w, gy = make_case(256, 64, 32, seed=0)
-    _, opt = both_configs(256, gx_scale=orc.SCALE_ROW)
-    with pytest.raises(ops.HotError, match="one step for the tensor"):
+    _, opt = both_configs(256, gx_scale=orc.SCALE_SAWB)
+    with pytest.raises(ops.HotError, match="absmax steps"):
         ops.gx_lowrank(gy.to(gpu), w.to(gpu), opt)
+    n, rows = orc.hla_rows(256)
+    big = ops.HotOptions(hla_n=n, hla_rows=tuple(int(v) for v in rows), gx_scale=orc.SCALE_ROW)
+    with pytest.raises(ops.HotError, match="token blocks up to 128"):
+        ops.gx_lowrank(gy.to(gpu), w.to(gpu), big)
     n, rows = orc.hla_rows(128)
     odd = ops.HotOptions(hla_n=n, hla_rows=tuple(int(v) for v in rows))
     with pytest.raises(ops.HotError, match="not a multiple of hla_n"):
@@ -874,6 +883,30 @@ def test_hq_linear_lowrank_gx_schemes(gpu, fresh_args, scheme, L):
     gi_ref, gw_ref = fq.backward(gy.cpu(), lin.weight.detach().cpu(), xq, sx, h_out, h_bs, fq.PortConfig(), scheme=scheme)
     assert rel(x.grad.cpu().numpy(), gi_ref.numpy()) < REL_TOL
     assert rel(lin.weight.grad.cpu().numpy(), gw_ref.numpy()) < REL_TOL
+
+
+def test_hq_linear_lowrank_with_per_token_quantisers(gpu, fresh_args):
+    """transform_scheme "low_rank" under the quantisers of the reference's canonical recipe for g_y
+    (quantBWDGogi = quantBWDGogw = "nq": a step per row of the quantised matrix, stochastic rounding,
+    utils/quant_matmul.py:19-37,244-255,307-318): the projected g_y [L', O] takes a step per coefficient row
+    on the g_x side, (P g_y)^T a step per channel on the g_W side.  Bit-exact against the oracle."""
+    from hot_amd.quant_matmul import HQ_Linear
+    L, I, O = 448, 96, 128
+    fresh_args.transform_scheme = "low_rank"
+    fresh_args.quantBWDGogi = fresh_args.quantBWDGogw = "nq"
+    torch.manual_seed(12)
+    lin = HQ_Linear(I, O, bias=False).to(gpu)
+    x = torch.randn(L, I, device=gpu, requires_grad=True)
+    gy = torch.randn(L, O, device=gpu) * 1e-3
+    step = fresh_args.sr_step
+    lin(x).backward(gy)
+    xn, gyn, wn = x.detach().cpu().numpy(), gy.cpu().numpy(), lin.weight.detach().cpu().numpy()
+    seed = (int(fresh_args.sr_seed) << 20) + step
+    ocfg, _ = both_configs(L, seed=seed, gx_round=orc.ROUND_STOCH, gx_scale=orc.SCALE_ROW, gw_round=orc.ROUND_STOCH,
+                           gw_scale=orc.SCALE_ROW)
+    xq_ref, sx_ref = orc.abc_forward(xn, ocfg)
+    assert np.array_equal(x.grad.cpu().numpy(), orc.gx_lowrank(gyn, wn, ocfg).g_x)
+    assert np.array_equal(lin.weight.grad.cpu().numpy(), orc.linear_backward(gyn, wn, xq_ref, sx_ref, ocfg).g_w)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
